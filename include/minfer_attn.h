@@ -1,0 +1,104 @@
+/*
+ * C ABI of the MI355X (gfx950) fused-attention library, libminfer_attn.so.
+ *
+ * Every entry point takes plain device pointers, sizes, element strides and a HIP stream
+ * (as void*), launches asynchronously on that stream and never synchronises or allocates.
+ * Scratch memory is a caller-provided workspace whose size the *_workspace_bytes
+ * functions report.  Return value: 0 on success, a negative MINFER_ATTN_E* code on a
+ * rejected call (nothing was launched); minfer_attn_last_error() then describes it.
+ *
+ * The operator-level contract these functions implement is the reference's
+ *   flash_attn(int qtype_int, int qblock_size, int qtype_size,
+ *              Tensor q, Tensor k, Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()
+ * (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:30), whose host function is
+ * flash_attn_cuda (reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/op.cuh:21-106).
+ */
+#ifndef MINFER_ATTN_H
+#define MINFER_ATTN_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Element types, numbered as the reference numbers its activations' GGML types
+ * (reference: src/minfer/const.py:4-35: F16 = 1, BF16 = 30). */
+#define MINFER_ATTN_F16 1
+#define MINFER_ATTN_BF16 30
+
+#define MINFER_ATTN_OK 0
+#define MINFER_ATTN_EINVAL (-1)    /* shape, stride, dtype or alignment rejected        */
+#define MINFER_ATTN_EWORKSPACE (-2) /* workspace missing or smaller than required       */
+#define MINFER_ATTN_ELAUNCH (-3)   /* the HIP runtime refused the launch                */
+
+/* Element strides of dims 0..2 of q, of k (v must share them) and of out; dim 3 (head_dim)
+ * always has stride 1.  Replaces the reference's QKVStrides, which carries no out strides
+ * (reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/kernels/kernel.cuh:12-15,
+ * filled at op.cuh:80-83). */
+typedef struct minfer_attn_strides {
+    int64_t q0, q1, q2;
+    int64_t kv0, kv1, kv2;
+    int64_t o0, o1, o2;
+} minfer_attn_strides;
+
+/* Library/ABI version (major * 1000 + minor). */
+int minfer_attn_version(void);
+
+/* Message for the most recent non-zero return on the calling thread ("" if none). */
+const char* minfer_attn_last_error(void);
+
+/* Bytes of workspace minfer_flash_attn needs for batch B and sequence length L (holds the
+ * per-tile mask classification). */
+size_t minfer_flash_attn_workspace_bytes(int64_t B, int64_t L);
+
+/*
+ * Dense-mask GQA attention (prefill):
+ *   out[b,h,i,:] = sum_j softmax_j(q[b,h,i,:].k[b,h/n_rep,j,:]/sqrt(D) | mask[b,0,i,j]) v[b,h/n_rep,j,:]
+ * q,out [B,Hq,L,D]; k,v [B,Hkv,L,D]; mask contiguous bool bytes [B,1,L,L], non-zero = attend;
+ * n_rep = Hq/Hkv.  A query row with no attended key yields zeros.
+ * Replaces flash_attn_cuda + flash_attn_cuda_impl (reference: flash_attn/op.cuh:21-106,
+ * flash_attn/kernels/kernel.cuh:16-27).  Beyond the reference's checks (op.cuh:32-96):
+ * dtype may be MINFER_ATTN_F16 or MINFER_ATTN_BF16, D may be 64 or 128, all data pointers must
+ * be 16-byte aligned and all strides multiples of 8 elements.
+ */
+int minfer_flash_attn(int dtype, const void* q, const void* k, const void* v,
+                      const uint8_t* mask, void* out,
+                      int64_t B, int64_t Hq, int64_t Hkv, int64_t L, int64_t D,
+                      const minfer_attn_strides* strides,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+/* Bytes of workspace minfer_flash_attn_decode needs (split-KV partial results). */
+size_t minfer_flash_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Lmax, int64_t D);
+
+/*
+ * Single-token decode over a KV cache: q,out [B,Hq,1,D]; k_cache,v_cache [B,Hkv,Lmax,D]
+ * (the reference's cache layout, src/minfer/core.py:105-127); ctx_lens int32 [B] on the device;
+ * query b attends cache rows 0..ctx_lens[b]-1 (rows beyond are never read into the result;
+ * ctx_lens[b] == 0 yields zeros).  The KV range is split across workgroups and merged by a
+ * log-sum-exp combine kernel.  No counterpart in the reference (its op requires Lq == Lk,
+ * flash_attn/op.cuh:74-78); strides->q2 and strides->o2 are ignored.
+ */
+int minfer_flash_attn_decode(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                             const int32_t* ctx_lens, void* out,
+                             int64_t B, int64_t Hq, int64_t Hkv, int64_t Lmax, int64_t D,
+                             const minfer_attn_strides* strides,
+                             void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Packed ragged causal prefill: q,out [1,Hq,T,D]; k,v [1,Hkv,T,D]; cu_seqlens int32 [n_seqs+1]
+ * on the device with cu_seqlens[0] == 0 and cu_seqlens[n_seqs] == T; token rows
+ * cu_seqlens[s]..cu_seqlens[s+1]-1 form sequence s and attend causally inside it only.
+ * Equals minfer_flash_attn with B = 1, L = T under the block-diagonal causal mask.  Needs no
+ * workspace.  No counterpart in the reference; strides->q0, kv0, o0 are ignored.
+ */
+int minfer_flash_attn_varlen(int dtype, const void* q, const void* k, const void* v,
+                             const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_seqlen,
+                             void* out, int64_t Hq, int64_t Hkv, int64_t T, int64_t D,
+                             const minfer_attn_strides* strides, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MINFER_ATTN_H */

@@ -1,0 +1,120 @@
+// Shared device helpers for the gfx950 attention kernels: element-type traits over the CDNA4
+// MFMA builtins, wave64 cross-lane helpers, direct global->LDS copies and LDS swizzles.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace minfer_attn {
+
+typedef short s16x4 __attribute__((ext_vector_type(4)));
+typedef short s16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 h16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 h16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 h16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 b16x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 b16x4 __attribute__((ext_vector_type(4)));
+typedef __bf16 b16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+#define MA_DEV __device__ __forceinline__
+
+// 16-bit element types.  Operand fragments travel as raw 16-bit lanes (s16x8 / s16x4) and are
+// bit-cast at the MFMA call, so one kernel body serves both.
+struct F16 {
+    // D[32x32] += A[32x16] * B[16x32]; lane l holds A row l%32, k = 8*(l/32)+0..7 (B alike, by
+    // column); D register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, column l%32.
+    static MA_DEV f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h16x8, a),
+                                                      __builtin_bit_cast(h16x8, b), c, 0, 0, 0);
+    }
+    // D[16x16] += A[16x32] * B[32x16]; lane l holds A row l%16, k = 8*(l/16)+0..7; D register r
+    // of lane l is row 4*(l/16) + r, column l%16.
+    static MA_DEV f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(h16x8, a),
+                                                      __builtin_bit_cast(h16x8, b), c, 0, 0, 0);
+    }
+    // D[16x16] += A[16x16] * B[16x16]; lane l holds A row l%16, k = 4*(l/16)+0..3.
+    static MA_DEV f32x4 mfma16k16(s16x4 a, s16x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(h16x4, a),
+                                                     __builtin_bit_cast(h16x4, b), c, 0, 0, 0);
+    }
+    static MA_DEV uint32_t pack2(float lo, float hi) {  // round-to-nearest-even pair
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
+    }
+    static MA_DEV float to_float(short bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+};
+
+struct BF16 {
+    static MA_DEV f32x16 mfma32(s16x8 a, s16x8 b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(b16x8, a),
+                                                       __builtin_bit_cast(b16x8, b), c, 0, 0, 0);
+    }
+    static MA_DEV f32x4 mfma16(s16x8 a, s16x8 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(b16x8, a),
+                                                       __builtin_bit_cast(b16x8, b), c, 0, 0, 0);
+    }
+    static MA_DEV f32x4 mfma16k16(s16x4 a, s16x4 b, f32x4 c) {
+        return __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, b, c, 0, 0, 0);
+    }
+    static MA_DEV uint32_t pack2(float lo, float hi) {
+        f32x2 f = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, b16x2));
+    }
+    static MA_DEV float to_float(short bits) {
+        return __builtin_bit_cast(float, (uint32_t)(uint16_t)bits << 16);
+    }
+};
+
+typedef __attribute__((address_space(3))) void lds_void;
+typedef __attribute__((address_space(1))) const void glb_cvoid;
+
+// Copies 16 bytes per lane from global memory straight into LDS without passing through VGPRs.
+// `lds_base` must be wave-uniform: lane i's 16 bytes land at lds_base + 16*i, whatever address
+// the lane read from.  Completion is tracked by vmcnt, and it is the caller who waits
+// (s_waitcnt vmcnt + barrier) before anyone reads the destination: the copy is issued from
+// inline assembly so that the compiler does not serialise every later LDS read behind it.
+MA_DEV void copy16_global_to_lds(const void* src, void* lds_base) {
+    const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_base);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                 :
+                 : "s"(dst), "v"(src)
+                 : "memory");
+}
+
+// Waits until at most N of this wave's vector-memory operations (global loads and global->LDS
+// copies, which retire in order) are outstanding.  Also a compiler barrier, so LDS reads of the
+// copied data cannot be hoisted above the wait.
+template <int N> MA_DEV void wait_vmcnt() {
+    static_assert(N >= 0 && N < 64, "vmcnt is a 6-bit counter");
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(N) : "memory");
+}
+
+// LDS transpose read: within each group of 16 lanes, lanes 4e..4e+3 together address row e of a
+// 4x16 tile of 16-bit elements (4 contiguous elements per lane); lane i receives column i, i.e.
+// {row0[i], row1[i], row2[i], row3[i]}.
+MA_DEV s16x4 lds_read_tr16(const void* lds_ptr) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)lds_ptr);
+}
+
+// Value of x held by lane (l ^ 32), combined with the lane's own by max / sum.
+MA_DEV float max_across_halves(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+}
+MA_DEV float sum_across_halves(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
+MA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+MA_DEV int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
+
+}  // namespace minfer_attn

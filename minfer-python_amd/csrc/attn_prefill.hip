@@ -1,0 +1,527 @@
+// Prefill attention for gfx950: single-pass online-softmax kernel over 64-key tiles.
+//
+// Work decomposition.  One workgroup = 8 waves (two per SIMD, so one wave's softmax overlaps the
+// other's MFMAs) = one KV head x (HPW query heads of that KV head's GQA group) x (QBW consecutive
+// 32-row query blocks), HPW*QBW = 8, so the K/V tiles a workgroup stages in LDS are shared by
+// every query head of the group.  Each wave owns 32 query rows of one head and keeps its Q
+// fragments, the 64x32 score tile and the Dx32 output accumulator in registers.
+//
+// Per 64-key tile a wave computes S^T = K Q^T (K from LDS as the MFMA A operand, Q as B), so
+// that a lane holds 16 keys of ONE query row per 32x32 block: row max / row sum need a single
+// exchange with lane^32.  The exponentiated scores are, without any data movement, the B operand
+// of O^T += V^T P^T; V^T fragments come from LDS transpose reads.  K and V tiles are copied
+// global->LDS directly (no VGPR staging) and double-buffered: the copy of tile t+1 is issued
+// right after the barrier that opens tile t.
+//
+// Masking.  The reference operator takes an arbitrary dense bool mask [B,1,L,L]
+// (reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/op.cuh:28).  A pre-pass
+// classifies every 64x64 mask tile as none / all / mixed; the main kernel skips "none" tiles,
+// runs "all" tiles unmasked and reads mask bytes only for "mixed" tiles, which keeps arbitrary
+// masks bit-exact while a causal mask costs one byte-read tile per row of tiles.
+#include "attn_common.h"
+#include "attn_host.h"
+
+namespace minfer_attn {
+
+enum : uint32_t { TILE_NONE = 0, TILE_ALL = 1, TILE_MIXED = 2 };
+constexpr int kMaxKeyTiles = 2048;  // active-tile list capacity (L <= 131072)
+
+// ------------------------------------------------------------------------------------------
+// Mask classification: cls[b][qt][kt] for 64x64 tiles.  grid (ceil(NKT/16), NQT, B), 256 threads.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void classify_mask_kernel(const uint8_t* __restrict__ mask,
+                                                            uint8_t* __restrict__ cls, int L, int NQT,
+                                                            int NKT, int vec) {
+    __shared__ uint32_t any_s[16], all_s[16];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int strip = blockIdx.x, qt = blockIdx.y, b = blockIdx.z;
+    if (tid < 16) { any_s[tid] = 0u; all_s[tid] = 0x01010101u; }
+    __syncthreads();
+    const uint8_t* mb = mask + (size_t)b * L * L;
+    const int col0 = strip * 1024 + lane * 16;  // this lane's 16 key columns
+    uint32_t any_acc = 0u, all_acc = 0x01010101u;
+    if (vec) {
+        if (col0 < L) {
+            for (int r = w; r < 64; r += 4) {
+                const int row = qt * 64 + r;
+                if (row >= L) break;
+                const uint4 x = *reinterpret_cast<const uint4*>(mb + (size_t)row * L + col0);
+                any_acc |= x.x | x.y | x.z | x.w;
+                all_acc &= x.x & x.y & x.z & x.w;
+            }
+        }
+    } else {
+        for (int r = w; r < 64; r += 4) {
+            const int row = qt * 64 + r;
+            if (row >= L) break;
+            for (int e = 0; e < 16; ++e) {
+                const int col = col0 + e;
+                if (col < L) {
+                    const uint32_t x = mb[(size_t)row * L + col] ? 1u : 0u;
+                    any_acc |= x;
+                    all_acc &= x * 0x01010101u;
+                }
+            }
+        }
+    }
+    // lanes 4t..4t+3 of each wave cover key tile (strip*16 + t)
+    any_acc |= __shfl_xor(any_acc, 1); any_acc |= __shfl_xor(any_acc, 2);
+    all_acc &= __shfl_xor(all_acc, 1); all_acc &= __shfl_xor(all_acc, 2);
+    if ((lane & 3) == 0) {
+        atomicOr(&any_s[lane >> 2], any_acc);
+        atomicAnd(&all_s[lane >> 2], all_acc);
+    }
+    __syncthreads();
+    if (tid < 16) {
+        const int kt = strip * 16 + tid;
+        if (kt < NKT) {
+            const uint32_t c = any_s[tid] == 0u ? TILE_NONE : (all_s[tid] == 0x01010101u ? TILE_ALL : TILE_MIXED);
+            cls[((size_t)b * NQT + qt) * NKT + kt] = (uint8_t)c;
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Main kernel
+// ------------------------------------------------------------------------------------------
+struct PrefillParams {
+    const void* q; const void* k; const void* v; void* out;
+    const uint8_t* mask;   // dense mode: [B,1,L,L]
+    const uint8_t* cls;    // dense mode: [B,NQT,NKT]
+    const int32_t* cu;     // varlen mode: [n_seqs+1]
+    int64_t q0, q1, q2, kv0, kv1, kv2, o0, o1, o2;
+    int L;                 // dense: sequence length; varlen: total packed tokens
+    int B, Hq, Hkv, n_rep;
+    int hpw_log2;          // query heads per workgroup = 1 << hpw_log2 (<= 8)
+    int n_hg;              // head groups per KV head = n_rep >> hpw_log2
+    int NQT, NKT;          // dense: 64-row query / key tile counts of the mask classification
+    int NQ;                // workgroup-level query tiles (dense: exact; varlen: upper bound)
+    int n_seqs;
+    int mask_vec;          // dense: mask rows may be read as aligned 32-bit words
+    float scale_log2;      // softmax scale * log2(e)
+};
+
+enum { MODE_DENSE = 0, MODE_VARLEN = 1 };
+constexpr int kWaves = 8;            // waves per workgroup (two per SIMD)
+constexpr int kThreads = kWaves * 64;
+
+template <int D> struct TileGeom {
+    static constexpr int RB = D * 2;          // bytes per K/V row
+    static constexpr int G = RB / 16;         // 16-byte granules per row
+    static constexpr int RPI = 1024 / RB;     // rows one wave-wide copy instruction covers
+    static constexpr int NLD = 64 / (kWaves * RPI);  // copy instructions per wave, per tile, per tensor
+    static constexpr int RPW = 256 / RB;      // rows per 256-byte bank window
+    static constexpr int TILE_BYTES = 64 * RB;
+    // XOR swizzles applied to the granule index of a row.  K is read 16 rows x one granule at a
+    // time (ds_read_b128), V 4 rows x 64 bytes at a time (transpose reads); both become
+    // conflict-free.
+    static MA_DEV int swz_k(int row) { return (row / RPW) & (G - 1); }
+    static MA_DEV int swz_v(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+};
+
+template <class T, int D, int MODE>
+__global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p) {
+    using GEO = TileGeom<D>;
+    constexpr int RB = GEO::RB, G = GEO::G, RPI = GEO::RPI, NLD = GEO::NLD;
+    constexpr int KC = D / 16;   // 16-wide contraction chunks of Q K^T
+    constexpr int DB = D / 32;   // 32-row blocks of O^T
+
+    __shared__ __attribute__((aligned(1024))) char k_lds[2][GEO::TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char v_lds[2][GEO::TILE_BYTES];
+    __shared__ uint32_t tile_list[MODE == MODE_DENSE ? kMaxKeyTiles : 1];
+    __shared__ int n_active_s;
+
+    const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
+    const int h = lane >> 5, l32 = lane & 31;
+    const int HPW = 1 << p.hpw_log2, QBW = kWaves >> p.hpw_log2;  // heads, 32-row query blocks per workgroup
+
+    // ---- which (batch, KV head, head group, query tile) is this workgroup -------------------
+    const int BG = p.B * p.Hkv;
+    const int NG = BG * p.n_hg;
+    int pidx, rank;
+    {
+        const int n = blockIdx.x;
+        if ((NG & 7) == 0) {  // keep all workgroups of one (batch, KV head) on one XCD (ids go round-robin)
+            const int per = NG >> 3, mm = n >> 3;
+            pidx = (mm % per) * 8 + (n & 7);
+            rank = mm / per;
+        } else {
+            pidx = n % NG;
+            rank = n / NG;
+        }
+    }
+    const int bg = pidx % BG, hg = pidx / BG;
+    const int g = bg % p.Hkv, b = bg / p.Hkv;
+
+    int seq_lo = 0, seq_len = p.L;  // token rows of the attended sequence
+    int qtile;                      // workgroup-level query tile (32*QBW rows) inside the sequence
+    if (MODE == MODE_DENSE) {
+        qtile = p.NQ - 1 - rank;    // longest rows of a causal mask first
+    } else {
+        int x = rank, s = 0, nt = 0;
+        for (; s < p.n_seqs; ++s) {
+            seq_lo = p.cu[s];
+            seq_len = p.cu[s + 1] - seq_lo;
+            nt = (seq_len + 32 * QBW - 1) / (32 * QBW);
+            if (x < nt) break;
+            x -= nt;
+        }
+        if (s >= p.n_seqs) return;
+        qtile = nt - 1 - x;
+    }
+
+    const int head = g * p.n_rep + hg * HPW + (w & (HPW - 1));
+    const int qblk = qtile * QBW + (w >> p.hpw_log2);           // 32-row block index inside the sequence
+    const int q_row0 = qblk * 32;                                // first query row (sequence-local)
+    const bool wave_on = q_row0 < seq_len;
+    const int last_row = seq_len - 1;
+    const int qrow = q_row0 + l32;                               // this lane's query row
+
+    const short* Qh = (const short*)p.q + (MODE == MODE_DENSE ? (int64_t)b * p.q0 : 0) + (int64_t)head * p.q1 + (int64_t)seq_lo * p.q2;
+    const short* Kh = (const short*)p.k + (MODE == MODE_DENSE ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
+    const short* Vh = (const short*)p.v + (MODE == MODE_DENSE ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
+    short* Oh = (short*)p.out + (MODE == MODE_DENSE ? (int64_t)b * p.o0 : 0) + (int64_t)head * p.o1 + (int64_t)seq_lo * p.o2;
+    const uint8_t* mrow = MODE == MODE_DENSE ? p.mask + ((size_t)b * p.L + min(qrow, last_row)) * p.L : nullptr;
+
+    // ---- list of key tiles this workgroup visits ---------------------------------------------
+    // entry = key tile | (2-bit class for each 64-row query tile the workgroup overlaps) << 16
+    const int qt64_first = (qtile * QBW * 32) >> 6;
+    const int n_qt64 = QBW >= 2 ? QBW / 2 : 1;
+    const int my_qt64_slot = (q_row0 >> 6) - qt64_first;
+    int n_active;
+    if (MODE == MODE_DENSE) {
+        if (w == 0) {
+            int cnt = 0;
+            for (int base = 0; base < p.NKT; base += 64) {
+                const int kt = base + lane;
+                uint32_t c = 0;
+                if (kt < p.NKT) {
+                    for (int s = 0; s < n_qt64; ++s) {
+                        const int qs = qt64_first + s;
+                        if (qs < p.NQT) c |= (uint32_t)p.cls[((size_t)b * p.NQT + qs) * p.NKT + kt] << (2 * s);
+                    }
+                }
+                const uint64_t bal = __ballot(c != 0);
+                const int pos = cnt + __popcll(bal & ((1ull << lane) - 1ull));
+                if (c) tile_list[pos] = (uint32_t)kt | (c << 16);
+                cnt += __popcll(bal);
+            }
+            if (lane == 0) n_active_s = cnt;
+        }
+        __syncthreads();
+        n_active = n_active_s;
+    } else {
+        const int top_row = min(qtile * QBW * 32 + QBW * 32, seq_len) - 1;  // causal: keys 0..top_row
+        n_active = (top_row >> 6) + 1;
+    }
+
+    // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
+    s16x8 qf[KC];
+    {
+        const short* src = Qh + (int64_t)min(qrow, last_row) * p.q2 + 8 * h;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) qf[c] = *reinterpret_cast<const s16x8*>(src + 16 * c);
+    }
+
+    // ---- global -> LDS tile copy ----------------------------------------------------------
+    auto issue_tile = [&](int kt, int stage) {
+        const int key0 = kt * 64;
+#pragma unroll
+        for (int j = 0; j < NLD; ++j) {
+            const int row0 = (j * kWaves + w) * RPI;     // wave-uniform first row of this instruction
+            const int row = row0 + lane / G;
+            const int pg = lane % G;                      // physical granule this lane fills
+            const int64_t grow = (int64_t)min(key0 + row, last_row) * p.kv2;
+            copy16_global_to_lds(Kh + grow + 8 * (pg ^ GEO::swz_k(row)), &k_lds[stage][row0 * RB]);
+            copy16_global_to_lds(Vh + grow + 8 * (pg ^ GEO::swz_v(row)), &v_lds[stage][row0 * RB]);
+        }
+    };
+
+    f32x16 o_acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.f;
+    float m_ref = -INFINITY;   // reference maximum (raw score units) of the lane's query row
+    float l_sum = 0.f;         // this lane's share of the softmax denominator
+    const float c2 = p.scale_log2;
+    constexpr float kLazyLog2 = 6.f;  // re-reference only when the row maximum grows by > 2^6
+
+    auto tile_of = [&](int it, int& kt, uint32_t& cls_w) {
+        if (MODE == MODE_DENSE) {
+            const uint32_t e = tile_list[it];
+            kt = (int)(e & 0xffffu);
+            cls_w = (e >> (16 + 2 * my_qt64_slot)) & 3u;
+        } else {
+            kt = it;
+            cls_w = (64 * kt + 63 <= q_row0) ? TILE_ALL : ((64 * kt > q_row0 + 31) ? TILE_NONE : TILE_MIXED);
+        }
+    };
+    // mask words of a MIXED dense tile: word [kb][j] covers keys key0 + 32kb + 8j + 4h + 0..3
+    uint32_t mw[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
+    auto fetch_mask = [&](int kt) {
+        const int key0 = kt * 64;
+        if (p.mask_vec && key0 + 64 <= seq_len) {
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    mw[kb][j] = *reinterpret_cast<const uint32_t*>(mrow + key0 + 32 * kb + 8 * j + 4 * h);
+        } else {  // unaligned rows or a tile crossing the end: bytes, clamped (the range test comes later)
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int kbase = key0 + 32 * kb + 8 * j + 4 * h;
+                    uint32_t x = 0;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) x |= (uint32_t)mrow[min(kbase + e, last_row)] << (8 * e);
+                    mw[kb][j] = x;
+                }
+        }
+    };
+
+    if (n_active > 0) {
+        int kt0; uint32_t c0;
+        tile_of(0, kt0, c0);
+        issue_tile(kt0, 0);
+        if (MODE == MODE_DENSE && wave_on && c0 == TILE_MIXED) fetch_mask(kt0);
+    }
+
+    for (int it = 0; it < n_active; ++it) {
+        const int stage = it & 1;
+        int kt; uint32_t cls_w;
+        tile_of(it, kt, cls_w);
+        wait_vmcnt<0>();                     // this wave's share of tile `it` (and its mask words) has landed
+        __syncthreads();                     // everyone's share has; stage^1 is no longer being read
+        uint32_t mcur[2][4];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) mcur[kb][j] = mw[kb][j];
+        if (it + 1 < n_active) {
+            int ktn; uint32_t cn;
+            tile_of(it + 1, ktn, cn);
+            issue_tile(ktn, stage ^ 1);
+            if (MODE == MODE_DENSE && wave_on && cn == TILE_MIXED) fetch_mask(ktn);
+        }
+        if (!wave_on || cls_w == TILE_NONE) continue;
+
+        const int key0 = kt * 64;
+        // ---- S^T = K Q^T ------------------------------------------------------------------
+        f32x16 s_acc[2];
+#pragma unroll
+        for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.f;
+        {
+            const char* rowp0 = &k_lds[stage][l32 * RB];
+            const char* rowp1 = rowp0 + 32 * RB;
+            const int sw0 = GEO::swz_k(l32), sw1 = GEO::swz_k(32 + l32);
+#pragma unroll
+            for (int c = 0; c < KC; ++c) {
+                const s16x8 a0 = *reinterpret_cast<const s16x8*>(rowp0 + 16 * ((2 * c + h) ^ sw0));
+                const s16x8 a1 = *reinterpret_cast<const s16x8*>(rowp1 + 16 * ((2 * c + h) ^ sw1));
+                s_acc[0] = T::mfma32(a0, qf[c], s_acc[0]);
+                s_acc[1] = T::mfma32(a1, qf[c], s_acc[1]);
+            }
+        }
+
+        // ---- masking ----------------------------------------------------------------------
+        // register r of block kb is key key0 + 32kb + 8(r/4) + 4h + r%4
+        if (cls_w == TILE_MIXED || key0 + 64 > seq_len) {
+            const bool use_bytes = MODE == MODE_DENSE && cls_w == TILE_MIXED;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const int kbase = key0 + 32 * kb + 8 * j + 4 * h;
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        bool keep = kbase + e < seq_len;
+                        if (MODE == MODE_DENSE) keep = keep && (!use_bytes || ((mcur[kb][j] >> (8 * e)) & 0xffu) != 0u);
+                        else keep = keep && (kbase + e <= qrow);
+                        s_acc[kb][4 * j + e] = keep ? s_acc[kb][4 * j + e] : -INFINITY;
+                    }
+                }
+            }
+        }
+
+        // ---- online softmax ----------------------------------------------------------------
+        uint32_t pf[4][4];  // P^T fragments (B operand): [16-key chunk][4 x packed pair]
+        {
+            float mx = s_acc[0][0];
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[kb][r]);
+            mx = max_across_halves(mx);
+            const bool grow = (mx - m_ref) * c2 > kLazyLog2 || (m_ref == -INFINITY && mx > -INFINITY);
+            if (__any(grow)) {  // wave-uniform: most tiles leave every row's reference unchanged
+                const float m_new = grow ? mx : m_ref;
+                const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2((m_ref - m_new) * c2);
+                m_ref = m_new;
+                l_sum *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; ++db)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+            }
+            const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * c2;
+            float ls = 0.f;
+#pragma unroll
+            for (int kb = 0; kb < 2; ++kb) {
+#pragma unroll
+                for (int r = 0; r < 16; r += 2) {
+                    const float p0 = fast_exp2(fmaf(s_acc[kb][r], c2, -mc));
+                    const float p1 = fast_exp2(fmaf(s_acc[kb][r + 1], c2, -mc));
+                    ls += p0 + p1;
+                    pf[2 * kb + (r >> 3)][(r & 7) >> 1] = T::pack2(p0, p1);
+                }
+            }
+            l_sum += ls;
+        }
+
+        // ---- O^T += V^T P^T ----------------------------------------------------------------
+        // chunk c contracts keys 16c..16c+15 in the order 16c + 8(i/4) + 4h + i%4 (i = element of the
+        // lane's 8-wide k slice), which is the order the score registers already have.
+        const int blk = lane >> 4, li = lane & 15;
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            uint4 pu; pu.x = pf[c][0]; pu.y = pf[c][1]; pu.z = pf[c][2]; pu.w = pf[c][3];
+            const s16x8 bfrag = __builtin_bit_cast(s16x8, pu);
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                s16x8 a;
+#pragma unroll
+                for (int half = 0; half < 2; ++half) {
+                    const int row = 16 * c + 8 * half + 4 * h + (li >> 2);
+                    const int dcol = 32 * db + 16 * (blk & 1) + 4 * (li & 3);
+                    const char* ptr = &v_lds[stage][row * RB + 16 * ((dcol >> 3) ^ GEO::swz_v(row)) + 2 * (dcol & 7)];
+                    const s16x4 t = lds_read_tr16(ptr);
+                    a[4 * half + 0] = t[0]; a[4 * half + 1] = t[1]; a[4 * half + 2] = t[2]; a[4 * half + 3] = t[3];
+                }
+                o_acc[db] = T::mfma32(a, bfrag, o_acc[db]);
+            }
+        }
+    }
+
+    // ---- epilogue: normalise and store -----------------------------------------------------
+    if (!wave_on) return;
+    const float l = sum_across_halves(l_sum);
+    const float inv = l > 0.f ? 1.f / l : 0.f;
+    if (qrow < seq_len) {
+        short* orow = Oh + (int64_t)qrow * p.o2;
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                uint2 pk;
+                pk.x = T::pack2(o_acc[db][4 * j + 0] * inv, o_acc[db][4 * j + 1] * inv);
+                pk.y = T::pack2(o_acc[db][4 * j + 2] * inv, o_acc[db][4 * j + 3] * inv);
+                *reinterpret_cast<uint2*>(orow + 32 * db + 8 * j + 4 * h) = pk;
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// Host side
+// ------------------------------------------------------------------------------------------
+static size_t cls_bytes(int64_t B, int64_t L) {
+    const int64_t nt = (L + 63) / 64;
+    return (size_t)(B * nt * nt + 255) / 256 * 256;
+}
+
+template <class T, int D, int MODE>
+static int launch_prefill(const PrefillParams& p, int grid, hipStream_t stream) {
+    hipLaunchKernelGGL((prefill_kernel<T, D, MODE>), dim3(grid), dim3(kThreads), 0, stream, p);
+    return check_launch("prefill_kernel");
+}
+
+template <int MODE>
+static int dispatch_prefill(int dtype, int64_t D, const PrefillParams& p, int grid, hipStream_t stream) {
+    if (dtype == MINFER_ATTN_F16) {
+        return D == 128 ? launch_prefill<F16, 128, MODE>(p, grid, stream) : launch_prefill<F16, 64, MODE>(p, grid, stream);
+    }
+    return D == 128 ? launch_prefill<BF16, 128, MODE>(p, grid, stream) : launch_prefill<BF16, 64, MODE>(p, grid, stream);
+}
+
+static void fill_common(PrefillParams& p, const void* q, const void* k, const void* v, void* out,
+                        int64_t Hq, int64_t Hkv, int64_t D, const minfer_attn_strides* st) {
+    p.q = q; p.k = k; p.v = v; p.out = out;
+    p.q0 = st->q0; p.q1 = st->q1; p.q2 = st->q2;
+    p.kv0 = st->kv0; p.kv1 = st->kv1; p.kv2 = st->kv2;
+    p.o0 = st->o0; p.o1 = st->o1; p.o2 = st->o2;
+    p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.n_rep = (int)(Hq / Hkv);
+    p.hpw_log2 = (p.n_rep % 8 == 0) ? 3 : (p.n_rep % 4 == 0) ? 2 : ((p.n_rep % 2 == 0) ? 1 : 0);
+    p.n_hg = p.n_rep >> p.hpw_log2;
+    p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+}
+
+}  // namespace minfer_attn
+
+using namespace minfer_attn;
+
+MINFER_ATTN_EXPORT size_t minfer_flash_attn_workspace_bytes(int64_t B, int64_t L) {
+    if (B <= 0 || L <= 0) return 256;
+    return cls_bytes(B, L);
+}
+
+MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k, const void* v,
+                                 const uint8_t* mask, void* out, int64_t B, int64_t Hq, int64_t Hkv,
+                                 int64_t L, int64_t D, const minfer_attn_strides* st, void* workspace,
+                                 size_t workspace_bytes, void* stream_v) {
+    clear_error();
+    if (int rc = check_common(dtype, q, k, v, out, Hq, Hkv, D, st)) return rc;
+    if (!mask) return fail(MINFER_ATTN_EINVAL, "flash_attn: mask is null");
+    if (B < 0 || L < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn: negative B or L");
+    if (B == 0 || L == 0) return MINFER_ATTN_OK;
+    if (L > 64 * (int64_t)kMaxKeyTiles) return fail(MINFER_ATTN_EINVAL, "flash_attn: L > 131072 unsupported");
+    if (B > 65535) return fail(MINFER_ATTN_EINVAL, "flash_attn: B > 65535 unsupported");
+    if (!workspace || workspace_bytes < cls_bytes(B, L))
+        return fail(MINFER_ATTN_EWORKSPACE, "flash_attn: workspace too small (see minfer_flash_attn_workspace_bytes)");
+    hipStream_t stream = (hipStream_t)stream_v;
+
+    PrefillParams p{};
+    fill_common(p, q, k, v, out, Hq, Hkv, D, st);
+    p.mask = mask; p.cls = (const uint8_t*)workspace; p.cu = nullptr;
+    p.L = (int)L; p.B = (int)B;
+    p.NQT = p.NKT = (int)((L + 63) / 64);
+    const int rows_per_wg = 32 * (kWaves >> p.hpw_log2);
+    p.NQ = (int)((L + rows_per_wg - 1) / rows_per_wg);
+    p.n_seqs = 0;
+    p.mask_vec = ((L & 15) == 0 && aligned16(mask)) ? 1 : 0;
+    const int64_t grid = (int64_t)p.NQ * B * Hkv * p.n_hg;
+    if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn: problem too large for one launch");
+
+    hipLaunchKernelGGL(classify_mask_kernel, dim3((p.NKT + 15) / 16, p.NQT, (unsigned)B), dim3(256), 0, stream,
+                       mask, (uint8_t*)workspace, p.L, p.NQT, p.NKT, p.mask_vec);
+    if (int rc = check_launch("classify_mask_kernel")) return rc;
+    return dispatch_prefill<MODE_DENSE>(dtype, D, p, (int)grid, stream);
+}
+
+MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const void* k, const void* v,
+                                        const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_seqlen,
+                                        void* out, int64_t Hq, int64_t Hkv, int64_t T, int64_t D,
+                                        const minfer_attn_strides* st, void* stream_v) {
+    clear_error();
+    if (int rc = check_common(dtype, q, k, v, out, Hq, Hkv, D, st)) return rc;
+    if (!cu_seqlens) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: cu_seqlens is null");
+    if (n_seqs < 0 || T < 0 || max_seqlen < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: negative size");
+    if (n_seqs == 0 || T == 0) return MINFER_ATTN_OK;
+    if (T > 0x7fffffffLL / 2) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: T too large");
+    hipStream_t stream = (hipStream_t)stream_v;
+
+    PrefillParams p{};
+    fill_common(p, q, k, v, out, Hq, Hkv, D, st);
+    p.mask = nullptr; p.cls = nullptr; p.cu = cu_seqlens;
+    p.L = (int)T; p.B = 1;
+    p.NQT = p.NKT = 0;
+    const int rows_per_wg = 32 * (kWaves >> p.hpw_log2);
+    p.NQ = (int)((T + rows_per_wg - 1) / rows_per_wg + n_seqs);  // >= sum over sequences of ceil(len / rows_per_wg)
+    p.n_seqs = (int)n_seqs;
+    const int64_t grid = (int64_t)p.NQ * Hkv * p.n_hg;
+    if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: problem too large for one launch");
+    return dispatch_prefill<MODE_VARLEN>(dtype, D, p, (int)grid, stream);
+}

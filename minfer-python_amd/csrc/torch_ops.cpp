@@ -1,0 +1,198 @@
+// PyTorch (stable ABI) registration of the attention operators in namespace `minfer`.
+//
+// This file is the only place where torch types appear: it validates tensors exactly as the
+// reference host function does, turns them into pointers/strides and calls the C ABI of
+// libminfer_attn.so (include/minfer_attn.h) on the current torch stream.  Loading the shared
+// object as the Python module `_C` runs the static registrations, which is how the reference
+// exposes its ops (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:7-33,
+// src/minfer/kernels/torch_ext/csrc/cuda/reg.cu:16-27).
+//
+// Only the accelerator dispatch key gets an implementation: calling these ops with CPU tensors
+// fails in the dispatcher instead of falling back to anything.
+#include <Python.h>
+
+#include <torch/csrc/inductor/aoti_torch/c/shim.h>
+#include <torch/csrc/stable/accelerator.h>
+#include <torch/csrc/stable/library.h>
+#include <torch/csrc/stable/ops.h>
+#include <torch/csrc/stable/tensor.h>
+#include <torch/headeronly/core/ScalarType.h>
+#include <torch/headeronly/util/Exception.h>
+
+#include "minfer_attn.h"
+
+extern "C" {
+PyObject* PyInit__C(void) {
+    static struct PyModuleDef module_def = {PyModuleDef_HEAD_INIT, "_C", NULL, -1, NULL};
+    return PyModule_Create(&module_def);
+}
+}
+
+namespace minfer {
+
+using torch::headeronly::DeviceType;
+using torch::headeronly::ScalarType;
+using torch::stable::Tensor;
+
+namespace {
+
+void* current_stream() {
+    auto device_index = torch::stable::accelerator::getCurrentDeviceIndex();
+    void* stream = nullptr;
+    TORCH_ERROR_CODE_CHECK(aoti_torch_get_current_cuda_stream(device_index, &stream));
+    return stream;
+}
+
+bool on_gpu(const Tensor& t) { return t.device().type() == DeviceType::CUDA; }
+
+int dtype_code(const Tensor& q, const Tensor& k, const Tensor& v, const Tensor& out, const char* op) {
+    const ScalarType t = q.scalar_type();
+    STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, op, ": q must be float16 or bfloat16");
+    STD_TORCH_CHECK(k.scalar_type() == t && v.scalar_type() == t && out.scalar_type() == t, op,
+                    ": q, k, v and out must share one dtype");
+    return t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16;
+}
+
+Tensor byte_workspace(const Tensor& like, size_t nbytes) {
+    const int64_t n = (int64_t)nbytes;
+    return torch::stable::new_empty(like, {n}, ScalarType::Byte);
+}
+
+void check_rc(int rc, const char* op) {
+    STD_TORCH_CHECK(rc == MINFER_ATTN_OK, op, ": ", minfer_attn_last_error());
+}
+
+minfer_attn_strides strides_of(const Tensor& q, const Tensor& k, const Tensor& out) {
+    return minfer_attn_strides{q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1),
+                               k.stride(2), out.stride(0), out.stride(1), out.stride(2)};
+}
+
+}  // namespace
+
+// Same signature, argument meaning and checks as the reference's flash_attn_cuda
+// (reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/op.cuh:21-106); the dtype check
+// also admits bfloat16 and head_dim may be 64 as well as 128.
+void flash_attn_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size,
+                    const Tensor& q,   // [B, n_heads, L, HEAD_DIM]
+                    const Tensor& k,   // [B, n_kv_heads, L, HEAD_DIM]
+                    const Tensor& v,   // [B, n_kv_heads, L, HEAD_DIM]
+                    Tensor& mask,      // [B, 1, L, L] bool, True = attend
+                    Tensor& out) {     // [B, n_heads, L, HEAD_DIM]
+    (void)qtype_int; (void)qblock_size; (void)qtype_size;  // unused by the reference as well
+    STD_TORCH_CHECK(on_gpu(q) && on_gpu(k) && on_gpu(v) && on_gpu(mask) && on_gpu(out),
+                    "flash_attn: all tensors must be on the GPU");
+    STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && out.dim() == 4 && mask.dim() == 4,
+                    "flash_attn: q, k, v, mask and out must be 4-D");
+    STD_TORCH_CHECK(q.stride(-1) == 1 && k.stride(-1) == 1 && v.stride(-1) == 1 && out.stride(-1) == 1,
+                    "flash_attn: q, k, v and out must be contiguous in head_dim");
+    STD_TORCH_CHECK(k.stride(0) == v.stride(0) && k.stride(1) == v.stride(1) && k.stride(2) == v.stride(2),
+                    "flash_attn: k and v must share strides");
+    STD_TORCH_CHECK(mask.is_contiguous(), "flash_attn: mask must be contiguous");
+    const int dtype = dtype_code(q, k, v, out, "flash_attn");
+    STD_TORCH_CHECK(mask.scalar_type() == ScalarType::Bool, "flash_attn: mask must be bool");
+    STD_TORCH_CHECK(q.sizes().equals(out.sizes()), "flash_attn: q and out shapes differ");
+    STD_TORCH_CHECK(k.sizes().equals(v.sizes()), "flash_attn: k and v shapes differ");
+    STD_TORCH_CHECK(q.size(0) == k.size(0) && q.size(0) == mask.size(0) && mask.size(1) == 1 &&
+                    q.size(2) == k.size(2) && q.size(2) == mask.size(2) && q.size(2) == mask.size(3) &&
+                    q.size(3) == k.size(3),
+                    "flash_attn: expected q [B,Hq,L,D], k/v [B,Hkv,L,D], mask [B,1,L,L]");
+    const int64_t B = q.size(0), Hq = q.size(1), Hkv = k.size(1), L = q.size(2), D = q.size(3);
+    STD_TORCH_CHECK(D == 128 || D == 64, "flash_attn: head_dim must be 128 (or 64)");
+    if (B == 0 || L == 0) return;
+
+    const minfer_attn_strides st = strides_of(q, k, out);
+    const size_t ws_bytes = minfer_flash_attn_workspace_bytes(B, L);
+    Tensor ws = byte_workspace(q, ws_bytes);
+    check_rc(minfer_flash_attn(dtype, q.const_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
+                               static_cast<const uint8_t*>(mask.const_data_ptr()), out.mutable_data_ptr(),
+                               B, Hq, Hkv, L, D, &st, ws.mutable_data_ptr(), ws_bytes, current_stream()),
+             "flash_attn");
+}
+
+// Decode over a KV cache laid out like the reference's cache (reference: src/minfer/core.py:105-127).
+void flash_attn_decode_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size,
+                           const Tensor& q,         // [B, n_heads, 1, HEAD_DIM]
+                           const Tensor& k_cache,   // [B, n_kv_heads, Lmax, HEAD_DIM]
+                           const Tensor& v_cache,   // [B, n_kv_heads, Lmax, HEAD_DIM]
+                           const Tensor& ctx_lens,  // [B] int32
+                           Tensor& out) {           // [B, n_heads, 1, HEAD_DIM]
+    (void)qtype_int; (void)qblock_size; (void)qtype_size;
+    STD_TORCH_CHECK(on_gpu(q) && on_gpu(k_cache) && on_gpu(v_cache) && on_gpu(ctx_lens) && on_gpu(out),
+                    "flash_attn_decode: all tensors must be on the GPU");
+    STD_TORCH_CHECK(q.dim() == 4 && k_cache.dim() == 4 && v_cache.dim() == 4 && out.dim() == 4 && ctx_lens.dim() == 1,
+                    "flash_attn_decode: q, k_cache, v_cache, out must be 4-D and ctx_lens 1-D");
+    STD_TORCH_CHECK(q.stride(-1) == 1 && k_cache.stride(-1) == 1 && v_cache.stride(-1) == 1 && out.stride(-1) == 1,
+                    "flash_attn_decode: tensors must be contiguous in head_dim");
+    STD_TORCH_CHECK(k_cache.stride(0) == v_cache.stride(0) && k_cache.stride(1) == v_cache.stride(1) &&
+                    k_cache.stride(2) == v_cache.stride(2), "flash_attn_decode: k_cache and v_cache must share strides");
+    const int dtype = dtype_code(q, k_cache, v_cache, out, "flash_attn_decode");
+    STD_TORCH_CHECK(ctx_lens.scalar_type() == ScalarType::Int && ctx_lens.is_contiguous(),
+                    "flash_attn_decode: ctx_lens must be contiguous int32");
+    STD_TORCH_CHECK(q.sizes().equals(out.sizes()), "flash_attn_decode: q and out shapes differ");
+    STD_TORCH_CHECK(k_cache.sizes().equals(v_cache.sizes()), "flash_attn_decode: cache shapes differ");
+    STD_TORCH_CHECK(q.size(2) == 1 && q.size(0) == k_cache.size(0) && q.size(0) == ctx_lens.size(0) &&
+                    q.size(3) == k_cache.size(3),
+                    "flash_attn_decode: expected q [B,Hq,1,D], caches [B,Hkv,Lmax,D], ctx_lens [B]");
+    const int64_t B = q.size(0), Hq = q.size(1), Hkv = k_cache.size(1), Lmax = k_cache.size(2), D = q.size(3);
+    STD_TORCH_CHECK(D == 128 || D == 64, "flash_attn_decode: head_dim must be 128 or 64");
+    if (B == 0) return;
+
+    const minfer_attn_strides st = strides_of(q, k_cache, out);
+    const size_t ws_bytes = minfer_flash_attn_decode_workspace_bytes(B, Hq, Lmax, D);
+    Tensor ws = byte_workspace(q, ws_bytes);
+    check_rc(minfer_flash_attn_decode(dtype, q.const_data_ptr(), k_cache.const_data_ptr(), v_cache.const_data_ptr(),
+                                      static_cast<const int32_t*>(ctx_lens.const_data_ptr()), out.mutable_data_ptr(),
+                                      B, Hq, Hkv, Lmax, D, &st, ws.mutable_data_ptr(), ws_bytes, current_stream()),
+             "flash_attn_decode");
+}
+
+// Packed ragged causal prefill.
+void flash_attn_varlen_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size,
+                           const Tensor& q,           // [1, n_heads, T, HEAD_DIM]
+                           const Tensor& k,           // [1, n_kv_heads, T, HEAD_DIM]
+                           const Tensor& v,           // [1, n_kv_heads, T, HEAD_DIM]
+                           const Tensor& cu_seqlens,  // [n_seqs + 1] int32
+                           int64_t max_seqlen,
+                           Tensor& out) {             // [1, n_heads, T, HEAD_DIM]
+    (void)qtype_int; (void)qblock_size; (void)qtype_size;
+    STD_TORCH_CHECK(on_gpu(q) && on_gpu(k) && on_gpu(v) && on_gpu(cu_seqlens) && on_gpu(out),
+                    "flash_attn_varlen: all tensors must be on the GPU");
+    STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && out.dim() == 4 && cu_seqlens.dim() == 1,
+                    "flash_attn_varlen: q, k, v, out must be 4-D and cu_seqlens 1-D");
+    STD_TORCH_CHECK(q.stride(-1) == 1 && k.stride(-1) == 1 && v.stride(-1) == 1 && out.stride(-1) == 1,
+                    "flash_attn_varlen: tensors must be contiguous in head_dim");
+    STD_TORCH_CHECK(k.stride(1) == v.stride(1) && k.stride(2) == v.stride(2), "flash_attn_varlen: k and v must share strides");
+    const int dtype = dtype_code(q, k, v, out, "flash_attn_varlen");
+    STD_TORCH_CHECK(cu_seqlens.scalar_type() == ScalarType::Int && cu_seqlens.is_contiguous() && cu_seqlens.size(0) >= 1,
+                    "flash_attn_varlen: cu_seqlens must be contiguous int32 with at least one entry");
+    STD_TORCH_CHECK(q.sizes().equals(out.sizes()), "flash_attn_varlen: q and out shapes differ");
+    STD_TORCH_CHECK(k.sizes().equals(v.sizes()), "flash_attn_varlen: k and v shapes differ");
+    STD_TORCH_CHECK(q.size(0) == 1 && k.size(0) == 1 && q.size(2) == k.size(2) && q.size(3) == k.size(3),
+                    "flash_attn_varlen: expected q [1,Hq,T,D], k/v [1,Hkv,T,D]");
+    const int64_t Hq = q.size(1), Hkv = k.size(1), T = q.size(2), D = q.size(3);
+    STD_TORCH_CHECK(D == 128 || D == 64, "flash_attn_varlen: head_dim must be 128 or 64");
+    const int64_t n_seqs = cu_seqlens.size(0) - 1;
+    if (n_seqs == 0 || T == 0) return;
+
+    const minfer_attn_strides st = strides_of(q, k, out);
+    check_rc(minfer_flash_attn_varlen(dtype, q.const_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
+                                      static_cast<const int32_t*>(cu_seqlens.const_data_ptr()), n_seqs, max_seqlen,
+                                      out.mutable_data_ptr(), Hq, Hkv, T, D, &st, current_stream()),
+             "flash_attn_varlen");
+}
+
+STABLE_TORCH_LIBRARY(minfer, m) {
+    // verbatim the reference's schema (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:30)
+    m.def("flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()");
+    // extensions in the same style: ints first, inputs, out-parameter last, no return value
+    m.def("flash_attn_decode(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k_cache, Tensor v_cache, Tensor ctx_lens, Tensor(a!) out) -> ()");
+    m.def("flash_attn_varlen(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor cu_seqlens, int max_seqlen, Tensor(a!) out) -> ()");
+}
+
+STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-key name for ROCm devices too
+    m.impl("flash_attn", TORCH_BOX(&flash_attn_hip));
+    m.impl("flash_attn_decode", TORCH_BOX(&flash_attn_decode_hip));
+    m.impl("flash_attn_varlen", TORCH_BOX(&flash_attn_varlen_hip));
+}
+
+}  // namespace minfer

@@ -1,0 +1,23 @@
+"""Element-type identifiers the attention operators are called with.
+
+Callers pass ``qtype, *GGML_QUANT_SIZES[qtype]`` as the three leading integers of every op
+(reference: test/kernels.py:226-227, apps/benchmark.py:216-217).  The numbering is GGML's
+(reference: src/minfer/const.py:4-35).  Only the types an attention activation can have are
+listed; the quantised weight formats of the reference belong to its dequant/gemm ops.
+"""
+from enum import IntEnum
+
+
+class GGMLQuantizationType(IntEnum):
+    F32 = 0
+    F16 = 1
+    BF16 = 30
+
+
+# (elements per block, bytes per block); reference: src/minfer/const.py:39-41.  The reference
+# lists BF16 as (256, 512) at const.py:67, the same bytes per element.
+GGML_QUANT_SIZES: dict[GGMLQuantizationType, tuple[int, int]] = {
+    GGMLQuantizationType.F32: (1, 4),
+    GGMLQuantizationType.F16: (1, 2),
+    GGMLQuantizationType.BF16: (1, 2),
+}

@@ -1,0 +1,13 @@
+"""Kernel facade, same shape as the reference's (reference: src/minfer/kernels/__init__.py:2-18):
+an attribute bag of callables for one backend.  Only the attention path lives here."""
+
+
+class KernelBackend:
+    def __init__(self, backend: str):
+        if backend == "torch_ext":
+            from .torch_ext import flash_attn, flash_attn_decode, flash_attn_varlen
+            self.flash_attn = flash_attn
+            self.flash_attn_decode = flash_attn_decode
+            self.flash_attn_varlen = flash_attn_varlen
+        else:
+            raise ValueError(f"KernelBackend init: unsupported backend {backend}")

@@ -1,0 +1,82 @@
+"""Python wrappers and fake (meta) kernels of the attention ops, mirroring the reference's
+wrapper layer (reference: src/minfer/kernels/torch_ext/ops.py:234-266): positional pass-through
+to ``torch.ops.minfer.<op>.default``; the result is written into ``out``."""
+import torch
+
+_ACT_DTYPES = (torch.float16, torch.bfloat16)
+
+
+def flash_attn(
+    qtype_int: int,
+    qblock_size: int,
+    qtype_size: int,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    mask: torch.Tensor,
+    out: torch.Tensor,
+):
+    """Fused GQA attention under a dense bool mask [B,1,L,L] (True = attend).
+    q/out [B,n_heads,L,D], k/v [B,n_kv_heads,L,D], any strides with unit stride on D."""
+    return torch.ops.minfer.flash_attn.default(qtype_int, qblock_size, qtype_size, q, k, v, mask, out)
+
+
+@torch.library.register_fake("minfer::flash_attn")
+def _(qtype_int, qblock_size, qtype_size, q, k, v, mask, out):
+    torch._check(q.dtype in _ACT_DTYPES)
+    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and out.dtype == q.dtype)
+    torch._check(mask.dtype == torch.bool)
+    torch._check(q.device == k.device == v.device == out.device)
+    torch._check(q.device.type == "cuda")
+    torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and mask.dim() == 4 and out.dim() == 4)
+
+
+def flash_attn_decode(
+    qtype_int: int,
+    qblock_size: int,
+    qtype_size: int,
+    q: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+    ctx_lens: torch.Tensor,
+    out: torch.Tensor,
+):
+    """Single-token decode: q/out [B,n_heads,1,D] against caches [B,n_kv_heads,Lmax,D]; query b
+    attends cache rows 0..ctx_lens[b]-1 (ctx_lens int32 [B])."""
+    return torch.ops.minfer.flash_attn_decode.default(qtype_int, qblock_size, qtype_size, q, k_cache, v_cache, ctx_lens, out)
+
+
+@torch.library.register_fake("minfer::flash_attn_decode")
+def _(qtype_int, qblock_size, qtype_size, q, k_cache, v_cache, ctx_lens, out):
+    torch._check(q.dtype in _ACT_DTYPES)
+    torch._check(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and out.dtype == q.dtype)
+    torch._check(ctx_lens.dtype == torch.int32)
+    torch._check(q.device == k_cache.device == v_cache.device == ctx_lens.device == out.device)
+    torch._check(q.device.type == "cuda")
+    torch._check(q.dim() == 4 and k_cache.dim() == 4 and v_cache.dim() == 4 and out.dim() == 4 and ctx_lens.dim() == 1)
+
+
+def flash_attn_varlen(
+    qtype_int: int,
+    qblock_size: int,
+    qtype_size: int,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens: torch.Tensor,
+    max_seqlen: int,
+    out: torch.Tensor,
+):
+    """Packed ragged causal prefill: q/out [1,n_heads,T,D], k/v [1,n_kv_heads,T,D], cu_seqlens
+    int32 [n_seqs+1]; rows cu_seqlens[s]..cu_seqlens[s+1]-1 attend causally among themselves."""
+    return torch.ops.minfer.flash_attn_varlen.default(qtype_int, qblock_size, qtype_size, q, k, v, cu_seqlens, max_seqlen, out)
+
+
+@torch.library.register_fake("minfer::flash_attn_varlen")
+def _(qtype_int, qblock_size, qtype_size, q, k, v, cu_seqlens, max_seqlen, out):
+    torch._check(q.dtype in _ACT_DTYPES)
+    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and out.dtype == q.dtype)
+    torch._check(cu_seqlens.dtype == torch.int32)
+    torch._check(q.device == k.device == v.device == cu_seqlens.device == out.device)
+    torch._check(q.device.type == "cuda")
+    torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and out.dim() == 4 and cu_seqlens.dim() == 1)

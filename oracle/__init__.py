@@ -1,0 +1,110 @@
+"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c.
+
+Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py may import this
+package.  The shipped operator never does: it launches HIP kernels or raises.
+
+Each wrapper takes numpy arrays or torch CPU tensors of any float dtype, up-casts them to
+contiguous fp32 and returns a float32 numpy array in the reference operator's layout
+([B,Hq,L,D]; reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/op.cuh:21-30).
+"""
+import ctypes
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+
+class _Strides(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("q0", "q1", "q2", "kv0", "kv1", "kv2", "o0", "o1", "o2")]
+
+
+def build(force=False):
+    """Compile attn_oracle.c into liboracle.so (gcc + OpenMP)."""
+    so = os.path.join(_HERE, "liboracle.so")
+    if force and os.path.exists(so):
+        os.remove(so)
+    subprocess.run(["make", "-C", _HERE, "liboracle.so"], check=True, stdout=subprocess.DEVNULL)
+    return so
+
+
+def lib():
+    global _LIB
+    if _LIB is None:
+        so = os.path.join(_HERE, "liboracle.so")
+        if not os.path.exists(so):
+            build()
+        _LIB = ctypes.CDLL(so)
+        for name in ("oracle_flash_attn", "oracle_flash_attn_decode", "oracle_flash_attn_varlen"):
+            getattr(_LIB, name).restype = ctypes.c_int
+    return _LIB
+
+
+def _f32(x):
+    if hasattr(x, "detach"):
+        x = x.detach().to("cpu").float().numpy()
+    return np.ascontiguousarray(np.asarray(x, dtype=np.float32))
+
+
+def _ptr(a, ty=ctypes.c_float):
+    return a.ctypes.data_as(ctypes.POINTER(ty))
+
+
+def _contig_strides(q, k, o):
+    s = lambda a: [x // a.itemsize for x in a.strides[:3]]
+    return _Strides(*s(q), *s(k), *s(o))
+
+
+def flash_attn(q, k, v, mask):
+    """Dense bool-mask GQA attention; the reference op's semantics (refs.py:53-55)."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    if hasattr(mask, "detach"):
+        mask = mask.detach().to("cpu").numpy()
+    B, Hq, L, D = q.shape
+    Hkv = k.shape[1]
+    mask = np.ascontiguousarray(np.broadcast_to(np.asarray(mask, dtype=np.bool_), (B, 1, L, L))).view(np.uint8)
+    out = np.empty_like(q)
+    st = _contig_strides(q, k, out)
+    rc = lib().oracle_flash_attn(_ptr(q), _ptr(k), _ptr(v), _ptr(mask, ctypes.c_uint8), _ptr(out),
+                                 *[ctypes.c_int64(x) for x in (B, Hq, Hkv, L, D)], ctypes.byref(st))
+    if rc != 0:
+        raise ValueError(f"oracle_flash_attn rc={rc}")
+    return out
+
+
+def flash_attn_decode(q, k_cache, v_cache, ctx_lens):
+    """q [B,Hq,1,D] against caches [B,Hkv,Lmax,D], keys 0..ctx_lens[b]-1."""
+    q, k_cache, v_cache = _f32(q), _f32(k_cache), _f32(v_cache)
+    if hasattr(ctx_lens, "detach"):
+        ctx_lens = ctx_lens.detach().to("cpu").numpy()
+    ctx = np.ascontiguousarray(np.asarray(ctx_lens, dtype=np.int32))
+    B, Hq, _, D = q.shape
+    Hkv, Lmax = k_cache.shape[1], k_cache.shape[2]
+    out = np.empty_like(q)
+    st = _contig_strides(q, k_cache, out)
+    rc = lib().oracle_flash_attn_decode(_ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(ctx, ctypes.c_int32),
+                                        _ptr(out), *[ctypes.c_int64(x) for x in (B, Hq, Hkv, Lmax, D)],
+                                        ctypes.byref(st))
+    if rc != 0:
+        raise ValueError(f"oracle_flash_attn_decode rc={rc}")
+    return out
+
+
+def flash_attn_varlen(q, k, v, cu_seqlens):
+    """Packed ragged causal prefill: q [1,Hq,T,D], k/v [1,Hkv,T,D], cu_seqlens [N+1]."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    if hasattr(cu_seqlens, "detach"):
+        cu_seqlens = cu_seqlens.detach().to("cpu").numpy()
+    cu = np.ascontiguousarray(np.asarray(cu_seqlens, dtype=np.int32))
+    _, Hq, T, D = q.shape
+    Hkv = k.shape[1]
+    out = np.empty_like(q)
+    st = _contig_strides(q, k, out)
+    rc = lib().oracle_flash_attn_varlen(_ptr(q), _ptr(k), _ptr(v), _ptr(cu, ctypes.c_int32),
+                                        ctypes.c_int64(len(cu) - 1), _ptr(out),
+                                        *[ctypes.c_int64(x) for x in (Hq, Hkv, T, D)], ctypes.byref(st))
+    if rc != 0:
+        raise ValueError(f"oracle_flash_attn_varlen rc={rc}")
+    return out
