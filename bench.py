@@ -1,0 +1,159 @@
+"""Benchmark of the fused-attention hot path on one MI355X.
+
+A step is one call of the prefill operator on the Llama-3-8B-shaped workload (B=1, Hq=32, Hkv=8,
+S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmic TFLOP/s
+(4*D*Hq*attended pairs), inputs resident in HBM, every kernel the op launches inside the timed
+region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
+under "decode" with its own HBM roofline, and the reference's CPU attention path (torch SDPA in
+fp32 on the host cores) under "cpu_baseline".  Prints ONE JSON line.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+PKG = os.path.join(ROOT, "minfer-python_amd")
+for p in (ROOT, PKG, os.path.join(PKG, "apps")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16/bf16
+PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+
+
+class HipEvents:
+    """hipEvent timing on an explicit stream through libamdhip64 (the kernels are launched on the
+    stream handed to the op, which is torch's current stream)."""
+
+    def __init__(self):
+        import torch
+        self.hip = ctypes.CDLL(os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so"))
+        self.hip.hipEventCreate.argtypes = [ctypes.POINTER(ctypes.c_void_p)]
+        self.hip.hipEventRecord.argtypes = [ctypes.c_void_p, ctypes.c_void_p]
+        self.hip.hipEventSynchronize.argtypes = [ctypes.c_void_p]
+        self.hip.hipEventElapsedTime.argtypes = [ctypes.POINTER(ctypes.c_float), ctypes.c_void_p, ctypes.c_void_p]
+
+    def event(self):
+        e = ctypes.c_void_p()
+        assert self.hip.hipEventCreate(ctypes.byref(e)) == 0
+        return e
+
+    def time_each(self, fn, stream, n):
+        """Average and median duration (ms) of n calls of fn, each bracketed by events on `stream`."""
+        pairs = [(self.event(), self.event()) for _ in range(n)]
+        for a, b in pairs:
+            assert self.hip.hipEventRecord(a, stream) == 0
+            fn()
+            assert self.hip.hipEventRecord(b, stream) == 0
+        ms = []
+        for a, b in pairs:
+            assert self.hip.hipEventSynchronize(b) == 0
+            t = ctypes.c_float()
+            assert self.hip.hipEventElapsedTime(ctypes.byref(t), a, b) == 0
+            ms.append(t.value)
+        ms_sorted = sorted(ms)
+        return sum(ms) / len(ms), ms_sorted[len(ms) // 2]
+
+
+def cpu_baseline(torch, workloads, refs, L):
+    """The reference's CPU attention path: refs.flash_attn = torch SDPA, fp32, K/V pre-expanded outside
+    the timed region, on the same seeded inputs up-cast (reference: apps/benchmark.py:240-248)."""
+    q, k, v, mask = workloads.llama8b_prefill(seed=0, L=L)
+    q, k, v = q.float(), k.float().repeat_interleave(4, 1), v.float().repeat_interleave(4, 1)
+    refs.flash_attn(q[:, :4], k[:, :4], v[:, :4], mask)  # warm-up on a slice
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        refs.flash_attn(q, k, v, mask)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[1]
+    flops = workloads.prefill_flops(32, 128, [L])
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"refs.flash_attn (torch SDPA, fp32, dense causal mask) on the full S={L} workload, median of 3: {t * 1e3:.1f} ms",
+            "host_cpus": os.cpu_count()}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the attention path shards by batch / KV head without any "
+                 "exchange, and this build has no multi-GPU launcher. Run with --gpus 1.")
+
+    import torch
+    import workloads
+    from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
+    from minfer.kernels import KernelBackend, refs
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU: the operators have no CPU implementation")
+    kerns = KernelBackend("torch_ext")
+    dev = "cuda:0"
+    torch.cuda.set_device(0)
+    qt = GGMLQuantizationType.F16
+    qb, qs = GGML_QUANT_SIZES[qt]
+    ev = HipEvents()
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    # ---- prefill: the step -----------------------------------------------------------------
+    L = 4096
+    q, k, v, mask = workloads.llama8b_prefill(seed=0, device=dev, L=L)
+    out = torch.zeros_like(q)
+    step = lambda: kerns.flash_attn(qt, qb, qs, q, k, v, mask, out)
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    avg_ms, med_ms = ev.time_each(step, stream, max(args.steps, 20))
+    flops = workloads.prefill_flops(32, 128, [L])
+    tflops = flops / (wall_ms * 1e-3) / 1e12
+    achieved = flops / (avg_ms * 1e-3) / 1e12
+
+    # ---- decode ------------------------------------------------------------------------------
+    qd, kc, vc, ctx = workloads.decode_cache(seed=0, device=dev)
+    outd = torch.zeros_like(qd)
+    dstep = lambda: kerns.flash_attn_decode(qt, qb, qs, qd, kc, vc, ctx, outd)
+    for _ in range(args.warmup):
+        dstep()
+    torch.cuda.synchronize()
+    d_avg_ms, d_med_ms = ev.time_each(dstep, stream, max(args.steps, 20))
+    dbytes = workloads.decode_bytes(ctx.tolist(), 32, 8, 128)
+    d_gbs = dbytes / (d_avg_ms * 1e-3) / 1e9
+    del kc, vc
+
+    rec = {
+        "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
+        "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "prefill B=1 Hq=32 Hkv=8 S=4096 D=128 fp16 causal dense-mask (BASELINE configs[1])",
+                   "global_batch": 1, "seq_len": L, "parallelism": "single-gpu"},
+        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": achieved / PEAK_MFMA_TFLOPS, "traffic": None,
+                     "kernel": "classify_mask_kernel + prefill_kernel<F16,128,dense>",
+                     "algorithmic_flops": flops, "avg_ms": avg_ms, "median_ms": med_ms},
+        "decode": {"value": d_gbs, "unit": "GB/s", "ms": d_avg_ms, "median_ms": d_med_ms,
+                   "workload": "decode B=64 Hq=32 Hkv=8 D=128 fp16 ctx~U[512,8192] cache [64,8,8192,128] (BASELINE configs[2])",
+                   "roofline": {"bound": "hbm", "achieved": d_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                "frac": d_gbs / PEAK_HBM_GBS, "traffic": None,
+                                "kernel": "decode_split_kernel<F16,128> + decode_combine_kernel",
+                                "algorithmic_bytes": dbytes}},
+    }
+    if not args.no_cpu_baseline:
+        rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
+    print(json.dumps(rec))
+
+
+if __name__ == "__main__":
+    main()

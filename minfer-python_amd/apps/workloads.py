@@ -1,0 +1,103 @@
+"""Seeded synthetic inputs for the attention workloads that tests, benchmarks and profiles share.
+
+Every generator draws from ``torch.Generator().manual_seed(seed)`` on the CPU (so the same seed
+gives the same bytes on any machine) and returns CPU tensors unless ``device`` is given.  The
+input recipes follow the reference's callers (reference: test/kernels.py:225-244,
+apps/benchmark.py:215-237): q/k/v are drawn as [B, L, H*D] and handed over as the transposed
+view [B, H, L, D] when ``views=True``.
+"""
+import torch
+
+
+def _qkv(gen, B, H, L, D, scale, dtype, views):
+    if views:
+        x = (scale * torch.randn(B, L, H * D, generator=gen)).to(dtype)
+        return x.view(B, L, H, D).transpose(1, 2)
+    return (scale * torch.randn(B, H, L, D, generator=gen)).to(dtype)
+
+
+def causal_mask(B, L, device="cpu"):
+    i = torch.arange(L, device=device)
+    return (i[None, :] <= i[:, None])[None, None].expand(B, 1, L, L).contiguous()
+
+
+def window_mask(B, L, window, device="cpu"):
+    i = torch.arange(L, device=device)
+    return ((i[None, :] - i[:, None]).abs() < window)[None, None].expand(B, 1, L, L).contiguous()
+
+
+def dense_prefill(B, Hq, Hkv, L, D, dtype, seed=0, scale=0.5, views=False, device="cpu"):
+    """q [B,Hq,L,D], k/v [B,Hkv,L,D] ~ scale * N(0,1)."""
+    gen = torch.Generator().manual_seed(seed)
+    q = _qkv(gen, B, Hq, L, D, scale, dtype, views)
+    k = _qkv(gen, B, Hkv, L, D, scale, dtype, views)
+    v = _qkv(gen, B, Hkv, L, D, scale, dtype, views)
+    if device != "cpu":
+        if views:  # keep the strided layout on the device
+            q, k, v = (t.transpose(1, 2).to(device).transpose(1, 2) for t in (q, k, v))
+        else:
+            q, k, v = q.to(device), k.to(device), v.to(device)
+    return q, k, v
+
+
+def cpu_plumbing(seed=0):
+    """B=1, Hq=8, Hkv=2, S=256, D=64, fp32, N(0,1), causal."""
+    q, k, v = dense_prefill(1, 8, 2, 256, 64, torch.float32, seed=seed, scale=1.0)
+    return q, k, v, causal_mask(1, 256)
+
+
+def llama8b_prefill(seed=0, device="cpu", views=False, L=4096):
+    """B=1, Hq=32, Hkv=8, S=4096, D=128, fp16, 0.5*N(0,1), causal."""
+    q, k, v = dense_prefill(1, 32, 8, L, 128, torch.float16, seed=seed, scale=0.5, views=views, device=device)
+    return q, k, v, causal_mask(1, L, device=device)
+
+
+def long_context_prefill(seed=0, device="cpu", L=32768):
+    """B=1, Hq=32, Hkv=8, S=32768, D=128, bf16, 0.5*N(0,1), causal."""
+    q, k, v = dense_prefill(1, 32, 8, L, 128, torch.bfloat16, seed=seed, scale=0.5, device=device)
+    return q, k, v, causal_mask(1, L, device=device)
+
+
+def decode_cache(seed=0, device="cpu", B=64, Hq=32, Hkv=8, Lmax=8192, D=128, dtype=torch.float16,
+                 ctx_lo=512, ctx_hi=8192):
+    """q [B,Hq,1,D] ~ N(0,1); caches [B,Hkv,Lmax,D] ~ N(0,1); ctx_lens uniform in [ctx_lo, ctx_hi]."""
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Hq, 1, D, generator=gen).to(dtype)
+    ctx = torch.randint(ctx_lo, ctx_hi + 1, (B,), generator=gen, dtype=torch.int32)
+    if device == "cpu":
+        kc = torch.randn(B, Hkv, Lmax, D, generator=gen).to(dtype)
+        vc = torch.randn(B, Hkv, Lmax, D, generator=gen).to(dtype)
+    else:  # the 2 GiB of cache entries are drawn on the device from the same seed
+        dgen = torch.Generator(device=device).manual_seed(seed)
+        kc = torch.randn(B, Hkv, Lmax, D, generator=dgen, device=device, dtype=dtype)
+        vc = torch.randn(B, Hkv, Lmax, D, generator=dgen, device=device, dtype=dtype)
+        q, ctx = q.to(device), ctx.to(device)
+    return q, kc, vc, ctx
+
+
+def ragged_prefill(seed=0, device="cpu", n_seqs=16, len_lo=128, len_hi=2048, Hq=64, Hkv=8, D=128,
+                   dtype=torch.float16, scale=1.0):
+    """Packed sequences with lengths uniform in [len_lo, len_hi]: q [1,Hq,T,D], k/v [1,Hkv,T,D] ~ N(0,1),
+    cu_seqlens int32 [n_seqs+1]."""
+    gen = torch.Generator().manual_seed(seed)
+    lens = torch.randint(len_lo, len_hi + 1, (n_seqs,), generator=gen)
+    cu = torch.zeros(n_seqs + 1, dtype=torch.int32)
+    cu[1:] = lens.cumsum(0).to(torch.int32)
+    T = int(cu[-1])
+    q = (scale * torch.randn(1, Hq, T, D, generator=gen)).to(dtype)
+    k = (scale * torch.randn(1, Hkv, T, D, generator=gen)).to(dtype)
+    v = (scale * torch.randn(1, Hkv, T, D, generator=gen)).to(dtype)
+    if device != "cpu":
+        q, k, v, cu = q.to(device), k.to(device), v.to(device), cu.to(device)
+    return q, k, v, cu
+
+
+def prefill_flops(Hq, D, lens):
+    """4*D*Hq*(attended pairs) for causal sequences of the given lengths."""
+    return 2 * D * Hq * sum(int(n) * (int(n) + 1) for n in lens)
+
+
+def decode_bytes(ctx_lens, Hq, Hkv, D, itemsize=2):
+    """K and V rows read once per KV head, plus q and out."""
+    B = len(ctx_lens)
+    return int(sum(int(c) for c in ctx_lens)) * Hkv * D * 2 * itemsize + 2 * B * Hq * D * itemsize

@@ -46,6 +46,11 @@ struct F16 {
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
     }
     static MA_DEV float to_float(short bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+    // acc + lo + hi of a packed pair, in fp32: sums exactly the rounded values the MFMA consumes
+    static MA_DEV float add_pair(uint32_t pair, float acc) {
+        const h16x2 ones = {(_Float16)1.f, (_Float16)1.f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, pair), ones, acc, false);
+    }
 };
 
 struct BF16 {
@@ -66,6 +71,10 @@ struct BF16 {
     }
     static MA_DEV float to_float(short bits) {
         return __builtin_bit_cast(float, (uint32_t)(uint16_t)bits << 16);
+    }
+    static MA_DEV float add_pair(uint32_t pair, float acc) {
+        const b16x2 ones = {(__bf16)1.f, (__bf16)1.f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b16x2, pair), ones, acc, false);
     }
 };
 

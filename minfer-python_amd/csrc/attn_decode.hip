@@ -164,8 +164,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64, 2) void decode_split_kernel(cons
         const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * c2;
         const float p0 = fast_exp2(fmaf(s[0], c2, -mc)), p1 = fast_exp2(fmaf(s[1], c2, -mc));
         const float p2 = fast_exp2(fmaf(s[2], c2, -mc)), p3 = fast_exp2(fmaf(s[3], c2, -mc));
-        l_sum += (p0 + p1) + (p2 + p3);
         uint2 pu; pu.x = T::pack2(p0, p1); pu.y = T::pack2(p2, p3);
+        l_sum = T::add_pair(pu.y, T::add_pair(pu.x, l_sum));   // sums the rounded weights the MFMA uses
         const s16x4 pfrag = __builtin_bit_cast(s16x4, pu);
 
         // ---- O^T += V^T P^T: A = V^T block (row d = 16db + l16, k = keys 4*quad + 0..3) -----------

@@ -375,8 +375,9 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
                 for (int r = 0; r < 16; r += 2) {
                     const float p0 = fast_exp2(fmaf(s_acc[kb][r], c2, -mc));
                     const float p1 = fast_exp2(fmaf(s_acc[kb][r + 1], c2, -mc));
-                    ls += p0 + p1;
-                    pf[2 * kb + (r >> 3)][(r & 7) >> 1] = T::pack2(p0, p1);
+                    const uint32_t pk = T::pack2(p0, p1);
+                    ls = T::add_pair(pk, ls);   // the denominator sums the rounded weights the MFMA uses
+                    pf[2 * kb + (r >> 3)][(r & 7) >> 1] = pk;
                 }
             }
             l_sum += ls;

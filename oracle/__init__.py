@@ -37,7 +37,8 @@ def lib():
         if not os.path.exists(so):
             build()
         _LIB = ctypes.CDLL(so)
-        for name in ("oracle_flash_attn", "oracle_flash_attn_decode", "oracle_flash_attn_varlen"):
+        for name in ("oracle_flash_attn", "oracle_flash_attn_rows", "oracle_flash_attn_decode",
+                     "oracle_flash_attn_varlen"):
             getattr(_LIB, name).restype = ctypes.c_int
     return _LIB
 
@@ -71,6 +72,27 @@ def flash_attn(q, k, v, mask):
                                  *[ctypes.c_int64(x) for x in (B, Hq, Hkv, L, D)], ctypes.byref(st))
     if rc != 0:
         raise ValueError(f"oracle_flash_attn rc={rc}")
+    return out
+
+
+def flash_attn_rows(q, k, v, mask_rows, rows):
+    """flash_attn restricted to query rows `rows`; mask_rows is bool [B,n,L] (= mask[:,0,rows,:]).
+    Returns [B,Hq,n,D]."""
+    q, k, v = _f32(q), _f32(k), _f32(v)
+    if hasattr(mask_rows, "detach"):
+        mask_rows = mask_rows.detach().to("cpu").numpy()
+    B, Hq, L, D = q.shape
+    Hkv = k.shape[1]
+    rows = np.ascontiguousarray(np.asarray(rows, dtype=np.int64))
+    n = len(rows)
+    mask_rows = np.ascontiguousarray(np.broadcast_to(np.asarray(mask_rows, dtype=np.bool_), (B, n, L))).view(np.uint8)
+    out = np.empty((B, Hq, n, D), dtype=np.float32)
+    st = _contig_strides(q, k, q)
+    rc = lib().oracle_flash_attn_rows(_ptr(q), _ptr(k), _ptr(v), _ptr(mask_rows, ctypes.c_uint8),
+                                      _ptr(rows, ctypes.c_int64), ctypes.c_int64(n), _ptr(out),
+                                      *[ctypes.c_int64(x) for x in (B, Hq, Hkv, L, D)], ctypes.byref(st))
+    if rc != 0:
+        raise ValueError(f"oracle_flash_attn_rows rc={rc}")
     return out
 
 

@@ -108,6 +108,34 @@ int oracle_flash_attn(const float* q, const float* k, const float* v, const uint
     return 0;
 }
 
+/* Same as oracle_flash_attn for a subset of query rows only (so that full-size problems can be
+ * spot-checked in seconds): rows[n] are query indices, mask_rows is [B,n,L] bool bytes holding
+ * mask[b,0,rows[r],:]; out is contiguous [B,Hq,n,D]. */
+int oracle_flash_attn_rows(const float* q, const float* k, const float* v, const uint8_t* mask_rows,
+                           const int64_t* rows, int64_t n, float* out,
+                           int64_t B, int64_t Hq, int64_t Hkv, int64_t L, int64_t D,
+                           const oracle_strides* st)
+{
+    if (D > 512 || Hq % Hkv != 0) return -1;
+    for (int64_t r = 0; r < n; ++r) if (rows[r] < 0 || rows[r] >= L) return -2;
+    const int64_t n_rep = Hq / Hkv;
+    const double scale = 1.0 / sqrt((double)D);
+    #pragma omp parallel
+    {
+        double* s_buf = (double*)malloc(sizeof(double) * (size_t)(L > 0 ? L : 1));
+        #pragma omp for schedule(dynamic, 4)
+        for (int64_t t = 0; t < B * Hq * n; ++t) {
+            int64_t r = t % n, h = (t / n) % Hq, b = t / (n * Hq), g = h / n_rep;
+            attend_row(q + b * st->q0 + h * st->q1 + rows[r] * st->q2,
+                       k + b * st->kv0 + g * st->kv1, v + b * st->kv0 + g * st->kv1, st->kv2,
+                       0, L, mask_rows + (b * n + r) * L, D, scale,
+                       out + ((b * Hq + h) * n + r) * D, s_buf);
+        }
+        free(s_buf);
+    }
+    return 0;
+}
+
 /* Single-token decode over a KV cache [B,Hkv,Lmax,D] (layout of core.py:105-127):
  * query b attends keys 0..ctx_lens[b]-1; q/out are [B,Hq,1,D] (q2/o2 unused). */
 int oracle_flash_attn_decode(const float* q, const float* k_cache, const float* v_cache,

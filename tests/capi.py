@@ -1,0 +1,97 @@
+"""ctypes view of libminfer_attn.so for the tests: calls the C ABI of include/minfer_attn.h with the
+device pointers, strides and current stream of torch tensors.  No torch types cross the boundary."""
+import ctypes
+import os
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+LIB_PATH = os.path.join(ROOT, "minfer-python_amd", "lib", "libminfer_attn.so")
+HEADER = os.path.join(ROOT, "include", "minfer_attn.h")
+
+F16, BF16 = 1, 30
+OK, EINVAL, EWORKSPACE, ELAUNCH = 0, -1, -2, -3
+
+
+class Strides(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int64) for n in ("q0", "q1", "q2", "kv0", "kv1", "kv2", "o0", "o1", "o2")]
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is not built; run python minfer-python_amd/build.py")
+        L = ctypes.CDLL(LIB_PATH)
+        i64, vp, sz = ctypes.c_int64, ctypes.c_void_p, ctypes.c_size_t
+        L.minfer_attn_version.restype = ctypes.c_int
+        L.minfer_attn_last_error.restype = ctypes.c_char_p
+        L.minfer_flash_attn_workspace_bytes.restype = sz
+        L.minfer_flash_attn_workspace_bytes.argtypes = [i64, i64]
+        L.minfer_flash_attn.restype = ctypes.c_int
+        L.minfer_flash_attn.argtypes = [ctypes.c_int, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
+                                        ctypes.POINTER(Strides), vp, sz, vp]
+        L.minfer_flash_attn_decode_workspace_bytes.restype = sz
+        L.minfer_flash_attn_decode_workspace_bytes.argtypes = [i64, i64, i64, i64]
+        L.minfer_flash_attn_decode.restype = ctypes.c_int
+        L.minfer_flash_attn_decode.argtypes = [ctypes.c_int, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
+                                               ctypes.POINTER(Strides), vp, sz, vp]
+        L.minfer_flash_attn_varlen.restype = ctypes.c_int
+        L.minfer_flash_attn_varlen.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, i64,
+                                               ctypes.POINTER(Strides), vp]
+        _lib = L
+    return _lib
+
+
+def last_error():
+    return lib().minfer_attn_last_error().decode()
+
+
+def _dtype_code(t):
+    import torch
+    return {torch.float16: F16, torch.bfloat16: BF16}[t.dtype]
+
+
+def _strides(q, k, o):
+    return Strides(q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+                   o.stride(0), o.stride(1), o.stride(2))
+
+
+def _stream():
+    import torch
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def flash_attn(q, k, v, mask, out, workspace=None):
+    """Returns the C ABI's return code; `out` is written in place."""
+    import torch
+    B, Hq, L, D = q.shape
+    need = lib().minfer_flash_attn_workspace_bytes(B, L)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    st = _strides(q, k, out)
+    return lib().minfer_flash_attn(_dtype_code(q), q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(),
+                                   out.data_ptr(), B, Hq, k.shape[1], L, D, ctypes.byref(st),
+                                   workspace.data_ptr(), workspace.numel(), _stream())
+
+
+def flash_attn_decode(q, k_cache, v_cache, ctx_lens, out, workspace=None):
+    import torch
+    B, Hq, _, D = q.shape
+    Hkv, Lmax = k_cache.shape[1], k_cache.shape[2]
+    need = lib().minfer_flash_attn_decode_workspace_bytes(B, Hq, Lmax, D)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    st = _strides(q, k_cache, out)
+    return lib().minfer_flash_attn_decode(_dtype_code(q), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                          ctx_lens.data_ptr(), out.data_ptr(), B, Hq, Hkv, Lmax, D,
+                                          ctypes.byref(st), workspace.data_ptr(), workspace.numel(), _stream())
+
+
+def flash_attn_varlen(q, k, v, cu_seqlens, max_seqlen, out):
+    _, Hq, T, D = q.shape
+    st = _strides(q, k, out)
+    return lib().minfer_flash_attn_varlen(_dtype_code(q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                          cu_seqlens.data_ptr(), cu_seqlens.numel() - 1, max_seqlen, out.data_ptr(),
+                                          Hq, k.shape[1], T, D, ctypes.byref(st), _stream())

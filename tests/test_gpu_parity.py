@@ -1,0 +1,373 @@
+"""GPU parity tests (-m gpu): the HIP kernels, called through the C ABI of libminfer_attn.so (and
+through the registered torch ops), against the CPU oracle on identical seeded inputs.
+
+Tolerances are the ones the task fixes: max-abs error <= 2e-3 for fp16 and <= 1e-2 for bf16 against
+an fp32-or-better reference.  Masking and the GQA head mapping are checked for exact equality.
+At full BASELINE sizes the oracle is evaluated on a sample of query rows (it is a scalar CPU
+program) and the whole output is additionally compared with a plain fp32 torch evaluation of the
+same formula on the GPU.
+"""
+import math
+
+import numpy as np
+import pytest
+import torch
+
+import capi
+import oracle
+import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+TOL = {torch.float16: 2e-3, torch.bfloat16: 1e-2}
+
+
+# ------------------------------------------------------------------------------------------------
+def torch_ref(q, k, v, mask, row_chunk=1024):
+    """softmax(q k^T / sqrt(D) | mask) v in fp32 on the GPU, a chunk of query rows at a time."""
+    B, Hq, L, D = q.shape
+    n_rep = Hq // k.shape[1]
+    kf = k.float().repeat_interleave(n_rep, 1).transpose(-1, -2).contiguous()
+    vf = v.float().repeat_interleave(n_rep, 1).contiguous()
+    out = torch.empty(B, Hq, L, D, dtype=torch.float32, device=q.device)
+    for lo in range(0, L, row_chunk):
+        hi = min(lo + row_chunk, L)
+        s = (q[:, :, lo:hi].float() @ kf) / math.sqrt(D)
+        s.masked_fill_(~mask[:, :, lo:hi], float("-inf"))
+        p = torch.nan_to_num(torch.softmax(s, -1), nan=0.0)
+        out[:, :, lo:hi] = p @ vf
+    return out
+
+
+def run_prefill(q, k, v, mask, out=None):
+    if out is None:
+        out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=q.device)
+    rc = capi.flash_attn(q, k, v, mask, out)
+    assert rc == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    return out
+
+
+def max_err(a, b):
+    return float((torch.as_tensor(a).float().cpu() - torch.as_tensor(b).float().cpu()).abs().max())
+
+
+def make_mask(kind, B, L, gen):
+    i = torch.arange(L)
+    if kind == "causal":
+        m = (i[None, :] <= i[:, None])[None].expand(B, L, L)
+    elif kind == "window":
+        m = ((i[None, :] - i[:, None]).abs() < 37)[None].expand(B, L, L)
+    elif kind == "full":
+        m = torch.ones(B, L, L, dtype=torch.bool)
+    elif kind == "random":       # different per batch element, with rows that attend nothing
+        m = torch.rand(B, L, L, generator=gen) < 0.5
+        m[:, L // 3, :] = False
+    elif kind == "blocky":       # whole 64x64 tiles switched off, to exercise tile skipping with holes
+        t = (L + 63) // 64
+        tiles = torch.rand(B, t, t, generator=gen) < 0.5
+        tiles[:, :, 0] = True
+        m = tiles.repeat_interleave(64, 1).repeat_interleave(64, 2)[:, :L, :L]
+    return m[:, None].contiguous()
+
+
+# ------------------------------------------------------------------------------------------------
+# golden vectors (pin: torch SDPA on the reference's call, see tests/golden/make_golden.py)
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["dense_causal_b1_h4_kv2_l16_d64", "dense_window_b2_h6_kv2_l40_d128",
+                                  "dense_random_b1_h8_kv1_l70_d64"])
+def test_golden_dense(name):
+    z = np.load(f"{capi.ROOT}/tests/golden/{name}.npz")
+    q, k, v = (torch.from_numpy(z[n]).to(DEV) for n in ("q", "k", "v"))
+    out = run_prefill(q, k, v, torch.from_numpy(z["mask"]).to(DEV))
+    assert max_err(out, z["out"]) <= TOL[torch.float16]
+
+
+def test_golden_decode_and_varlen():
+    z = np.load(f"{capi.ROOT}/tests/golden/decode_b3_h8_kv2_l50_d128.npz")
+    q, k, v = (torch.from_numpy(z[n]).to(DEV) for n in ("q", "k", "v"))
+    out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)
+    assert capi.flash_attn_decode(q, k, v, torch.from_numpy(z["ctx"]).to(DEV), out) == capi.OK, capi.last_error()
+    assert max_err(out, z["out"]) <= TOL[torch.float16]
+    z = np.load(f"{capi.ROOT}/tests/golden/varlen_h4_kv2_d64.npz")
+    q, k, v = (torch.from_numpy(z[n]).to(DEV) for n in ("q", "k", "v"))
+    out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)
+    assert capi.flash_attn_varlen(q, k, v, torch.from_numpy(z["cu"]).to(DEV), 70, out) == capi.OK, capi.last_error()
+    assert max_err(out, z["out"]) <= TOL[torch.float16]
+
+
+# ------------------------------------------------------------------------------------------------
+# dense prefill against the oracle: shapes, masks, dtypes, layouts
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hq,Hkv,L,D,kind,views", [
+    (1, 8, 2, 256, 64, "causal", False),     # BASELINE config 1 shape
+    (2, 8, 2, 320, 128, "causal", True),     # reference-style transposed views
+    (2, 6, 2, 200, 128, "window", False),    # n_rep = 3, symmetric window (reference test case B)
+    (2, 4, 4, 333, 128, "random", False),    # L % 4 != 0: byte-wise mask path, per-batch masks
+    (1, 16, 2, 520, 64, "random", True),     # n_rep = 8
+    (1, 12, 2, 136, 128, "blocky", False),   # n_rep = 6
+    (1, 16, 1, 264, 128, "causal", False),   # n_rep = 16
+    (1, 2, 2, 1, 128, "full", False),        # single token
+    (1, 4, 2, 63, 64, "causal", False),
+    (3, 4, 1, 65, 128, "full", False),
+    (1, 4, 1, 1040, 128, "blocky", False),
+])
+def test_dense_matches_oracle(dtype, B, Hq, Hkv, L, D, kind, views):
+    gen = torch.Generator().manual_seed(1000 * L + D + Hq)
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, dtype, seed=L + Hq, scale=0.5, views=views, device=DEV)
+    q = q * 2 if dtype == torch.float16 else q   # fp16: logits with a wider spread
+    mask = make_mask(kind, B, L, gen)
+    out = run_prefill(q, k, v, mask.to(DEV))
+    want = oracle.flash_attn(q, k, v, mask)
+    assert not torch.isnan(out).any()
+    assert max_err(out, want) <= TOL[dtype]
+
+
+def test_cpu_plumbing_config_on_gpu():
+    """BASELINE config 1 (fp32 N(0,1) inputs, S=256, D=64): the same seeded inputs rounded to fp16."""
+    q, k, v, mask = workloads.cpu_plumbing(seed=0)
+    want = oracle.flash_attn(q.half(), k.half(), v.half(), mask)
+    out = run_prefill(q.half().to(DEV), k.half().to(DEV), v.half().to(DEV), mask.to(DEV))
+    assert out.shape == (1, 8, 256, 64)
+    assert max_err(out, want) <= TOL[torch.float16]
+
+
+def test_strided_out_and_determinism():
+    B, Hq, Hkv, L, D = 2, 8, 2, 192, 128
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, torch.float16, seed=5, views=True, device=DEV)
+    mask = workloads.causal_mask(B, L, device=DEV)
+    a = run_prefill(q, k, v, mask)
+    out_t = torch.full((B, L, Hq, D), float("nan"), dtype=torch.float16, device=DEV).transpose(1, 2)
+    b = run_prefill(q, k, v, mask, out=out_t)
+    assert torch.equal(a, b)
+    assert torch.equal(a, run_prefill(q, k, v, mask))
+    assert max_err(a, oracle.flash_attn(q, k, v, mask)) <= TOL[torch.float16]
+
+
+# ------------------------------------------------------------------------------------------------
+# exact properties: masking and GQA mapping are bit-identical
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_masking_and_gqa_mapping_exact(dtype):
+    B, Hq, Hkv, L, D = 2, 8, 2, 200, 128
+    gen = torch.Generator().manual_seed(9)
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, dtype, seed=9, scale=1.0, device=DEV)
+    n_rep = Hq // Hkv
+    # one attended key per row: the output row is that V row, bit for bit
+    sel = torch.randint(0, L, (B, L), generator=gen)
+    onehot = torch.zeros(B, L, L, dtype=torch.bool)
+    onehot.scatter_(2, sel[:, :, None], True)
+    out = run_prefill(q, k, v, onehot[:, None].contiguous().to(DEV))
+    for b in range(B):
+        for h in range(Hq):
+            assert torch.equal(out[b, h], v[b, h // n_rep, sel[b].to(DEV)])
+    # causal: row 0 is V row 0
+    out = run_prefill(q, k, v, workloads.causal_mask(B, L, device=DEV))
+    for h in range(Hq):
+        assert torch.equal(out[:, h, 0], v[:, h // n_rep, 0])
+    # V constant per KV head: every row of query head h equals the constant of KV head h // n_rep
+    vc = torch.empty_like(v)
+    for g in range(Hkv):
+        vc[:, g] = float(g + 1)
+    out = run_prefill(q, k, vc, workloads.causal_mask(B, L, device=DEV))
+    for h in range(Hq):
+        assert torch.equal(out[:, h], torch.full_like(out[:, h], float(h // n_rep + 1)))
+    # rows that attend nothing give zeros, their neighbours are unaffected
+    m = workloads.causal_mask(B, L)
+    m[:, :, 70, :] = False
+    out2 = run_prefill(q, k, v, m.to(DEV))
+    assert torch.all(out2[:, :, 70] == 0)
+    ref = run_prefill(q, k, v, workloads.causal_mask(B, L, device=DEV))
+    keep = torch.arange(L) != 70
+    assert torch.equal(out2[:, :, keep], ref[:, :, keep])
+
+
+# ------------------------------------------------------------------------------------------------
+# BASELINE configs at full size
+# ------------------------------------------------------------------------------------------------
+def sample_rows(L, n, gen):
+    fixed = [0, 1, 31, 32, 63, 64, 65, L // 2, L - 65, L - 2, L - 1]
+    extra = torch.randint(0, L, (n,), generator=gen).tolist()
+    return sorted(set(r for r in fixed + extra if 0 <= r < L))
+
+
+@pytest.mark.parametrize("views", [False, True])
+def test_llama8b_prefill_full(views):
+    """BASELINE config 2: B=1, Hq=32, Hkv=8, S=4096, D=128, fp16, causal, 0.5*N(0,1)."""
+    q, k, v, mask = workloads.llama8b_prefill(seed=0, device=DEV, views=views)
+    out = run_prefill(q, k, v, mask)
+    assert max_err(out, torch_ref(q, k, v, mask)) <= TOL[torch.float16]
+    rows = sample_rows(4096, 150, torch.Generator().manual_seed(1))
+    want = oracle.flash_attn_rows(q, k, v, mask[:, 0, rows].cpu(), rows)
+    assert max_err(out[:, :, rows], want) <= TOL[torch.float16]
+    assert torch.equal(out[0, :, 0], v[0].repeat_interleave(4, 0)[:, 0])
+
+
+def test_long_context_prefill_full():
+    """BASELINE config 4: B=1, Hq=32, Hkv=8, S=32768, D=128, bf16, causal, 0.5*N(0,1)."""
+    L = 32768
+    q, k, v, mask = workloads.long_context_prefill(seed=0, device=DEV, L=L)
+    out = run_prefill(q, k, v, mask)
+    rows = sample_rows(L, 40, torch.Generator().manual_seed(2))
+    want = oracle.flash_attn_rows(q, k, v, mask[:, 0, rows].cpu(), rows)
+    assert max_err(out[:, :, rows], want) <= TOL[torch.bfloat16]
+    assert torch.equal(out[0, :, 0], v[0].repeat_interleave(4, 0)[:, 0])
+    assert max_err(out, torch_ref(q, k, v, mask, row_chunk=512)) <= TOL[torch.bfloat16]
+
+
+def test_decode_full():
+    """BASELINE config 3: B=64, Hq=32, Hkv=8, D=128, fp16, ctx in [512, 8192], cache [B,Hkv,8192,128]."""
+    q, kc, vc, ctx = workloads.decode_cache(seed=0, device=DEV)
+    # rows beyond ctx are garbage that must not reach the result
+    for b in range(0, 64, 7):
+        kc[b, :, int(ctx[b]):] = float("nan")
+        vc[b, :, int(ctx[b]):] = float("inf")
+    out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)
+    assert capi.flash_attn_decode(q, kc, vc, ctx, out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    want = oracle.flash_attn_decode(q, kc, vc, ctx)
+    assert max_err(out, want) <= TOL[torch.float16]
+
+
+def test_ragged_prefill_full():
+    """BASELINE config 5: 16 sequences, lengths in [128, 2048], Hq=64, Hkv=8, D=128, fp16, N(0,1)."""
+    q, k, v, cu = workloads.ragged_prefill(seed=0, device=DEV)
+    lens = (cu[1:] - cu[:-1]).tolist()
+    out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)
+    assert capi.flash_attn_varlen(q, k, v, cu, max(lens), out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert not torch.isnan(out).any()
+    worst, lo = 0.0, 0
+    for n in lens:
+        m = workloads.causal_mask(1, n, device=DEV)
+        worst = max(worst, max_err(out[:, :, lo:lo + n], torch_ref(q[:, :, lo:lo + n], k[:, :, lo:lo + n], v[:, :, lo:lo + n], m)))
+        lo += n
+    assert worst <= TOL[torch.float16]
+    # the shortest sequence in full against the oracle
+    s = int(np.argmin(lens))
+    lo, hi = int(cu[s]), int(cu[s + 1])
+    want = oracle.flash_attn(q[:, :, lo:hi], k[:, :, lo:hi], v[:, :, lo:hi], workloads.causal_mask(1, hi - lo))
+    assert max_err(out[:, :, lo:hi], want) <= TOL[torch.float16]
+
+
+# ------------------------------------------------------------------------------------------------
+# decode and varlen edge cases against the oracle
+# ------------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("B,Hq,Hkv,Lmax,D,lo,hi", [
+    (2, 8, 2, 256, 128, 1, 256),
+    (5, 8, 2, 1000, 64, 0, 1000),      # ctx = 0 allowed, Lmax not a multiple of 16
+    (2, 40, 2, 700, 128, 500, 700),    # n_rep = 20: two head groups
+    (3, 6, 6, 1537, 128, 1537, 1537),  # ctx = Lmax, n_rep = 1, 4 chunks with a 1-row tail
+    (4, 4, 1, 17, 64, 1, 17),
+])
+def test_decode_matches_oracle(dtype, B, Hq, Hkv, Lmax, D, lo, hi):
+    scale = 1.0 if dtype == torch.float16 else 0.5
+    q, kc, vc, ctx = workloads.decode_cache(seed=Lmax, device="cpu", B=B, Hq=Hq, Hkv=Hkv, Lmax=Lmax, D=D, dtype=dtype,
+                                            ctx_lo=lo, ctx_hi=hi)
+    vc = (vc.float() * scale).to(dtype)
+    out = torch.full(q.shape, float("nan"), dtype=dtype, device=DEV)
+    assert capi.flash_attn_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), ctx.to(DEV), out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert max_err(out, oracle.flash_attn_decode(q, kc, vc, ctx)) <= TOL[dtype]
+    assert torch.all(out[ctx.to(DEV) == 0] == 0)
+
+
+def test_decode_equals_last_prefill_row():
+    """Splitting the KV range and merging by log-sum-exp must not change the result: the decode of
+    position ctx-1 equals the last row of a causal prefill over the same ctx rows."""
+    B, Hq, Hkv, Lmax, D = 1, 8, 2, 2048, 128
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, Lmax, D, torch.float16, seed=21, device=DEV)
+    pre = run_prefill(q, k, v, workloads.causal_mask(B, Lmax, device=DEV))
+    for ctx_len in (1, 511, 512, 513, 2048):
+        out = torch.empty(B, Hq, 1, D, dtype=torch.float16, device=DEV)
+        ctx = torch.tensor([ctx_len], dtype=torch.int32, device=DEV)
+        assert capi.flash_attn_decode(q[:, :, ctx_len - 1:ctx_len].contiguous(), k, v, ctx, out) == capi.OK
+        assert max_err(out[:, :, 0], pre[:, :, ctx_len - 1]) <= 1e-3
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("Hq,Hkv,D,lens", [
+    (8, 2, 128, [5, 64, 100, 1, 257]),
+    (8, 1, 64, [130, 31, 0, 77]),
+    (6, 2, 128, [1, 1, 1]),
+    (4, 4, 64, [300]),
+])
+def test_varlen_matches_oracle_and_dense(dtype, Hq, Hkv, D, lens):
+    g = torch.Generator().manual_seed(sum(lens))
+    T = sum(lens)
+    q = torch.randn(1, Hq, T, D, generator=g).to(dtype)
+    k = torch.randn(1, Hkv, T, D, generator=g).to(dtype)
+    v = (0.5 * torch.randn(1, Hkv, T, D, generator=g)).to(dtype)
+    cu = torch.tensor(np.concatenate([[0], np.cumsum(lens)]), dtype=torch.int32)
+    out = torch.full(q.shape, float("nan"), dtype=dtype, device=DEV)
+    assert capi.flash_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), max(lens), out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert max_err(out, oracle.flash_attn_varlen(q, k, v, cu)) <= TOL[dtype]
+    # same result as the reference-signature op under the block-diagonal causal mask
+    blk = torch.zeros(T, T, dtype=torch.bool)
+    for lo, hi in zip(cu[:-1].tolist(), cu[1:].tolist()):
+        blk[lo:hi, lo:hi] = torch.ones(hi - lo, hi - lo, dtype=torch.bool).tril()
+    dense = run_prefill(q.to(DEV), k.to(DEV), v.to(DEV), blk[None, None].contiguous().to(DEV))
+    assert max_err(out, dense) <= TOL[dtype] / 2
+
+
+# ------------------------------------------------------------------------------------------------
+# the registered torch ops (the reference's call path) give the same bits and the same errors
+# ------------------------------------------------------------------------------------------------
+def test_torch_ops_match_c_abi(kerns):
+    from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
+    qt = GGMLQuantizationType.F16
+    qb, qs = GGML_QUANT_SIZES[qt]
+    B, Hq, Hkv, L, D = 2, 12, 2, 300, 128
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, torch.float16, seed=31, views=True, device=DEV)
+    mask = workloads.window_mask(B, L, 100, device=DEV)
+    a = torch.zeros(B, Hq, L, D, dtype=torch.float16, device=DEV)
+    kerns.flash_attn(qt, qb, qs, q, k, v, mask, a)           # reference call shape: test/kernels.py:246-248
+    torch.cuda.synchronize()
+    assert torch.equal(a, run_prefill(q, k, v, mask))
+
+    qd, kc, vc, ctx = workloads.decode_cache(seed=3, device=DEV, B=4, Lmax=1024, ctx_lo=1, ctx_hi=1024)
+    a = torch.zeros_like(qd)
+    kerns.flash_attn_decode(qt, qb, qs, qd, kc, vc, ctx, a)
+    b = torch.zeros_like(qd)
+    assert capi.flash_attn_decode(qd, kc, vc, ctx, b) == capi.OK
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+    qv, kv, vv, cu = workloads.ragged_prefill(seed=3, device=DEV, n_seqs=4, len_lo=1, len_hi=200, Hq=8, Hkv=2)
+    a = torch.zeros_like(qv)
+    kerns.flash_attn_varlen(qt, qb, qs, qv, kv, vv, cu, 200, a)
+    b = torch.zeros_like(qv)
+    assert capi.flash_attn_varlen(qv, kv, vv, cu, 200, b) == capi.OK
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+
+
+def test_torch_op_validation(kerns):
+    """The checks of the reference host function (flash_attn/op.cuh:32-96) raise RuntimeError."""
+    B, Hq, Hkv, L, D = 1, 4, 2, 64, 128
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, torch.float16, seed=1, device=DEV)
+    mask = workloads.causal_mask(B, L, device=DEV)
+    out = torch.empty_like(q)
+    args = lambda **kw: [1, 1, 2] + [kw.get(n, d) for n, d in (("q", q), ("k", k), ("v", v), ("mask", mask), ("out", out))]
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(q=q.float()))                                   # dtype
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(mask=mask.to(torch.uint8)))                     # mask dtype
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(mask=mask.expand(B, 1, L, L).transpose(2, 3)))  # mask not contiguous
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(q=q[..., ::2].repeat_interleave(2, -1)[..., ::1].transpose(2, 3).transpose(2, 3)[:, :, :, :64]))  # head_dim 64 vs k 128
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(k=k[:, :, :32]))                                # Lk != Lq
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(out=out[0]))                                    # rank
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(v=v.transpose(1, 2).contiguous().transpose(1, 2)))  # k/v strides differ
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(*args(mask=mask.cpu()))                               # device
+    kerns.flash_attn(*args())                                                  # and the good call passes
+    torch.cuda.synchronize()

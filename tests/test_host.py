@@ -1,0 +1,120 @@
+"""CPU-only checks of the boundary: the C-ABI library loads and exports what the header declares,
+argument validation rejects bad calls before anything is launched, and the Python surface keeps
+the reference's names (reference: src/minfer/kernels/__init__.py, torch_ext/ops.py:234-266)."""
+import ctypes
+import inspect
+import re
+
+import pytest
+import torch
+
+import capi
+
+
+def declared_functions():
+    text = open(capi.HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(minfer_[a-z_]+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol():
+    names = declared_functions()
+    assert {"minfer_flash_attn", "minfer_flash_attn_decode", "minfer_flash_attn_varlen",
+            "minfer_flash_attn_workspace_bytes", "minfer_flash_attn_decode_workspace_bytes",
+            "minfer_attn_last_error", "minfer_attn_version"} <= set(names)
+    L = capi.lib()
+    for n in names:
+        assert hasattr(L, n), n
+    assert L.minfer_attn_version() >= 1000
+
+
+def test_workspace_sizes():
+    L = capi.lib()
+    # one class byte per 64x64 mask tile
+    assert L.minfer_flash_attn_workspace_bytes(1, 4096) >= 64 * 64
+    assert L.minfer_flash_attn_workspace_bytes(2, 100) >= 2 * 2 * 2
+    assert L.minfer_flash_attn_workspace_bytes(1, 32768) >= 512 * 512
+    # fp32 partial (D values + max + sum) per (sequence, head, 512-row chunk)
+    assert L.minfer_flash_attn_decode_workspace_bytes(64, 32, 8192, 128) >= 64 * 32 * 16 * 130 * 4
+
+
+def _call_prefill(dtype=capi.F16, q=0x1000, k=0x2000, v=0x3000, mask=0x4000, out=0x5000, B=1, Hq=8, Hkv=2,
+                  L=64, D=128, st=None, ws=0x6000, ws_bytes=1 << 20):
+    st = st or capi.Strides(Hq * L * D, L * D, D, Hkv * L * D, L * D, D, Hq * L * D, L * D, D)
+    return capi.lib().minfer_flash_attn(dtype, q, k, v, mask, out, B, Hq, Hkv, L, D, ctypes.byref(st), ws, ws_bytes, None)
+
+
+def test_validation_rejects_before_launch():
+    """Every case must be refused on the host: the pointers are fake, so a launch would fault."""
+    assert _call_prefill(dtype=7) == capi.EINVAL and "dtype" in capi.last_error()
+    assert _call_prefill(D=96) == capi.EINVAL and "head_dim" in capi.last_error()
+    assert _call_prefill(Hq=6, Hkv=4) == capi.EINVAL
+    assert _call_prefill(q=0) == capi.EINVAL
+    assert _call_prefill(k=0x2004) == capi.EINVAL and "aligned" in capi.last_error()
+    assert _call_prefill(st=capi.Strides(1, 1, 130, 1, 1, 128, 1, 1, 128)) == capi.EINVAL and "strides" in capi.last_error()
+    assert _call_prefill(mask=0) == capi.EINVAL
+    assert _call_prefill(ws=0) == capi.EWORKSPACE
+    assert _call_prefill(ws_bytes=0) == capi.EWORKSPACE and "workspace" in capi.last_error()
+    assert _call_prefill(L=1 << 20) == capi.EINVAL
+    # empty problems are accepted and launch nothing
+    assert _call_prefill(B=0) == capi.OK and capi.last_error() == ""
+    assert _call_prefill(L=0) == capi.OK
+
+    L = capi.lib()
+    st = capi.Strides(1024, 128, 128, 1024, 128, 128, 1024, 128, 128)
+    assert L.minfer_flash_attn_decode(capi.F16, 0x1000, 0x2000, 0x3000, None, 0x5000, 1, 8, 2, 64, 128,
+                                      ctypes.byref(st), 0x6000, 1 << 20, None) == capi.EINVAL
+    assert L.minfer_flash_attn_decode(capi.F16, 0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 1, 8, 2, 64, 128,
+                                      ctypes.byref(st), 0x6000, 16, None) == capi.EWORKSPACE
+    assert L.minfer_flash_attn_decode(capi.F16, 0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 0, 8, 2, 64, 128,
+                                      ctypes.byref(st), 0x6000, 1 << 20, None) == capi.OK
+    assert L.minfer_flash_attn_varlen(capi.BF16, 0x1000, 0x2000, 0x3000, None, 2, 64, 0x5000, 8, 2, 64, 128,
+                                      ctypes.byref(st), None) == capi.EINVAL
+    assert L.minfer_flash_attn_varlen(capi.BF16, 0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 0x5000, 8, 2, 64, 128,
+                                      ctypes.byref(st), None) == capi.OK
+
+
+def test_python_surface_matches_reference_names(kerns):
+    from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
+    from minfer.kernels import KernelBackend, refs
+    import minfer.kernels.torch_ext as te
+
+    assert GGMLQuantizationType.F16 == 1 and GGML_QUANT_SIZES[GGMLQuantizationType.F16] == (1, 2)
+    assert list(inspect.signature(te.flash_attn).parameters) == [
+        "qtype_int", "qblock_size", "qtype_size", "q", "k", "v", "mask", "out"]
+    assert callable(kerns.flash_attn) and callable(kerns.flash_attn_decode) and callable(kerns.flash_attn_varlen)
+    with pytest.raises(ValueError):
+        KernelBackend("triton")
+    schema = str(torch.ops.minfer.flash_attn.default._schema)
+    assert schema == ("minfer::flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, "
+                      "Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()")
+    q = torch.randn(1, 2, 4, 8)
+    m = torch.ones(1, 1, 4, 4, dtype=torch.bool).tril()
+    assert torch.equal(refs.flash_attn(q, q, q, m), torch.nn.functional.scaled_dot_product_attention(q, q, q, attn_mask=m))
+
+
+def test_no_cpu_fallback(kerns):
+    """CPU tensors must fail loudly: there is no CPU implementation behind the ops."""
+    q = torch.zeros(1, 2, 64, 128, dtype=torch.float16)
+    mask = torch.ones(1, 1, 64, 64, dtype=torch.bool)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.flash_attn(1, 1, 2, q, q, q, mask, torch.empty_like(q))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.flash_attn_decode(1, 1, 2, q[:, :, :1], q, q, torch.ones(1, dtype=torch.int32), torch.empty_like(q[:, :, :1]))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.flash_attn_varlen(1, 1, 2, q, q, q, torch.tensor([0, 64], dtype=torch.int32), 64, torch.empty_like(q))
+
+
+def test_workload_generators_are_seeded():
+    import workloads
+    a = workloads.llama8b_prefill(seed=3, L=128)
+    b = workloads.llama8b_prefill(seed=3, L=128)
+    c = workloads.llama8b_prefill(seed=4, L=128)
+    assert all(torch.equal(x, y) for x, y in zip(a, b)) and not torch.equal(a[0], c[0])
+    qv = workloads.llama8b_prefill(seed=3, L=128, views=True)[0]
+    assert qv.shape == (1, 32, 128, 128) and qv.stride() == (128 * 32 * 128, 128, 32 * 128, 1)
+    q, k, v, cu = workloads.ragged_prefill(seed=0)
+    lens = (cu[1:] - cu[:-1]).tolist()
+    assert len(lens) == 16 and min(lens) >= 128 and max(lens) <= 2048 and q.shape == (1, 64, int(cu[-1]), 128)
+    assert workloads.prefill_flops(32, 128, [4096]) == 2 * 128 * 32 * 4096 * 4097
+    assert workloads.decode_bytes([10, 20], 32, 8, 128) == 30 * 4096 + 2 * 2 * 32 * 128 * 2
