@@ -1,0 +1,92 @@
+"""One un-timed call of an attention op, for an external profiler, e.g.
+
+    rocprofv3 --kernel-trace --stats --output-format csv -- python minfer-python_amd/apps/profile.py --kernel flash_attn --which minfer
+    rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_BUSY_CYCLES -- python minfer-python_amd/apps/profile.py --kernel flash_attn --which minfer
+
+Same command-line shape as the reference's profiling script (reference: apps/profile.py:96-143);
+`--workload` chooses between the reference's own shape and the shapes the benchmarks use.
+"""
+import argparse
+import os
+import sys
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(HERE))
+sys.path.insert(0, HERE)
+
+import workloads  # noqa: E402
+from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType  # noqa: E402
+from minfer.kernels import KernelBackend, refs  # noqa: E402
+
+QT = GGMLQuantizationType.F16
+QB, QS = GGML_QUANT_SIZES[QT]
+
+
+def flash_attn(backend: str, which: str, workload: str, repeat: int):
+    kerns = KernelBackend(backend)
+    if workload == "reference":   # reference: apps/profile.py:98 (B=4, L=4096, 48 heads over 8 KV heads)
+        B, L, Hq, Hkv, D = 4, 4096, 48, 8, 128
+        q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, torch.float16, scale=1.0, views=True, device="cuda")
+        mask = workloads.causal_mask(B, L, device="cuda")
+    elif workload == "long":
+        q, k, v, mask = workloads.long_context_prefill(device="cuda")
+    else:
+        q, k, v, mask = workloads.llama8b_prefill(device="cuda")
+    out = torch.zeros(q.shape, dtype=q.dtype, device="cuda")
+    n_rep = q.shape[1] // k.shape[1]
+    if which == "minfer":
+        fn = lambda: kerns.flash_attn(QT, QB, QS, q, k, v, mask, out)
+    else:
+        k_exp, v_exp = k.repeat_interleave(n_rep, dim=1), v.repeat_interleave(n_rep, dim=1)
+        fn = lambda: refs.flash_attn(q, k_exp, v_exp, mask)
+    with torch.no_grad():
+        for _ in range(repeat):
+            fn()
+    torch.cuda.synchronize()
+
+
+def flash_attn_decode(backend: str, which: str, workload: str, repeat: int):
+    kerns = KernelBackend(backend)
+    q, kc, vc, ctx = workloads.decode_cache(device="cuda")
+    out = torch.zeros_like(q)
+    if which == "minfer":
+        fn = lambda: kerns.flash_attn_decode(QT, QB, QS, q, kc, vc, ctx, out)
+    else:
+        n_rep = q.shape[1] // kc.shape[1]
+        fn = lambda: [refs.flash_attn_decode(q[b:b + 1], kc[b:b + 1].repeat_interleave(n_rep, 1),
+                                             vc[b:b + 1].repeat_interleave(n_rep, 1), ctx[b:b + 1]) for b in range(q.shape[0])]
+    with torch.no_grad():
+        for _ in range(repeat):
+            fn()
+    torch.cuda.synchronize()
+
+
+def flash_attn_varlen(backend: str, which: str, workload: str, repeat: int):
+    kerns = KernelBackend(backend)
+    q, k, v, cu = workloads.ragged_prefill(device="cuda")
+    out = torch.zeros_like(q)
+    max_len = int((cu[1:] - cu[:-1]).max())
+    if which == "minfer":
+        fn = lambda: kerns.flash_attn_varlen(QT, QB, QS, q, k, v, cu, max_len, out)
+    else:
+        n_rep = q.shape[1] // k.shape[1]
+        k_exp, v_exp = k.repeat_interleave(n_rep, dim=1), v.repeat_interleave(n_rep, dim=1)
+        fn = lambda: refs.flash_attn_varlen(q, k_exp, v_exp, cu)
+    with torch.no_grad():
+        for _ in range(repeat):
+            fn()
+    torch.cuda.synchronize()
+
+
+if __name__ == "__main__":
+    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen}
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
+    parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)
+    parser.add_argument("--which", choices=["minfer", "ref"], required=True)
+    parser.add_argument("--workload", choices=["llama8b", "reference", "long"], default="llama8b")
+    parser.add_argument("--repeat", type=int, default=1)
+    args = parser.parse_args()
+    KERNELS[args.kernel](args.backend, args.which, args.workload, args.repeat)
