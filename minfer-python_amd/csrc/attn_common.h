@@ -46,6 +46,14 @@ struct F16 {
         return __builtin_bit_cast(uint32_t, __builtin_convertvector(f, h16x2));
     }
     static MA_DEV float to_float(short bits) { return (float)__builtin_bit_cast(_Float16, bits); }
+    // x * f elementwise, computed in fp32 and rounded back (round-to-nearest-even)
+    static MA_DEV s16x8 scale8(s16x8 x, float f) {
+        const h16x8 v = __builtin_bit_cast(h16x8, x);
+        h16x8 r;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) r[i] = (_Float16)((float)v[i] * f);
+        return __builtin_bit_cast(s16x8, r);
+    }
     // acc + lo + hi of a packed pair, in fp32: sums exactly the rounded values the MFMA consumes
     static MA_DEV float add_pair(uint32_t pair, float acc) {
         const h16x2 ones = {(_Float16)1.f, (_Float16)1.f};
@@ -72,6 +80,13 @@ struct BF16 {
     static MA_DEV float to_float(short bits) {
         return __builtin_bit_cast(float, (uint32_t)(uint16_t)bits << 16);
     }
+    static MA_DEV s16x8 scale8(s16x8 x, float f) {
+        uint32_t w[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[i] = pack2(to_float(x[2 * i]) * f, to_float(x[2 * i + 1]) * f);
+        uint4 u; u.x = w[0]; u.y = w[1]; u.z = w[2]; u.w = w[3];
+        return __builtin_bit_cast(s16x8, u);
+    }
     static MA_DEV float add_pair(uint32_t pair, float acc) {
         const b16x2 ones = {(__bf16)1.f, (__bf16)1.f};
         return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(b16x2, pair), ones, acc, false);
@@ -93,6 +108,28 @@ MA_DEV void copy16_global_to_lds(const void* src, void* lds_base) {
                  : "s"(dst), "v"(src)
                  : "memory");
 }
+// Same, with the source given as a wave-uniform base plus a 32-bit unsigned per-lane byte offset, which
+// costs no vector ALU work when the offset is loop-invariant.
+MA_DEV void copy16_global_to_lds(const void* uniform_base, uint32_t lane_byte_offset, void* lds_base) {
+    const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_base);
+    const uint64_t b = (uint64_t)(uintptr_t)uniform_base;
+    // readfirstlane returns a signed int: go through uint32_t, or a low word with bit 31 set would be
+    // sign-extended into the high word of the address
+    const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32) |
+                        (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 :
+                 : "s"(dst), "v"(lane_byte_offset), "s"(sb)
+                 : "memory");
+}
+
+// 32-bit LDS address of a __shared__ object, and reads at such an address plus a compile-time offset
+// (which the instruction carries as an immediate, so one address register serves many reads).
+MA_DEV uint32_t lds_addr(const void* p) { return (uint32_t)(uintptr_t)(lds_void*)p; }
+MA_DEV s16x8 lds_read_b128(uint32_t addr, int imm) {
+    typedef __attribute__((address_space(3))) s16x8 lds_s16x8;
+    return *(const lds_s16x8*)(uintptr_t)(addr + imm);
+}
 
 // Waits until at most N of this wave's vector-memory operations (global loads and global->LDS
 // copies, which retire in order) are outstanding.  Also a compiler barrier, so LDS reads of the
@@ -108,6 +145,10 @@ template <int N> MA_DEV void wait_vmcnt() {
 MA_DEV s16x4 lds_read_tr16(const void* lds_ptr) {
     typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)lds_ptr);
+}
+MA_DEV s16x4 lds_read_tr16(uint32_t addr, int imm) {
+    typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+    return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uintptr_t)(addr + imm));
 }
 
 // Value of x held by lane (l ^ 32), combined with the lane's own by max / sum.

@@ -18,6 +18,8 @@
 // classifies every 64x64 mask tile as none / all / mixed; the main kernel skips "none" tiles,
 // runs "all" tiles unmasked and reads mask bytes only for "mixed" tiles, which keeps arbitrary
 // masks bit-exact while a causal mask costs one byte-read tile per row of tiles.
+#include <type_traits>
+
 #include "attn_common.h"
 #include "attn_host.h"
 
@@ -216,46 +218,93 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
     }
 
     // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
+    // Q is multiplied by scale*log2(e) once, here, so that the MFMA accumulator of Q K^T is directly
+    // the base-2 exponent of the softmax weight (minus the running reference it is initialised with).
+    const float c2 = p.scale_log2;
     s16x8 qf[KC];
     {
         const short* src = Qh + (int64_t)min(qrow, last_row) * p.q2 + 8 * h;
 #pragma unroll
-        for (int c = 0; c < KC; ++c) qf[c] = *reinterpret_cast<const s16x8*>(src + 16 * c);
+        for (int c = 0; c < KC; ++c) qf[c] = T::scale8(*reinterpret_cast<const s16x8*>(src + 16 * c), c2);
     }
 
     // ---- global -> LDS tile copy ----------------------------------------------------------
+    // Instruction j of this wave fills rows (j*kWaves + w)*RPI .. +RPI-1 of the tile; the lane's byte
+    // offset from the tile's first key row is a constant (row and swizzled granule), so a full tile
+    // costs no vector ALU work: scalar base + constant per-lane offset.
+    uint32_t k_off[NLD], v_off[NLD];
+#pragma unroll
+    for (int j = 0; j < NLD; ++j) {
+        const int row = (j * kWaves + w) * RPI + lane / G, pg = lane % G;
+        k_off[j] = (uint32_t)((int64_t)row * p.kv2 + 8 * (pg ^ GEO::swz_k(row))) * 2u;
+        v_off[j] = (uint32_t)((int64_t)row * p.kv2 + 8 * (pg ^ GEO::swz_v(row))) * 2u;
+    }
     auto issue_tile = [&](int kt, int stage) {
         const int key0 = kt * 64;
+        const short* kbase = Kh + (int64_t)key0 * p.kv2;
+        const short* vbase = Vh + (int64_t)key0 * p.kv2;
+        if (key0 + 64 <= seq_len) {
 #pragma unroll
-        for (int j = 0; j < NLD; ++j) {
-            const int row0 = (j * kWaves + w) * RPI;     // wave-uniform first row of this instruction
-            const int row = row0 + lane / G;
-            const int pg = lane % G;                      // physical granule this lane fills
-            const int64_t grow = (int64_t)min(key0 + row, last_row) * p.kv2;
-            copy16_global_to_lds(Kh + grow + 8 * (pg ^ GEO::swz_k(row)), &k_lds[stage][row0 * RB]);
-            copy16_global_to_lds(Vh + grow + 8 * (pg ^ GEO::swz_v(row)), &v_lds[stage][row0 * RB]);
+            for (int j = 0; j < NLD; ++j) {
+                const int row0 = (j * kWaves + w) * RPI;
+                copy16_global_to_lds(kbase, k_off[j], &k_lds[stage][row0 * RB]);
+                copy16_global_to_lds(vbase, v_off[j], &v_lds[stage][row0 * RB]);
+            }
+        } else {   // tile crossing the end of the sequence: rows past it re-read the last row
+#pragma unroll
+            for (int j = 0; j < NLD; ++j) {
+                const int row0 = (j * kWaves + w) * RPI;
+                const int row = row0 + lane / G, pg = lane % G;
+                const int64_t grow = (int64_t)(min(key0 + row, last_row) - key0) * p.kv2;
+                copy16_global_to_lds(kbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_k(row))) * 2u, &k_lds[stage][row0 * RB]);
+                copy16_global_to_lds(vbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_v(row))) * 2u, &v_lds[stage][row0 * RB]);
+            }
         }
     };
+
+    // ---- per-lane LDS read addresses (stage 0; the other stage and the row blocks are immediates) ----
+    // K fragment c of key block kb: row 32kb + l32, granule (2c+h) ^ swz_k(row); swz_k is the same for
+    // rows l32 and 32 + l32.  V^T fragment (chunk c, half, db): row 16c + 8half + 4h + li/4, columns
+    // 32db + 16(blk&1) + 4(li&3); swz_v depends on li only.
+    const int blk = lane >> 4, li = lane & 15;
+    uint32_t k_rd[KC], v_rd[DB];
+    {
+        const int sw = GEO::swz_k(l32);
+#pragma unroll
+        for (int c = 0; c < KC; ++c) k_rd[c] = lds_addr(&k_lds[0][0]) + l32 * RB + 16 * ((2 * c + h) ^ sw);
+        const int vrow = 4 * h + (li >> 2);
+        const int swv = GEO::swz_v(vrow);
+#pragma unroll
+        for (int db = 0; db < DB; ++db) {
+            const int dcol = 32 * db + 16 * (blk & 1) + 4 * (li & 3);
+            v_rd[db] = lds_addr(&v_lds[0][0]) + vrow * RB + 16 * ((dcol >> 3) ^ swv) + 2 * (dcol & 7);
+        }
+    }
 
     f32x16 o_acc[DB];
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
         for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.f;
-    float m_ref = -INFINITY;   // reference maximum (raw score units) of the lane's query row
-    float l_sum = 0.f;         // this lane's share of the softmax denominator
-    const float c2 = p.scale_log2;
-    constexpr float kLazyLog2 = 6.f;  // re-reference only when the row maximum grows by > 2^6
+    // Reference exponent of the lane's query row (log2 units; -inf until a key has been seen) and the
+    // lane's share of the softmax denominator.  The reference moves only when a tile's largest exponent
+    // exceeds it by more than kLazyLog2, so most tiles rescale nothing and weights stay below 2^kLazyLog2.
+    float m_ref = -INFINITY, l_sum = 0.f;
+    constexpr float kLazyLog2 = 8.f;
 
-    auto tile_of = [&](int it, int& kt, uint32_t& cls_w) {
+    auto tile_of = [&](uint32_t e, int it, int& kt, uint32_t& cls_w) {
         if (MODE == MODE_DENSE) {
-            const uint32_t e = tile_list[it];
             kt = (int)(e & 0xffffu);
             cls_w = (e >> (16 + 2 * my_qt64_slot)) & 3u;
         } else {
             kt = it;
             cls_w = (64 * kt + 63 <= q_row0) ? TILE_ALL : ((64 * kt > q_row0 + 31) ? TILE_NONE : TILE_MIXED);
         }
+        if (!wave_on) cls_w = TILE_NONE;
+    };
+    auto list_entry = [&](int it) -> uint32_t {   // wave-uniform
+        if (MODE != MODE_DENSE || n_active <= 0) return 0u;
+        return __builtin_amdgcn_readfirstlane(tile_list[min(it, n_active - 1)]);
     };
     // mask words of a MIXED dense tile: word [kb][j] covers keys key0 + 32kb + 8j + 4h + 0..3
     uint32_t mw[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
@@ -281,54 +330,47 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
         }
     };
 
-    if (n_active > 0) {
-        int kt0; uint32_t c0;
-        tile_of(0, kt0, c0);
-        issue_tile(kt0, 0);
-        if (MODE == MODE_DENSE && wave_on && c0 == TILE_MIXED) fetch_mask(kt0);
-    }
-
-    for (int it = 0; it < n_active; ++it) {
-        const int stage = it & 1;
-        int kt; uint32_t cls_w;
-        tile_of(it, kt, cls_w);
-        wait_vmcnt<0>();                     // this wave's share of tile `it` (and its mask words) has landed
-        __syncthreads();                     // everyone's share has; stage^1 is no longer being read
-        uint32_t mcur[2][4];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) mcur[kb][j] = mw[kb][j];
-        if (it + 1 < n_active) {
-            int ktn; uint32_t cn;
-            tile_of(it + 1, ktn, cn);
-            issue_tile(ktn, stage ^ 1);
-            if (MODE == MODE_DENSE && wave_on && cn == TILE_MIXED) fetch_mask(ktn);
-        }
-        if (!wave_on || cls_w == TILE_NONE) continue;
-
+    // ---- one key tile, K/V in LDS stage STAGE (compile-time, so every LDS address is base + immediate) ----
+    auto process_tile = [&](auto stage_tag, int kt, uint32_t cls_w) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        constexpr int SOFF = STAGE * GEO::TILE_BYTES;
         const int key0 = kt * 64;
-        // ---- S^T = K Q^T ------------------------------------------------------------------
-        f32x16 s_acc[2];
+
+        // S^T = K Q^T, accumulated on top of -reference: register r of block kb is key 32kb + 8(r/4) + 4h + r%4.
+        // All K fragments are requested before the first MFMA: the LDS latency is paid once per tile.
+        s16x8 ka[KC], kb_[KC];
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            ka[c] = lds_read_b128(k_rd[c], SOFF);
+            kb_[c] = lds_read_b128(k_rd[c], SOFF + 32 * RB);
+        }
+        const float init = (m_ref == -INFINITY) ? 0.f : -m_ref;
+        f32x16 e_acc[2];
 #pragma unroll
         for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) s_acc[kb][r] = 0.f;
-        {
-            const char* rowp0 = &k_lds[stage][l32 * RB];
-            const char* rowp1 = rowp0 + 32 * RB;
-            const int sw0 = GEO::swz_k(l32), sw1 = GEO::swz_k(32 + l32);
+            for (int r = 0; r < 16; ++r) e_acc[kb][r] = init;
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int c = 0; c < KC; ++c) {
-                const s16x8 a0 = *reinterpret_cast<const s16x8*>(rowp0 + 16 * ((2 * c + h) ^ sw0));
-                const s16x8 a1 = *reinterpret_cast<const s16x8*>(rowp1 + 16 * ((2 * c + h) ^ sw1));
-                s_acc[0] = T::mfma32(a0, qf[c], s_acc[0]);
-                s_acc[1] = T::mfma32(a1, qf[c], s_acc[1]);
-            }
+        for (int c = 0; c < KC; ++c) {
+            e_acc[0] = T::mfma32(ka[c], qf[c], e_acc[0]);
+            e_acc[1] = T::mfma32(kb_[c], qf[c], e_acc[1]);
         }
+        // first two chunks of V^T fragments: their latency hides behind the max and the first exponentials
+        s16x8 va[2][DB];
+        auto load_v = [&](int c, s16x8 (&a)[DB]) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (16 * c) * RB);
+                const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (16 * c + 8) * RB);
+                a[db] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+            }
+        };
+        load_v(0, va[0]);
+        load_v(1, va[1]);
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- masking ----------------------------------------------------------------------
-        // register r of block kb is key key0 + 32kb + 8(r/4) + 4h + r%4
         if (cls_w == TILE_MIXED || key0 + 64 > seq_len) {
             const bool use_bytes = MODE == MODE_DENSE && cls_w == TILE_MIXED;
 #pragma unroll
@@ -339,72 +381,102 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         bool keep = kbase + e < seq_len;
-                        if (MODE == MODE_DENSE) keep = keep && (!use_bytes || ((mcur[kb][j] >> (8 * e)) & 0xffu) != 0u);
+                        if (MODE == MODE_DENSE) keep = keep && (!use_bytes || ((mw[kb][j] >> (8 * e)) & 0xffu) != 0u);
                         else keep = keep && (kbase + e <= qrow);
-                        s_acc[kb][4 * j + e] = keep ? s_acc[kb][4 * j + e] : -INFINITY;
+                        e_acc[kb][4 * j + e] = keep ? e_acc[kb][4 * j + e] : -INFINITY;
                     }
                 }
             }
         }
-
-        // ---- online softmax ----------------------------------------------------------------
-        uint32_t pf[4][4];  // P^T fragments (B operand): [16-key chunk][4 x packed pair]
+        // ---- reference update (rare after the first tiles) --------------------------------------
         {
-            float mx = s_acc[0][0];
+            float mx = e_acc[0][0];
 #pragma unroll
             for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, s_acc[kb][r]);
-            mx = max_across_halves(mx);
-            const bool grow = (mx - m_ref) * c2 > kLazyLog2 || (m_ref == -INFINITY && mx > -INFINITY);
-            if (__any(grow)) {  // wave-uniform: most tiles leave every row's reference unchanged
-                const float m_new = grow ? mx : m_ref;
-                const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2((m_ref - m_new) * c2);
-                m_ref = m_new;
+                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, e_acc[kb][r]);
+            mx = max_across_halves(mx);   // largest exponent of the row in this tile, relative to the reference
+            const bool grow = mx > kLazyLog2 || (m_ref == -INFINITY && mx > -INFINITY);
+            if (__any(grow)) {  // wave-uniform branch
+                const float delta = grow ? mx : 0.f;
+                const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2(-delta);
+                m_ref = grow ? ((m_ref == -INFINITY) ? mx : m_ref + mx) : m_ref;
                 l_sum *= alpha;
+#pragma unroll
+                for (int kb = 0; kb < 2; ++kb)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) e_acc[kb][r] -= delta;
 #pragma unroll
                 for (int db = 0; db < DB; ++db)
 #pragma unroll
                     for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
             }
-            const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * c2;
-            float ls = 0.f;
-#pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
-#pragma unroll
-                for (int r = 0; r < 16; r += 2) {
-                    const float p0 = fast_exp2(fmaf(s_acc[kb][r], c2, -mc));
-                    const float p1 = fast_exp2(fmaf(s_acc[kb][r + 1], c2, -mc));
-                    const uint32_t pk = T::pack2(p0, p1);
-                    ls = T::add_pair(pk, ls);   // the denominator sums the rounded weights the MFMA uses
-                    pf[2 * kb + (r >> 3)][(r & 7) >> 1] = pk;
-                }
-            }
-            l_sum += ls;
         }
-
-        // ---- O^T += V^T P^T ----------------------------------------------------------------
-        // chunk c contracts keys 16c..16c+15 in the order 16c + 8(i/4) + 4h + i%4 (i = element of the
-        // lane's 8-wide k slice), which is the order the score registers already have.
-        const int blk = lane >> 4, li = lane & 15;
+        // ---- P = 2^E and O^T += V^T P^T, one 16-key chunk at a time -------------------------------
+        // Chunk c contracts keys 16c..16c+15 in the order 16c + 8(i/4) + 4h + i%4 (i = element of the
+        // lane's 8-wide k slice), which is the order the exponent registers already have.  The weights of
+        // chunk c+1 are computed between the MFMAs of chunk c (one MFMA, a few vector instructions, ...),
+        // which is what lets the matrix pipe and the vector ALU of this SIMD run at the same time.
+        float ls = 0.f;
+        auto weights = [&](int c) -> s16x8 {
+            uint32_t pk[4];
+#pragma unroll
+            for (int i = 0; i < 8; i += 2) {
+                const int kb = c >> 1, r = 8 * (c & 1) + i;
+                pk[i >> 1] = T::pack2(fast_exp2(e_acc[kb][r]), fast_exp2(e_acc[kb][r + 1]));
+                ls = T::add_pair(pk[i >> 1], ls);   // the denominator sums the rounded weights the MFMA uses
+            }
+            uint4 pu; pu.x = pk[0]; pu.y = pk[1]; pu.z = pk[2]; pu.w = pk[3];
+            return __builtin_bit_cast(s16x8, pu);
+        };
+        s16x8 pcur = weights(0);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
-            uint4 pu; pu.x = pf[c][0]; pu.y = pf[c][1]; pu.z = pf[c][2]; pu.w = pf[c][3];
-            const s16x8 bfrag = __builtin_bit_cast(s16x8, pu);
+            s16x8 pnext = pcur;
+            if (c + 1 < 4) pnext = weights(c + 1);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                s16x8 a;
+            for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma32(va[c & 1][db], pcur, o_acc[db]);
+            if (c + 1 < 4) {
+                // interleave: 1 MFMA, then a quarter of the next chunk's vector work
 #pragma unroll
-                for (int half = 0; half < 2; ++half) {
-                    const int row = 16 * c + 8 * half + 4 * h + (li >> 2);
-                    const int dcol = 32 * db + 16 * (blk & 1) + 4 * (li & 3);
-                    const char* ptr = &v_lds[stage][row * RB + 16 * ((dcol >> 3) ^ GEO::swz_v(row)) + 2 * (dcol & 7)];
-                    const s16x4 t = lds_read_tr16(ptr);
-                    a[4 * half + 0] = t[0]; a[4 * half + 1] = t[1]; a[4 * half + 2] = t[2]; a[4 * half + 3] = t[3];
+                for (int i = 0; i < DB; ++i) {
+                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                    __builtin_amdgcn_sched_group_barrier(0x002, 24 / DB, 0);
                 }
-                o_acc[db] = T::mfma32(a, bfrag, o_acc[db]);
             }
+            __builtin_amdgcn_sched_barrier(0);
+            if (c + 2 < 4) load_v(c + 2, va[c & 1]);
+            pcur = pnext;
         }
+        l_sum += ls;
+    };
+
+    // ---- main loop: one barrier per tile; the copy of tile t+1 is issued right after the barrier that
+    // opens tile t, into the stage tile t-1 has just vacated ---------------------------------------
+    uint32_t e_cur = list_entry(0), e_next = list_entry(1);
+    if (n_active > 0) {
+        int kt0; uint32_t c0;
+        tile_of(e_cur, 0, kt0, c0);
+        issue_tile(kt0, 0);
+        if (MODE == MODE_DENSE && c0 == TILE_MIXED) fetch_mask(kt0);
+    }
+    auto iteration = [&](auto stage_tag, int it) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        int kt, ktn; uint32_t cls_w, cn;
+        tile_of(e_cur, it, kt, cls_w);
+        tile_of(e_next, it + 1, ktn, cn);
+        const uint32_t e_after = list_entry(it + 2);   // read early, used next iteration
+        wait_vmcnt<0>();       // this wave's share of tile `it` (and its mask words) has landed
+        __syncthreads();       // everyone's has; stage STAGE^1 is no longer being read
+        if (it + 1 < n_active) issue_tile(ktn, STAGE ^ 1);
+        if (cls_w != TILE_NONE) process_tile(stage_tag, kt, cls_w);
+        if (MODE == MODE_DENSE && it + 1 < n_active && cn == TILE_MIXED) fetch_mask(ktn);   // after this tile's words were used
+        e_cur = e_next; e_next = e_after;
+    };
+    for (int it = 0; it < n_active; it += 2) {
+        iteration(std::integral_constant<int, 0>{}, it);
+        if (it + 1 < n_active) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
 
     // ---- epilogue: normalise and store -----------------------------------------------------
