@@ -44,12 +44,18 @@ __global__ __launch_bounds__(256) void classify_mask_kernel(const uint8_t* __res
     uint32_t any_acc = 0u, all_acc = 0x01010101u;
     if (vec) {
         if (col0 < L) {
-            for (int r = w; r < 64; r += 4) {
-                const int row = qt * 64 + r;
-                if (row >= L) break;
-                const uint4 x = *reinterpret_cast<const uint4*>(mb + (size_t)row * L + col0);
-                any_acc |= x.x | x.y | x.z | x.w;
-                all_acc &= x.x & x.y & x.z & x.w;
+            // all 16 row segments of this lane are requested before any is used (rows past the end
+            // re-read the last row, which changes neither the OR nor the AND)
+            uint4 x[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                const int row = min(qt * 64 + w + 4 * i, L - 1);
+                x[i] = *reinterpret_cast<const uint4*>(mb + (size_t)row * L + col0);
+            }
+#pragma unroll
+            for (int i = 0; i < 16; ++i) {
+                any_acc |= x[i].x | x[i].y | x[i].z | x[i].w;
+                all_acc &= x[i].x & x[i].y & x[i].z & x[i].w;
             }
         }
     } else {
@@ -104,7 +110,10 @@ struct PrefillParams {
 };
 
 enum { MODE_DENSE = 0, MODE_VARLEN = 1 };
-constexpr int kWaves = 8;            // waves per workgroup (two per SIMD)
+#ifndef MINFER_PREFILL_WAVES
+#define MINFER_PREFILL_WAVES 8
+#endif
+constexpr int kWaves = MINFER_PREFILL_WAVES;   // waves per workgroup
 constexpr int kThreads = kWaves * 64;
 
 template <int D> struct TileGeom {
@@ -122,7 +131,7 @@ template <int D> struct TileGeom {
 };
 
 template <class T, int D, int MODE>
-__global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p) {
+__global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParams p) {
     using GEO = TileGeom<D>;
     constexpr int RB = GEO::RB, G = GEO::G, RPI = GEO::RPI, NLD = GEO::NLD;
     constexpr int KC = D / 16;   // 16-wide contraction chunks of Q K^T
@@ -291,6 +300,9 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
     // exceeds it by more than kLazyLog2, so most tiles rescale nothing and weights stay below 2^kLazyLog2.
     float m_ref = -INFINITY, l_sum = 0.f;
     constexpr float kLazyLog2 = 8.f;
+    f32x16 neg_ref;   // -m_ref in every register (0 while there is no reference): the MFMA C operand of Q K^T
+#pragma unroll
+    for (int r = 0; r < 16; ++r) neg_ref[r] = 0.f;
 
     auto tile_of = [&](uint32_t e, int it, int& kt, uint32_t& cls_w) {
         if (MODE == MODE_DENSE) {
@@ -341,28 +353,43 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
         s16x8 ka[KC], kb_[KC];
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
+#ifdef ABL_NOLDSREAD
+            ka[c] = qf[c]; kb_[c] = qf[(c + 1) % KC];
+#else
             ka[c] = lds_read_b128(k_rd[c], SOFF);
             kb_[c] = lds_read_b128(k_rd[c], SOFF + 32 * RB);
+#endif
         }
-        const float init = (m_ref == -INFINITY) ? 0.f : -m_ref;
-        f32x16 e_acc[2];
-#pragma unroll
-        for (int kb = 0; kb < 2; ++kb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) e_acc[kb][r] = init;
         __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-        for (int c = 0; c < KC; ++c) {
+        // the accumulators start from -reference (neg_ref, a register block that changes only when the
+        // reference does), so the MFMA output is the exponent relative to the reference
+        f32x16 e_acc[2];
+#ifdef ABL_NOQK
+        e_acc[0] = neg_ref; e_acc[1] = neg_ref;
+        for (int c = 0; c < 1; ++c) {
             e_acc[0] = T::mfma32(ka[c], qf[c], e_acc[0]);
             e_acc[1] = T::mfma32(kb_[c], qf[c], e_acc[1]);
         }
+#else
+        e_acc[0] = T::mfma32(ka[0], qf[0], neg_ref);
+        e_acc[1] = T::mfma32(kb_[0], qf[0], neg_ref);
+#pragma unroll
+        for (int c = 1; c < KC; ++c) {
+            e_acc[0] = T::mfma32(ka[c], qf[c], e_acc[0]);
+            e_acc[1] = T::mfma32(kb_[c], qf[c], e_acc[1]);
+        }
+#endif
         // first two chunks of V^T fragments: their latency hides behind the max and the first exponentials
         s16x8 va[2][DB];
         auto load_v = [&](int c, s16x8 (&a)[DB]) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
+#ifdef ABL_NOLDSREAD
+                const s16x4 t0 = {qf[db][0], qf[c][1], qf[db][2], qf[c][3]}, t1 = {qf[db][4], qf[c][5], qf[db][6], qf[c][7]};
+#else
                 const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (16 * c) * RB);
                 const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (16 * c + 8) * RB);
+#endif
                 a[db] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
             }
         };
@@ -401,6 +428,9 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
                 const float delta = grow ? mx : 0.f;
                 const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2(-delta);
                 m_ref = grow ? ((m_ref == -INFINITY) ? mx : m_ref + mx) : m_ref;
+                const float nr = (m_ref == -INFINITY) ? 0.f : -m_ref;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) neg_ref[r] = nr;
                 l_sum *= alpha;
 #pragma unroll
                 for (int kb = 0; kb < 2; ++kb)
@@ -423,7 +453,11 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
 #pragma unroll
             for (int i = 0; i < 8; i += 2) {
                 const int kb = c >> 1, r = 8 * (c & 1) + i;
+#ifdef ABL_NOEXP
+                pk[i >> 1] = T::pack2(e_acc[kb][r], e_acc[kb][r + 1]);
+#else
                 pk[i >> 1] = T::pack2(fast_exp2(e_acc[kb][r]), fast_exp2(e_acc[kb][r + 1]));
+#endif
                 ls = T::add_pair(pk[i >> 1], ls);   // the denominator sums the rounded weights the MFMA uses
             }
             uint4 pu; pu.x = pk[0]; pu.y = pk[1]; pu.z = pk[2]; pu.w = pk[3];
@@ -435,8 +469,12 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
         for (int c = 0; c < 4; ++c) {
             s16x8 pnext = pcur;
             if (c + 1 < 4) pnext = weights(c + 1);
+#ifdef ABL_NOPV
+            for (int db = 0; db < (c == 0 ? 1 : 0); ++db) o_acc[db] = T::mfma32(va[c & 1][db], pcur, o_acc[db]);
+#else
 #pragma unroll
             for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma32(va[c & 1][db], pcur, o_acc[db]);
+#endif
             if (c + 1 < 4) {
                 // interleave: 1 MFMA, then a quarter of the next chunk's vector work
 #pragma unroll
@@ -468,8 +506,12 @@ __global__ __launch_bounds__(kThreads) void prefill_kernel(const PrefillParams p
         tile_of(e_next, it + 1, ktn, cn);
         const uint32_t e_after = list_entry(it + 2);   // read early, used next iteration
         wait_vmcnt<0>();       // this wave's share of tile `it` (and its mask words) has landed
+#ifndef ABL_NOBARRIER
         __syncthreads();       // everyone's has; stage STAGE^1 is no longer being read
+#endif
+#ifndef ABL_NODMA
         if (it + 1 < n_active) issue_tile(ktn, STAGE ^ 1);
+#endif
         if (cls_w != TILE_NONE) process_tile(stage_tag, kt, cls_w);
         if (MODE == MODE_DENSE && it + 1 < n_active && cn == TILE_MIXED) fetch_mask(ktn);   // after this tile's words were used
         e_cur = e_next; e_next = e_after;
@@ -527,7 +569,7 @@ static void fill_common(PrefillParams& p, const void* q, const void* k, const vo
     p.kv0 = st->kv0; p.kv1 = st->kv1; p.kv2 = st->kv2;
     p.o0 = st->o0; p.o1 = st->o1; p.o2 = st->o2;
     p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.n_rep = (int)(Hq / Hkv);
-    p.hpw_log2 = (p.n_rep % 8 == 0) ? 3 : (p.n_rep % 4 == 0) ? 2 : ((p.n_rep % 2 == 0) ? 1 : 0);
+    p.hpw_log2 = (p.n_rep % 8 == 0 && kWaves >= 8) ? 3 : (p.n_rep % 4 == 0) ? 2 : ((p.n_rep % 2 == 0) ? 1 : 0);
     p.n_hg = p.n_rep >> p.hpw_log2;
     p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
 }
