@@ -22,6 +22,10 @@ for p in (ROOT, PKG, os.path.join(PKG, "apps")):
 
 PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
+# HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
+# same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
+PREFILL_TRAFFIC_BYTES = 110289 * 1024
+DECODE_TRAFFIC_BYTES = 1098181 * 1024
 
 
 class HipEvents:
@@ -140,13 +144,13 @@ def main():
         "config": {"workload": "prefill B=1 Hq=32 Hkv=8 S=4096 D=128 fp16 causal dense-mask (BASELINE configs[1])",
                    "global_batch": 1, "seq_len": L, "parallelism": "single-gpu"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_MFMA_TFLOPS, "traffic": None,
+                     "frac": achieved / PEAK_MFMA_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
                      "kernel": "classify_mask_kernel + prefill_kernel<F16,128,dense>",
                      "algorithmic_flops": flops, "avg_ms": avg_ms, "median_ms": med_ms},
         "decode": {"value": d_gbs, "unit": "GB/s", "ms": d_avg_ms, "median_ms": d_med_ms,
                    "workload": "decode B=64 Hq=32 Hkv=8 D=128 fp16 ctx~U[512,8192] cache [64,8,8192,128] (BASELINE configs[2])",
                    "roofline": {"bound": "hbm", "achieved": d_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                "frac": d_gbs / PEAK_HBM_GBS, "traffic": None,
+                                "frac": d_gbs / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES,
                                 "kernel": "decode_split_kernel<F16,128> + decode_combine_kernel",
                                 "algorithmic_bytes": dbytes}},
     }

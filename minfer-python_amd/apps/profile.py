@@ -80,8 +80,19 @@ def flash_attn_varlen(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def copy(backend: str, which: str, workload: str, repeat: int):
+    """A plain device-to-device copy of 1 GiB: the known-size kernel that HBM byte counters
+    (FETCH_SIZE / WRITE_SIZE) are calibrated against."""
+    src = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").fill_(1)
+    dst = torch.empty_like(src)
+    for _ in range(repeat):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+
+
 if __name__ == "__main__":
-    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen}
+    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
+               "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)
