@@ -353,24 +353,13 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         s16x8 ka[KC], kb_[KC];
 #pragma unroll
         for (int c = 0; c < KC; ++c) {
-#ifdef ABL_NOLDSREAD
-            ka[c] = qf[c]; kb_[c] = qf[(c + 1) % KC];
-#else
             ka[c] = lds_read_b128(k_rd[c], SOFF);
             kb_[c] = lds_read_b128(k_rd[c], SOFF + 32 * RB);
-#endif
         }
         __builtin_amdgcn_sched_barrier(0);
         // the accumulators start from -reference (neg_ref, a register block that changes only when the
         // reference does), so the MFMA output is the exponent relative to the reference
         f32x16 e_acc[2];
-#ifdef ABL_NOQK
-        e_acc[0] = neg_ref; e_acc[1] = neg_ref;
-        for (int c = 0; c < 1; ++c) {
-            e_acc[0] = T::mfma32(ka[c], qf[c], e_acc[0]);
-            e_acc[1] = T::mfma32(kb_[c], qf[c], e_acc[1]);
-        }
-#else
         e_acc[0] = T::mfma32(ka[0], qf[0], neg_ref);
         e_acc[1] = T::mfma32(kb_[0], qf[0], neg_ref);
 #pragma unroll
@@ -378,18 +367,13 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
             e_acc[0] = T::mfma32(ka[c], qf[c], e_acc[0]);
             e_acc[1] = T::mfma32(kb_[c], qf[c], e_acc[1]);
         }
-#endif
         // first two chunks of V^T fragments: their latency hides behind the max and the first exponentials
         s16x8 va[2][DB];
         auto load_v = [&](int c, s16x8 (&a)[DB]) {
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
-#ifdef ABL_NOLDSREAD
-                const s16x4 t0 = {qf[db][0], qf[c][1], qf[db][2], qf[c][3]}, t1 = {qf[db][4], qf[c][5], qf[db][6], qf[c][7]};
-#else
                 const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (16 * c) * RB);
                 const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (16 * c + 8) * RB);
-#endif
                 a[db] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
             }
         };
@@ -445,19 +429,15 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         // ---- P = 2^E and O^T += V^T P^T, one 16-key chunk at a time -------------------------------
         // Chunk c contracts keys 16c..16c+15 in the order 16c + 8(i/4) + 4h + i%4 (i = element of the
         // lane's 8-wide k slice), which is the order the exponent registers already have.  The weights of
-        // chunk c+1 are computed between the MFMAs of chunk c (one MFMA, a few vector instructions, ...),
-        // which is what lets the matrix pipe and the vector ALU of this SIMD run at the same time.
+        // chunk c+1 are computed before the MFMAs of chunk c are issued, so they run while that chunk is in
+        // the matrix pipe.
         float ls = 0.f;
         auto weights = [&](int c) -> s16x8 {
             uint32_t pk[4];
 #pragma unroll
             for (int i = 0; i < 8; i += 2) {
                 const int kb = c >> 1, r = 8 * (c & 1) + i;
-#ifdef ABL_NOEXP
-                pk[i >> 1] = T::pack2(e_acc[kb][r], e_acc[kb][r + 1]);
-#else
                 pk[i >> 1] = T::pack2(fast_exp2(e_acc[kb][r]), fast_exp2(e_acc[kb][r + 1]));
-#endif
                 ls = T::add_pair(pk[i >> 1], ls);   // the denominator sums the rounded weights the MFMA uses
             }
             uint4 pu; pu.x = pk[0]; pu.y = pk[1]; pu.z = pk[2]; pu.w = pk[3];
@@ -469,20 +449,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         for (int c = 0; c < 4; ++c) {
             s16x8 pnext = pcur;
             if (c + 1 < 4) pnext = weights(c + 1);
-#ifdef ABL_NOPV
-            for (int db = 0; db < (c == 0 ? 1 : 0); ++db) o_acc[db] = T::mfma32(va[c & 1][db], pcur, o_acc[db]);
-#else
 #pragma unroll
             for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma32(va[c & 1][db], pcur, o_acc[db]);
-#endif
-            if (c + 1 < 4) {
-                // interleave: 1 MFMA, then a quarter of the next chunk's vector work
-#pragma unroll
-                for (int i = 0; i < DB; ++i) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 24 / DB, 0);
-                }
-            }
             __builtin_amdgcn_sched_barrier(0);
             if (c + 2 < 4) load_v(c + 2, va[c & 1]);
             pcur = pnext;
@@ -506,12 +474,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         tile_of(e_next, it + 1, ktn, cn);
         const uint32_t e_after = list_entry(it + 2);   // read early, used next iteration
         wait_vmcnt<0>();       // this wave's share of tile `it` (and its mask words) has landed
-#ifndef ABL_NOBARRIER
         __syncthreads();       // everyone's has; stage STAGE^1 is no longer being read
-#endif
-#ifndef ABL_NODMA
         if (it + 1 < n_active) issue_tile(ktn, STAGE ^ 1);
-#endif
         if (cls_w != TILE_NONE) process_tile(stage_tag, kt, cls_w);
         if (MODE == MODE_DENSE && it + 1 < n_active && cn == TILE_MIXED) fetch_mask(ktn);   // after this tile's words were used
         e_cur = e_next; e_next = e_after;
