@@ -30,15 +30,6 @@ namespace minfer_attn {
 #ifndef MINFER_DECODE_STAGES
 #define MINFER_DECODE_STAGES 3
 #endif
-#ifndef MINFER_DECODE_CHUNK
-#define MINFER_DECODE_CHUNK 512
-#endif
-#ifndef MINFER_DECODE_K_VIA_LDS
-#define MINFER_DECODE_K_VIA_LDS 1
-#endif
-#ifndef MINFER_DECODE_ROTATE
-#define MINFER_DECODE_ROTATE 0
-#endif
 #ifndef MINFER_DECODE_MIN_WAVES_PER_SIMD
 #define MINFER_DECODE_MIN_WAVES_PER_SIMD 2
 #endif
@@ -112,7 +103,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     constexpr int PS = D + 4;    // floats per head in a wave's partial result (O, max, sum, pad)
 
     __shared__ __attribute__((aligned(1024))) char v_lds[kDecodeWaves][kGroupRows * RB];
-    __shared__ __attribute__((aligned(1024))) char k_lds[MINFER_DECODE_K_VIA_LDS ? kDecodeWaves : 1][kGroupRows * RB];
+    __shared__ __attribute__((aligned(1024))) char k_lds[kDecodeWaves][kGroupRows * RB];
     __shared__ __attribute__((aligned(16))) float part_lds[kDecodeWaves][16 * PS];
 
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
@@ -128,22 +119,15 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     const int row_hi = min(row_lo + p.chunk, ctx);
     const int n_groups = (row_hi - row_lo + kGroupRows - 1) / kGroupRows;
     const int my_groups = (n_groups - w + kDecodeWaves - 1) / kDecodeWaves;  // groups w, w+4, ...
-    // Workgroups that start together would otherwise walk their chunks in lockstep, all touching the
-    // same offset modulo the chunk size at the same time; each starts at its own rotation instead
-    // (the softmax merge does not care about the order of the keys).
-    const int rot = MINFER_DECODE_ROTATE && my_groups > 0 ? (int)((blockIdx.x * 2654435761u) >> 8) % my_groups : 0;
-    auto group_of = [&](int t) {   // t-th group this wave visits, as a group index inside the chunk
-        int j = t + rot;
-        if (j >= my_groups) j -= my_groups;
-        return w + (t < my_groups ? j : t) * kDecodeWaves;
-    };
+    auto group_of = [&](int t) { return w + t * kDecodeWaves; };
+    auto wave_has_work = [&](int ww) { return ww < n_groups; };
 
     const int heads_here = min(16, p.n_rep - hg * 16);
     const int head0 = g * p.n_rep + hg * 16;
     const short* Kb = (const short*)p.k + (int64_t)b * p.kv0 + (int64_t)g * p.kv1;
     const short* Vb = (const short*)p.v + (int64_t)b * p.kv0 + (int64_t)g * p.kv1;
     char* my_v = v_lds[w];
-    char* my_k = k_lds[MINFER_DECODE_K_VIA_LDS ? w : 0];
+    char* my_k = k_lds[w];
 
     // ---- Q^T fragments (B operand): column = head l16, k = d = 32c + 8*quad + 0..7 ------------
     s16x8 qf[KC];
@@ -163,16 +147,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     static_assert(NI == KC, "a 16-row group is NI row loads and KC contraction chunks");
     auto load_group = [&](int t, s16x8 (&kk)[NI], s16x8 (&vv)[NI]) {
         const int r0 = row_lo + group_of(t) * kGroupRows;
-        if (MINFER_DECODE_K_VIA_LDS) {
 #pragma unroll
-            for (int j = 0; j < NI; ++j) {
-                const int row = j * RPI + lane / G;
-                kk[j] = *reinterpret_cast<const s16x8*>(Kb + (int64_t)min(r0 + row, row_hi - 1) * p.kv2 + 8 * (lane % G));
-            }
-        } else {   // straight into the A-operand layout (row l16, d = 32c + 8*quad + 0..7): 64-byte pieces
-            const short* ksrc = Kb + (int64_t)min(r0 + l16, row_hi - 1) * p.kv2 + 8 * quad;
-#pragma unroll
-            for (int c = 0; c < KC; ++c) kk[c] = *reinterpret_cast<const s16x8*>(ksrc + 32 * c);
+        for (int j = 0; j < NI; ++j) {
+            const int row = j * RPI + lane / G;
+            kk[j] = *reinterpret_cast<const s16x8*>(Kb + (int64_t)min(r0 + row, row_hi - 1) * p.kv2 + 8 * (lane % G));
         }
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
@@ -196,7 +174,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     auto consume = [&](int t, const s16x8 (&kk)[NI], const s16x8 (&vv)[NI]) {
         // ---- S^T = K Q^T: lane gets head l16, keys 4*quad + r --------------------------------
         f32x4 s = {0.f, 0.f, 0.f, 0.f};
-        if (MINFER_DECODE_K_VIA_LDS) {
+        {   // park the K rows in LDS (swizzled) and read them back as A operands (row l16, d = 32c + 8*quad + 0..7)
 #pragma unroll
             for (int j = 0; j < NI; ++j) {
                 const int row = j * RPI + lane / G;
@@ -209,9 +187,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
                 const s16x8 a = *reinterpret_cast<const s16x8*>(rowp + 16 * ((4 * c + quad) ^ sw));
                 s = T::mfma16(a, qf[c], s);
             }
-        } else {
-#pragma unroll
-            for (int c = 0; c < KC; ++c) s = T::mfma16(kk[c], qf[c], s);
         }
         const int key0 = row_lo + group_of(t) * kGroupRows + 4 * quad;
 #pragma unroll
@@ -278,12 +253,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
         float M = -INFINITY;
 #pragma unroll
         for (int ww = 0; ww < kDecodeWaves; ++ww)
-            if (ww < n_groups) M = fmaxf(M, part_lds[ww][hh * PS + D]);
+            if (wave_has_work(ww)) M = fmaxf(M, part_lds[ww][hh * PS + D]);
         float o = 0.f, l = 0.f;
 #pragma unroll
         for (int ww = 0; ww < kDecodeWaves; ++ww) {
             const float* src = part_lds[ww] + hh * PS;
-            if (ww < n_groups && src[D] > -INFINITY) {
+            if (wave_has_work(ww) && src[D] > -INFINITY) {
                 const float wgt = fast_exp2((src[D] - M) * c2);
                 o += src[d] * wgt;
                 l += src[D + 1] * wgt;
@@ -348,17 +323,28 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     }
 }
 
-constexpr int kDecodeChunk = MINFER_DECODE_CHUNK;
-
-// cache rows per workgroup: 512, or more for very long caches so that a row never has more than 64 chunks
-static int decode_chunk_rows(int64_t Lmax) {
+// Cache rows per workgroup.  Smallest: 256 (or more for very long caches, so that a row never has more
+// than 64 chunks, which is what one wave of the combine kernel merges).  Larger chunks mean fewer
+// partials and fewer workgroup start-ups, so the launcher doubles the chunk while the grid would still
+// hold well over a thousand workgroups.  The workspace is sized for the smallest chunk.
+static int decode_min_chunk_rows(int64_t Lmax) {
     int64_t c = (Lmax + 63) / 64;
     c = (c + 63) / 64 * 64;
-    return (int)(c > kDecodeChunk ? c : kDecodeChunk);
+    return (int)(c > 256 ? c : 256);
+}
+static int decode_chunk_rows(int64_t B, int64_t Hkv, int64_t n_hg, int64_t Lmax) {
+#ifdef MINFER_DECODE_CHUNK
+    const int forced = MINFER_DECODE_CHUNK;
+    return forced > decode_min_chunk_rows(Lmax) ? forced : decode_min_chunk_rows(Lmax);
+#else
+    int chunk = decode_min_chunk_rows(Lmax);
+    while (chunk < 1024 && B * Hkv * n_hg * ((Lmax + 2 * chunk - 1) / (2 * chunk)) >= 2048) chunk *= 2;
+    return chunk;
+#endif
 }
 
 static size_t decode_ws_bytes(int64_t B, int64_t Hq, int64_t Lmax, int64_t D) {
-    const int64_t chunk = decode_chunk_rows(Lmax);
+    const int64_t chunk = decode_min_chunk_rows(Lmax);
     const int64_t S = (Lmax + chunk - 1) / chunk;
     return (size_t)(B * Hq * S * (D + 2) * 4 + 255) / 256 * 256 + 256;
 }
@@ -401,12 +387,12 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode(int dtype, const void* q, const 
     p.q = q; p.k = k_cache; p.v = v_cache; p.ctx = ctx_lens;
     p.q0 = st->q0; p.q1 = st->q1; p.kv0 = st->kv0; p.kv1 = st->kv1; p.kv2 = st->kv2;
     p.B = (int)B; p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.n_rep = (int)(Hq / Hkv); p.Lmax = (int)Lmax;
-    p.chunk = decode_chunk_rows(Lmax);
+    p.n_hg = (p.n_rep + 15) / 16;
+    p.chunk = decode_chunk_rows(B, Hkv, p.n_hg, Lmax);
     p.S = (int)((Lmax + p.chunk - 1) / p.chunk);
     if (p.S < 1) p.S = 1;
     if ((int64_t)B * p.S * Hkv * ((Hq / Hkv + 15) / 16) > 0x7fffffffLL)
         return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: problem too large for one launch");
-    p.n_hg = (p.n_rep + 15) / 16;
     p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
     const size_t o_bytes = (size_t)B * Hq * p.S * D * 4;
     p.part_o = (float*)workspace;
