@@ -4,8 +4,9 @@ A step is one call of the prefill operator on the Llama-3-8B-shaped workload (B=
 S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmic TFLOP/s
 (4*D*Hq*attended pairs), inputs resident in HBM, every kernel the op launches inside the timed
 region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
-under "decode" with its own HBM roofline, and the reference's CPU attention path (torch SDPA in
-fp32 on the host cores) under "cpu_baseline".  Prints ONE JSON line.
+under "decode" with its own HBM roofline, the rotary-embedding step that feeds attention under "rope"
+and "rope_kv_append", and the reference's CPU attention path (torch SDPA in fp32 on the host cores) under
+"cpu_baseline".  Prints ONE JSON line.
 """
 import argparse
 import ctypes
@@ -78,6 +79,21 @@ def cpu_baseline(torch, workloads, refs, L):
     return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"refs.flash_attn (torch SDPA, fp32, dense causal mask) on the full S={L} workload, median of 3: {t * 1e3:.1f} ms",
             "host_cpus": os.cpu_count()}
+
+
+def rope_cpu_baseline(torch, workloads, refs):
+    """The reference's CPU statement of il_rope (torch expressions in fp32; reference: refs.py:12-29) on one
+    batch entry of the reference test's shape."""
+    x = workloads.rope_input(seed=0, B=1)
+    refs.il_rope(x[:, :64], 64, 2048, 1e6)
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        refs.il_rope(x, 64, 2048, 1e6)
+        ts.append(time.perf_counter() - t0)
+    t = sorted(ts)[1]
+    return {"value": workloads.rope_bytes(1, 4096, 48, 64) / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"refs.il_rope (torch, fp32) on x [1,4096,48,128], median of 3: {t * 1e3:.1f} ms"}
 
 
 def main():
@@ -159,6 +175,26 @@ def main():
     d_gbs = dbytes / (d_avg_ms * 1e-3) / 1e9
     del kc, vc
 
+    # ---- the step before attention: rotary embedding, alone and fused with the cache append ----
+    x = workloads.rope_input(seed=0, device=dev)                      # the reference test's shape
+    rstep = lambda: kerns.il_rope(64, 2048, 1e6, x)
+    for _ in range(3):
+        rstep()
+    torch.cuda.synchronize()
+    r_avg_ms, r_med_ms = ev.time_each(rstep, stream, 20)
+    rbytes = workloads.rope_bytes(8, 4096, 48, 64)
+    r_gbs = rbytes / (r_avg_ms * 1e-3) / 1e9
+    del x
+    aq, ak, av, apos, akc, avc = workloads.kv_append(seed=0, device=dev, B=8, L=4096)
+    astep = lambda: kerns.rope_kv_append(1, 128, 5e5, aq, ak, av, apos, akc, avc)
+    for _ in range(3):
+        astep()
+    torch.cuda.synchronize()
+    a_avg_ms, a_med_ms = ev.time_each(astep, stream, 20)
+    abytes = workloads.kv_append_bytes(8, 4096, 32, 8, 128, 128)
+    a_gbs = abytes / (a_avg_ms * 1e-3) / 1e9
+    del aq, ak, av, akc, avc
+
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -177,8 +213,17 @@ def main():
                                 "kernel": "decode_split_kernel<F16,128> + decode_combine_kernel",
                                 "algorithmic_bytes": dbytes}},
     }
+    rec["rope"] = {"value": r_gbs, "unit": "GB/s", "ms": r_avg_ms, "median_ms": r_med_ms,
+                   "workload": "il_rope in place, x [8,4096,48,128] fp16, rotary_dim 64, base 1e6, start_pos 2048 (reference test/kernels.py:76-96)",
+                   "roofline": {"bound": "hbm", "achieved": r_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r_gbs / PEAK_HBM_GBS,
+                                "traffic": None, "kernel": "rope_kernel<F16,interleaved,in place>", "algorithmic_bytes": rbytes}}
+    rec["rope_kv_append"] = {"value": a_gbs, "unit": "GB/s", "ms": a_avg_ms, "median_ms": a_med_ms,
+                             "workload": "NeoX rope(q) in place + rope(k), v appended to the cache: B=8 L=4096 Hq=32 Hkv=8 D=128 fp16, rotary_dim 128, base 5e5",
+                             "roofline": {"bound": "hbm", "achieved": a_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a_gbs / PEAK_HBM_GBS,
+                                          "traffic": None, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
+        rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)
     print(json.dumps(rec))
 
 

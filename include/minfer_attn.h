@@ -98,6 +98,38 @@ int minfer_flash_attn_varlen(int dtype, const void* q, const void* k, const void
                              void* out, int64_t Hq, int64_t Hkv, int64_t T, int64_t D,
                              const minfer_attn_strides* strides, void* stream);
 
+/* Rotary embedding styles. */
+#define MINFER_ROPE_INTERLEAVED 0   /* pairs (2i, 2i+1) of a head   (reference: il_rope) */
+#define MINFER_ROPE_NEOX 1          /* pairs (i, i + rotary_dim/2)  (reference: neox_rope) */
+
+/*
+ * Rotary position embedding, in place: x [B,L,H,D] contiguous; for the token at index l the position is
+ * start_pos + l; pair i < rotary_dim/2 of every head is rotated by the angle
+ * pos * freq_base^(-2i/rotary_dim): (x0, x1) -> (cos*x0 - sin*x1, sin*x0 + cos*x1); elements
+ * rotary_dim..D-1 are not touched.  Replaces il_rope_cuda / neox_rope_cuda and their kernels
+ * (reference: il_rope/op.cuh:20-58, il_rope/kernel.cuh:9-39, neox_rope/op.cuh, neox_rope/kernel.cuh:9-38;
+ * oracle refs.py:12-47).  Beyond the reference: dtype may be MINFER_ATTN_BF16; rotary_dim must be even
+ * and at most 256.
+ */
+int minfer_rope(int dtype, int style, void* x, int64_t B, int64_t L, int64_t H, int64_t D,
+                int64_t rotary_dim, int64_t start_pos, double freq_base, void* stream);
+
+/*
+ * The step before attention, fused (reference: the il_rope(q), il_rope(k) calls and the cache they feed,
+ * src/minfer/core.py:228-232, cache layout core.py:105-127): q [B,L,Hq,D] is rotated in place; k [B,L,Hkv,D]
+ * is rotated and written to k_cache[b, g, positions[b] + l, :]; v [B,L,Hkv,D] is copied to the same row of
+ * v_cache.  positions is int32 [B] on the device (the number of rows sequence b already holds); token l of
+ * sequence b has position positions[b] + l.  Caches are [B,Hkv,Lmax,D] with the given element strides
+ * (multiples of 8) for their first three dims; rows outside 0..Lmax-1 are not written (q is still
+ * rotated).  k and v are only read.  All pointers 16-byte aligned, D a multiple of 8, rotary_dim a
+ * multiple of 8 (interleaved) or 16 (NeoX).  No counterpart as one call in the reference.
+ */
+int minfer_rope_kv_append(int dtype, int style, void* q, const void* k, const void* v,
+                          const int32_t* positions, void* k_cache, void* v_cache,
+                          int64_t B, int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
+                          int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_row,
+                          int64_t rotary_dim, double freq_base, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

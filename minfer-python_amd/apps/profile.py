@@ -1,4 +1,4 @@
-"""One un-timed call of an attention op, for an external profiler, e.g.
+"""One un-timed call of an op of the attention path, for an external profiler, e.g.
 
     rocprofv3 --kernel-trace --stats --output-format csv -- python minfer-python_amd/apps/profile.py --kernel flash_attn --which minfer
     rocprofv3 --pmc SQ_INSTS_VALU_MFMA_MOPS_F16 SQ_BUSY_CYCLES -- python minfer-python_amd/apps/profile.py --kernel flash_attn --which minfer
@@ -80,6 +80,32 @@ def flash_attn_varlen(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def il_rope(backend: str, which: str, workload: str, repeat: int):
+    """The reference test's shape (reference: test/kernels.py:80): x [8,4096,48,128], rotary 64, base 1e6."""
+    kerns = KernelBackend(backend)
+    x = workloads.rope_input(device="cuda")
+    fn = (lambda: kerns.il_rope(64, 2048, 1e6, x)) if which == "minfer" else (lambda: refs.il_rope(x, 64, 2048, 1e6))
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
+def rope_kv_append(backend: str, which: str, workload: str, repeat: int):
+    """NeoX rope(q), rope(k) -> cache, v -> cache at the Llama-3-8B head shape, B=8, L=4096."""
+    kerns = KernelBackend(backend)
+    q, k, v, pos, kc, vc = workloads.kv_append(device="cuda", B=8, L=4096)
+    if which == "minfer":
+        fn = lambda: kerns.rope_kv_append(1, 128, 5e5, q, k, v, pos, kc, vc)
+    else:
+        def fn():
+            refs.neox_rope(q, 128, 0, 5e5)
+            kc[:, :, :4096] = refs.neox_rope(k, 128, 0, 5e5).transpose(1, 2)
+            vc[:, :, :4096] = v.transpose(1, 2)
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def copy(backend: str, which: str, workload: str, repeat: int):
     """A plain device-to-device copy of 1 GiB: the known-size kernel that HBM byte counters
     (FETCH_SIZE / WRITE_SIZE) are calibrated against."""
@@ -92,7 +118,7 @@ def copy(backend: str, which: str, workload: str, repeat: int):
 
 if __name__ == "__main__":
     KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
-               "copy": copy}
+               "il_rope": il_rope, "rope_kv_append": rope_kv_append, "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)

@@ -101,3 +101,38 @@ def decode_bytes(ctx_lens, Hq, Hkv, D, itemsize=2):
     """K and V rows read once per KV head, plus q and out."""
     B = len(ctx_lens)
     return int(sum(int(c) for c in ctx_lens)) * Hkv * D * 2 * itemsize + 2 * B * Hq * D * itemsize
+
+
+def rope_input(seed=0, device="cpu", B=8, L=4096, H=48, D=128, dtype=torch.float16):
+    """x [B,L,H,D] ~ N(0,1): the shape the reference tests its rotary kernels on
+    (reference: test/kernels.py:80-82; rotary_dim 64, base 1e6, start_pos 0 or 2048 there)."""
+    gen = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, L, H, D, generator=gen).to(dtype)
+    return x.to(device) if device != "cpu" else x
+
+
+def kv_append(seed=0, device="cpu", B=1, L=4096, Hq=32, Hkv=8, D=128, Lmax=None, dtype=torch.float16, pos_hi=1):
+    """Inputs of the rope + cache-append step at the Llama-3-8B shape: q [B,L,Hq,D], k/v [B,L,Hkv,D]
+    ~ N(0,1), positions int32 [B] uniform in [0, pos_hi), zero-filled caches [B,Hkv,Lmax,D]
+    (Lmax defaults to pos_hi - 1 + L, so that every row fits)."""
+    gen = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, L, Hq, D, generator=gen).to(dtype)
+    k = torch.randn(B, L, Hkv, D, generator=gen).to(dtype)
+    v = torch.randn(B, L, Hkv, D, generator=gen).to(dtype)
+    positions = torch.randint(0, pos_hi, (B,), generator=gen, dtype=torch.int32)
+    Lmax = Lmax if Lmax is not None else pos_hi - 1 + L
+    if device != "cpu":
+        q, k, v, positions = q.to(device), k.to(device), v.to(device), positions.to(device)
+    k_cache = torch.zeros(B, Hkv, Lmax, D, dtype=dtype, device=device)
+    v_cache = torch.zeros(B, Hkv, Lmax, D, dtype=dtype, device=device)
+    return q, k, v, positions, k_cache, v_cache
+
+
+def rope_bytes(B, L, H, rotary_dim, itemsize=2):
+    """Algorithmic HBM bytes of an in-place rotary embedding: the rotary part, read and written once."""
+    return 2 * B * L * H * rotary_dim * itemsize
+
+
+def kv_append_bytes(B, L, Hq, Hkv, D, rotary_dim, itemsize=2):
+    """q's rotary part read and written; k and v read once; their cache rows written once."""
+    return (2 * B * L * Hq * rotary_dim + 4 * B * L * Hkv * D) * itemsize

@@ -1,0 +1,288 @@
+// Rotary position embedding for gfx950, in place and fused with the KV-cache append.
+//
+// What the reference computes (reference: src/minfer/kernels/torch_ext/csrc/cuda/il_rope/kernel.cuh:9-39,
+// neox_rope/kernel.cuh:9-38, oracle src/minfer/kernels/refs.py:12-47): for token position `pos` and pair
+// index i < rotary_dim/2, angle = pos * freq_base^(-2i/rotary_dim), and the pair (x0, x1) becomes
+// (cos*x0 - sin*x1, sin*x0 + cos*x1).  Interleaved style pairs elements (2i, 2i+1) of a head, NeoX style
+// pairs (i, i + rotary_dim/2).  Elements past rotary_dim are left alone.  x is [B, L, n_heads, head_dim].
+//
+// These are HBM-bound byte movers, so the design is about touching each byte once in 16-byte lane
+// accesses and about not paying for the transcendental per element as the reference's one-thread-per-pair
+// kernels do: the angle depends only on (position, pair), so a workgroup computes one cos/sin table per
+// token in LDS (rotary_dim/2 entries; the frequencies arrive as kernel arguments, the angle is reduced in
+// fp64 so that positions in the hundreds of thousands lose nothing) and every head of the token reuses
+// it.  Only the rotary part of a head is read and written.
+//
+// The fused producer does what the model does right before attention (reference: src/minfer/core.py:228-232,
+// cache layout core.py:105-127): rotate q in place, rotate k while copying it into the KV cache
+// [B, n_kv_heads, Lmax, head_dim] at row positions[b] + l, copy v into the cache.  k is read once and never
+// written back, the cache row is written once.
+#include <algorithm>
+
+#include "attn_common.h"
+#include "attn_host.h"
+
+namespace minfer_attn {
+
+constexpr int kRopeThreads = 256;
+constexpr int kMaxPairs = 128;    // rotary_dim <= 256
+
+enum { ROPE_IL = MINFER_ROPE_INTERLEAVED, ROPE_NEOX = MINFER_ROPE_NEOX };
+
+struct RopeParams {
+    void* x;                  // [B, L, H, D], rotated in place (q of the fused producer)
+    const void* k;            // fused: [B, L, Hkv, D]
+    const void* v;            // fused: [B, L, Hkv, D]
+    void* k_cache;            // fused: [B, Hkv, Lmax, D] with element strides c0, c1, c2
+    void* v_cache;
+    const int32_t* positions; // fused: [B] first cache row of each sequence; otherwise null
+    int64_t c0, c1, c2;
+    int B, L, H, Hkv, D, rd, Lmax;
+    int start_pos;            // not fused: position of token l is start_pos + l
+    double inv_freq[kMaxPairs];
+};
+
+// The rotated pair, rounded to the element type: low half = cos*x0 - sin*x1, high half = sin*x0 + cos*x1.
+template <class T> MA_DEV uint32_t rotate_pair(float c, float s, short a, short b) {
+    const float x0 = T::to_float(a), x1 = T::to_float(b);
+    return T::pack2(c * x0 - s * x1, s * x0 + c * x1);
+}
+
+// cos/sin of pos * inv_freq[i]: the product and its reduction to a fraction of a turn are done in fp64
+// (exact enough for any int32 position), the sine and cosine of the reduced angle in fp32.
+MA_DEV f32x2 table_entry(double inv_freq, int pos) {
+    const double turns = (double)pos * inv_freq * 0.15915494309189535;   // angle / 2pi
+    const float r = (float)((turns - rint(turns)) * 6.283185307179586);  // in [-pi, pi]
+    float s, c;
+    sincosf(r, &s, &c);
+    return f32x2{c, s};
+}
+
+// One token per loop trip: every thread requests the 16-byte chunks it owns (a few in flight), the first
+// rd/2 threads meanwhile fill the token's cos/sin table, one barrier, then rotate and store.
+//
+// Chunk numbering inside a token.  Rotary chunks of a tensor with NH heads: interleaved style, chunk c of
+// head hd covers elements 8c..8c+7 (pairs 4c..4c+3), rd/8 chunks per head; NeoX style, chunk c covers
+// elements 8c..8c+7 and their partners rd/2 + 8c.., rd/16 chunks per head.  Sections, in order: q rotary,
+// then (fused only) k rotary, k tail (elements rd..D-1, copied), v (copied).
+template <class T, int STYLE, bool FUSED>
+__global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) {
+    __shared__ f32x2 tab[2][kMaxPairs];
+    const int tid = threadIdx.x;
+    const int half_rd = p.rd >> 1;
+    const int cph = STYLE == ROPE_IL ? p.rd >> 3 : p.rd >> 4;   // rotary chunks per head
+    const int tail = (p.D - p.rd) >> 3;                         // copy chunks per head past the rotary part
+    const int n_q = p.H * cph;
+    const int n_kr = FUSED ? p.Hkv * cph : 0;
+    const int n_kt = FUSED ? p.Hkv * tail : 0;
+    const int n_v = FUSED ? p.Hkv * (p.D >> 3) : 0;
+    const int n_all = n_q + n_kr + n_kt + n_v;
+    const int tokens = p.B * p.L;
+
+    int parity = 0;
+    for (int tok = blockIdx.x; tok < tokens; tok += gridDim.x, parity ^= 1) {
+        const int b = tok / p.L, l = tok - b * p.L;
+        const int pos = FUSED ? p.positions[b] + l : p.start_pos + l;
+        const bool row_ok = !FUSED || (pos >= 0 && pos < p.Lmax);   // cache row exists
+
+        short* xq = (short*)p.x + (int64_t)tok * p.H * p.D;
+        const short* xk = FUSED ? (const short*)p.k + (int64_t)tok * p.Hkv * p.D : nullptr;
+        const short* xv = FUSED ? (const short*)p.v + (int64_t)tok * p.Hkv * p.D : nullptr;
+        short* ck = FUSED ? (short*)p.k_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
+        short* cv = FUSED ? (short*)p.v_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
+
+        // Where chunk t of the token lives: kind 0 rotate, 1 copy, 2 nothing.  Evaluated once to request the
+        // chunk and again to store it (the index is made opaque in between), so that only the loaded data
+        // stays in registers across the barrier.
+        auto locate = [&](int t, const short*& src, short*& dst, int& kind, int& chunk) __attribute__((always_inline)) {
+            src = xq; dst = xq; kind = 2; chunk = 0;
+            if (t < n_q) {
+                const int hd = t / cph; chunk = t - hd * cph;
+                src = dst = xq + hd * p.D + 8 * chunk;
+                kind = 0;
+            } else if (FUSED && t < n_all && row_ok) {
+                t -= n_q;
+                if (t < n_kr) {
+                    const int hd = t / cph; chunk = t - hd * cph;
+                    src = xk + hd * p.D + 8 * chunk;
+                    dst = ck + hd * p.c1 + 8 * chunk;
+                    kind = 0;
+                } else if (t < n_kr + n_kt) {
+                    t -= n_kr;
+                    const int hd = t / tail, c = t - hd * tail;
+                    src = xk + hd * p.D + p.rd + 8 * c;
+                    dst = ck + hd * p.c1 + p.rd + 8 * c;
+                    kind = 1;
+                } else {
+                    t -= n_kr + n_kt;
+                    const int per = p.D >> 3, hd = t / per, c = t - hd * per;
+                    src = xv + hd * p.D + 8 * c;
+                    dst = cv + hd * p.c1 + 8 * c;
+                    kind = 1;
+                }
+            }
+        };
+        // chunks in flight per thread: a NeoX rotary chunk is two 16-byte pieces, so half as many
+        constexpr int UN = STYLE == ROPE_IL ? 4 : 2;
+        s16x8 lo[UN], hi[UN];
+        auto request = [&](int t0) __attribute__((always_inline)) {
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const short* src; short* dst; int kind, chunk;
+                locate(t0 + u * kRopeThreads, src, dst, kind, chunk);
+                lo[u] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+                if (kind != 2) lo[u] = *reinterpret_cast<const s16x8*>(src);
+                hi[u] = lo[u];
+                if (STYLE == ROPE_NEOX && kind == 0) hi[u] = *reinterpret_cast<const s16x8*>(src + half_rd);
+            }
+        };
+        auto finish = [&](int t0) __attribute__((always_inline)) {
+            asm volatile("" : "+v"(t0));
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const short* src; short* dst; int kind, chunk;
+                locate(t0 + u * kRopeThreads, src, dst, kind, chunk);
+                if (kind == 2) continue;
+                s16x8 a = lo[u];
+                if (kind == 0) {
+                    if (STYLE == ROPE_IL) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) {
+                            const f32x2 cs = tab[parity][4 * chunk + j];
+                            const uint32_t pk = rotate_pair<T>(cs[0], cs[1], a[2 * j], a[2 * j + 1]);
+                            a[2 * j] = (short)(pk & 0xffffu);
+                            a[2 * j + 1] = (short)(pk >> 16);
+                        }
+                    } else {
+                        s16x8 b = hi[u];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const f32x2 cs = tab[parity][8 * chunk + j];
+                            const uint32_t pk = rotate_pair<T>(cs[0], cs[1], a[j], b[j]);
+                            a[j] = (short)(pk & 0xffffu);
+                            b[j] = (short)(pk >> 16);
+                        }
+                        *reinterpret_cast<s16x8*>(dst + half_rd) = b;
+                    }
+                }
+                *reinterpret_cast<s16x8*>(dst) = a;
+            }
+        };
+        // first batch of chunks requested, then the token's table while those loads are in flight
+        request(tid);
+        if (tid < half_rd) tab[parity][tid] = table_entry(p.inv_freq[tid], pos);
+        __syncthreads();   // the only barrier of the token: the next token writes the other table
+        finish(tid);
+        for (int t0 = tid + UN * kRopeThreads; t0 < n_all; t0 += UN * kRopeThreads) {
+            request(t0);
+            finish(t0);
+        }
+    }
+}
+
+// Any even rotary_dim, any alignment: one thread per (token, head, pair), as the reference launches it.
+template <class T, int STYLE>
+__global__ __launch_bounds__(kRopeThreads) void rope_scalar_kernel(const RopeParams p) {
+    const int half_rd = p.rd >> 1;
+    const int64_t total = (int64_t)p.B * p.L * p.H * half_rd;
+    for (int64_t i = (int64_t)blockIdx.x * kRopeThreads + threadIdx.x; i < total; i += (int64_t)gridDim.x * kRopeThreads) {
+        const int pair = (int)(i % half_rd);
+        const int64_t row = i / half_rd;                 // (token, head)
+        const int l = (int)((row / p.H) % p.L);
+        const f32x2 cs = table_entry(p.inv_freq[pair], p.start_pos + l);
+        short* xh = (short*)p.x + row * p.D;
+        const int i0 = STYLE == ROPE_IL ? 2 * pair : pair, i1 = STYLE == ROPE_IL ? 2 * pair + 1 : pair + half_rd;
+        const uint32_t pk = rotate_pair<T>(cs[0], cs[1], xh[i0], xh[i1]);
+        xh[i0] = (short)(pk & 0xffffu);
+        xh[i1] = (short)(pk >> 16);
+    }
+}
+
+static int fill_rope(RopeParams& p, int dtype, int style, int64_t B, int64_t L, int64_t H, int64_t D,
+                     int64_t rotary_dim, double freq_base, const char* op) {
+    char msg[160];
+    auto bad = [&](const char* what) {
+        snprintf(msg, sizeof msg, "%s: %s", op, what);
+        return fail(MINFER_ATTN_EINVAL, msg);
+    };
+    if (dtype != MINFER_ATTN_F16 && dtype != MINFER_ATTN_BF16) return bad("dtype must be MINFER_ATTN_F16 or MINFER_ATTN_BF16");
+    if (style != ROPE_IL && style != ROPE_NEOX) return bad("style must be MINFER_ROPE_INTERLEAVED or MINFER_ROPE_NEOX");
+    if (B < 0 || L < 0 || H < 0 || D <= 0) return bad("negative size");
+    if (rotary_dim < 0 || rotary_dim > D) return bad("rotary_dim must be in 0..head_dim");
+    if (rotary_dim % 2 != 0) return bad("rotary_dim must be even");
+    if (rotary_dim > 2 * kMaxPairs) return bad("rotary_dim > 256 unsupported");
+    if (!(freq_base > 0.0)) return bad("freq_base must be positive");
+    if (B * L > 0x7fffffffLL || H > 65535 || D > 65535) return bad("problem too large");
+    p.B = (int)B; p.L = (int)L; p.H = (int)H; p.D = (int)D; p.rd = (int)rotary_dim;
+    for (int i = 0; i < rotary_dim / 2; ++i) p.inv_freq[i] = pow(freq_base, -2.0 * i / (double)rotary_dim);
+    return MINFER_ATTN_OK;
+}
+
+static bool vector_ok(int style, int64_t D, int64_t rd) {
+    return D % 8 == 0 && rd % (style == ROPE_IL ? 8 : 16) == 0;
+}
+
+template <bool FUSED>
+static int launch_rope(int dtype, int style, const RopeParams& p, hipStream_t stream) {
+    const int tokens = p.B * p.L;
+    const int grid = std::min(tokens, 256 * 16);
+    if (dtype == MINFER_ATTN_F16) {
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<F16, ROPE_IL, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_kernel<F16, ROPE_NEOX, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+    } else {
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<BF16, ROPE_IL, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_kernel<BF16, ROPE_NEOX, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+    }
+    return check_launch("rope_kernel");
+}
+
+}  // namespace minfer_attn
+
+using namespace minfer_attn;
+
+MINFER_ATTN_EXPORT int minfer_rope(int dtype, int style, void* x, int64_t B, int64_t L, int64_t H, int64_t D,
+                                   int64_t rotary_dim, int64_t start_pos, double freq_base, void* stream_v) {
+    clear_error();
+    RopeParams p{};
+    if (int rc = fill_rope(p, dtype, style, B, L, H, D, rotary_dim, freq_base, "rope")) return rc;
+    if (!x) return fail(MINFER_ATTN_EINVAL, "rope: x is null");
+    if (start_pos < 0 || start_pos + L > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "rope: positions must fit in int32");
+    if (B == 0 || L == 0 || H == 0 || rotary_dim == 0) return MINFER_ATTN_OK;
+    p.x = x; p.start_pos = (int)start_pos;
+    hipStream_t stream = (hipStream_t)stream_v;
+    if (vector_ok(style, D, rotary_dim) && aligned16(x)) return launch_rope<false>(dtype, style, p, stream);
+
+    const int64_t pairs = B * L * H * (rotary_dim / 2);
+    const int grid = (int)std::min<int64_t>((pairs + kRopeThreads - 1) / kRopeThreads, 256 * 32);
+    if (dtype == MINFER_ATTN_F16) {
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_scalar_kernel<F16, ROPE_IL>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_scalar_kernel<F16, ROPE_NEOX>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+    } else {
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_scalar_kernel<BF16, ROPE_IL>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_scalar_kernel<BF16, ROPE_NEOX>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+    }
+    return check_launch("rope_scalar_kernel");
+}
+
+MINFER_ATTN_EXPORT int minfer_rope_kv_append(int dtype, int style, void* q, const void* k, const void* v,
+                                             const int32_t* positions, void* k_cache, void* v_cache, int64_t B,
+                                             int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
+                                             int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_row,
+                                             int64_t rotary_dim, double freq_base, void* stream_v) {
+    clear_error();
+    RopeParams p{};
+    if (int rc = fill_rope(p, dtype, style, B, L, Hq, D, rotary_dim, freq_base, "rope_kv_append")) return rc;
+    if (!q || !k || !v || !positions || !k_cache || !v_cache) return fail(MINFER_ATTN_EINVAL, "rope_kv_append: null pointer");
+    if (Hkv <= 0 || Hkv > 65535 || Lmax < 0 || Lmax > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "rope_kv_append: bad n_kv_heads or Lmax");
+    if (!vector_ok(style, D, rotary_dim))
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append: head_dim must be a multiple of 8 and rotary_dim of 8 (interleaved) or 16 (NeoX)");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || !aligned16(k_cache) || !aligned16(v_cache))
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append: tensors must be 16-byte aligned");
+    if (cache_stride_b % 8 || cache_stride_h % 8 || cache_stride_row % 8 || cache_stride_b < 0 || cache_stride_h < 0 || cache_stride_row < 0)
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append: cache strides must be non-negative multiples of 8 elements");
+    if (B == 0 || L == 0) return MINFER_ATTN_OK;
+    p.x = q; p.k = k; p.v = v; p.k_cache = k_cache; p.v_cache = v_cache; p.positions = positions;
+    p.Hkv = (int)Hkv; p.Lmax = (int)Lmax;
+    p.c0 = cache_stride_b; p.c1 = cache_stride_h; p.c2 = cache_stride_row;
+    return launch_rope<true>(dtype, style, p, (hipStream_t)stream_v);
+}

@@ -1,4 +1,5 @@
-// PyTorch (stable ABI) registration of the attention operators in namespace `minfer`.
+// PyTorch (stable ABI) registration of the attention operators, and of the rotary-embedding step
+// that feeds them, in namespace `minfer`.
 //
 // This file is the only place where torch types appear: it validates tensors exactly as the
 // reference host function does, turns them into pointers/strides and calls the C ABI of
@@ -181,18 +182,86 @@ void flash_attn_varlen_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype
              "flash_attn_varlen");
 }
 
+// Rotary embedding in place, same signature, argument meaning and checks as the reference's il_rope_cuda /
+// neox_rope_cuda (reference: src/minfer/kernels/torch_ext/csrc/cuda/il_rope/op.cuh:20-58 and
+// neox_rope/op.cuh); bfloat16 is admitted as well.
+namespace {
+void rope_hip(int style, const char* op, int64_t rotary_dim, int64_t start_pos, double freq_base,
+              Tensor& x) {   // [B, L, n_heads, head_dim] (before the transpose for flash_attn)
+    STD_TORCH_CHECK(on_gpu(x), op, ": x must be on the GPU");
+    STD_TORCH_CHECK(x.is_contiguous(), op, ": x must be contiguous");
+    STD_TORCH_CHECK(x.dim() == 4, op, ": x must be 4-D");
+    const ScalarType t = x.scalar_type();
+    STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, op, ": x must be float16 or bfloat16");
+    STD_TORCH_CHECK(rotary_dim <= x.size(3), op, ": rotary_dim exceeds head_dim");
+    check_rc(minfer_rope(t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16, style, x.mutable_data_ptr(),
+                         x.size(0), x.size(1), x.size(2), x.size(3), rotary_dim, start_pos, freq_base,
+                         current_stream()),
+             op);
+}
+}  // namespace
+
+void il_rope_hip(int64_t rotary_dim, int64_t start_pos, double freq_base, Tensor& x) {
+    rope_hip(MINFER_ROPE_INTERLEAVED, "il_rope", rotary_dim, start_pos, freq_base, x);
+}
+
+void neox_rope_hip(int64_t rotary_dim, int64_t start_pos, double freq_base, Tensor& x) {
+    rope_hip(MINFER_ROPE_NEOX, "neox_rope", rotary_dim, start_pos, freq_base, x);
+}
+
+// rope(q) in place, rope(k) -> k_cache, v -> v_cache in one pass: the step before attention
+// (reference: src/minfer/core.py:228-232) writing the reference's cache layout (core.py:105-127).
+void rope_kv_append_hip(int64_t style, int64_t rotary_dim, double freq_base,
+                        Tensor& q,                 // [B, L, n_heads, head_dim], rotated in place
+                        const Tensor& k,           // [B, L, n_kv_heads, head_dim]
+                        const Tensor& v,           // [B, L, n_kv_heads, head_dim]
+                        const Tensor& positions,   // [B] int32: rows each sequence already holds
+                        Tensor& k_cache,           // [B, n_kv_heads, Lmax, head_dim]
+                        Tensor& v_cache) {
+    STD_TORCH_CHECK(on_gpu(q) && on_gpu(k) && on_gpu(v) && on_gpu(positions) && on_gpu(k_cache) && on_gpu(v_cache),
+                    "rope_kv_append: all tensors must be on the GPU");
+    STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && k_cache.dim() == 4 && v_cache.dim() == 4 && positions.dim() == 1,
+                    "rope_kv_append: q, k, v and the caches must be 4-D and positions 1-D");
+    STD_TORCH_CHECK(q.is_contiguous() && k.is_contiguous() && v.is_contiguous(), "rope_kv_append: q, k and v must be contiguous");
+    STD_TORCH_CHECK(style == MINFER_ROPE_INTERLEAVED || style == MINFER_ROPE_NEOX, "rope_kv_append: style must be 0 (interleaved) or 1 (NeoX)");
+    const int dtype = dtype_code(q, k, v, k_cache, "rope_kv_append");
+    STD_TORCH_CHECK(v_cache.scalar_type() == q.scalar_type(), "rope_kv_append: caches must share q's dtype");
+    STD_TORCH_CHECK(positions.scalar_type() == ScalarType::Int && positions.is_contiguous(), "rope_kv_append: positions must be contiguous int32");
+    STD_TORCH_CHECK(k.sizes().equals(v.sizes()) && k_cache.sizes().equals(v_cache.sizes()), "rope_kv_append: k/v or cache shapes differ");
+    STD_TORCH_CHECK(k_cache.stride(-1) == 1 && v_cache.stride(-1) == 1 && k_cache.stride(0) == v_cache.stride(0) &&
+                    k_cache.stride(1) == v_cache.stride(1) && k_cache.stride(2) == v_cache.stride(2),
+                    "rope_kv_append: caches must be contiguous in head_dim and share strides");
+    STD_TORCH_CHECK(q.size(0) == k.size(0) && q.size(1) == k.size(1) && q.size(3) == k.size(3) && q.size(0) == k_cache.size(0) &&
+                    k.size(2) == k_cache.size(1) && q.size(3) == k_cache.size(3) && positions.size(0) == q.size(0),
+                    "rope_kv_append: expected q [B,L,Hq,D], k/v [B,L,Hkv,D], caches [B,Hkv,Lmax,D], positions [B]");
+    STD_TORCH_CHECK(rotary_dim <= q.size(3), "rope_kv_append: rotary_dim exceeds head_dim");
+    check_rc(minfer_rope_kv_append(dtype, (int)style, q.mutable_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
+                                   static_cast<const int32_t*>(positions.const_data_ptr()), k_cache.mutable_data_ptr(),
+                                   v_cache.mutable_data_ptr(), q.size(0), q.size(1), q.size(2), k.size(2), q.size(3),
+                                   k_cache.size(2), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2), rotary_dim,
+                                   freq_base, current_stream()),
+             "rope_kv_append");
+}
+
 STABLE_TORCH_LIBRARY(minfer, m) {
     // verbatim the reference's schema (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:30)
     m.def("flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()");
+    // verbatim the reference's schemas (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:25-26)
+    m.def("il_rope(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()");
+    m.def("neox_rope(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()");
     // extensions in the same style: ints first, inputs, out-parameter last, no return value
     m.def("flash_attn_decode(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k_cache, Tensor v_cache, Tensor ctx_lens, Tensor(a!) out) -> ()");
     m.def("flash_attn_varlen(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor cu_seqlens, int max_seqlen, Tensor(a!) out) -> ()");
+    m.def("rope_kv_append(int style, int rotary_dim, float freq_base, Tensor(a!) q, Tensor k, Tensor v, Tensor positions, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
 }
 
 STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-key name for ROCm devices too
     m.impl("flash_attn", TORCH_BOX(&flash_attn_hip));
     m.impl("flash_attn_decode", TORCH_BOX(&flash_attn_decode_hip));
     m.impl("flash_attn_varlen", TORCH_BOX(&flash_attn_varlen_hip));
+    m.impl("il_rope", TORCH_BOX(&il_rope_hip));
+    m.impl("neox_rope", TORCH_BOX(&neox_rope_hip));
+    m.impl("rope_kv_append", TORCH_BOX(&rope_kv_append_hip));
 }
 
 }  // namespace minfer

@@ -1,5 +1,5 @@
-"""PyTorch statements of what each attention op computes, for callers that want to compare or
-time against them the way the reference's apps do (reference: src/minfer/kernels/refs.py:53-55,
+"""PyTorch statements of what each op computes, for callers that want to compare or time against
+them the way the reference's apps do (reference: src/minfer/kernels/refs.py:12-55,
 apps/benchmark.py:240-248).  Nothing in the operator path calls these."""
 import torch
 import torch.nn.functional as F
@@ -27,3 +27,33 @@ def flash_attn_varlen(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, cu_seql
         if hi > lo:
             out[:, :, lo:hi] = F.scaled_dot_product_attention(Q[:, :, lo:hi], K[:, :, lo:hi], V[:, :, lo:hi], is_causal=True)
     return out
+
+
+def _rope_angles(L: int, rotary_dim: int, start_pos: int, base_freq: float, device) -> torch.Tensor:
+    """angle[l, i] = (start_pos + l) * base_freq^(-2i/rotary_dim), fp32 like the reference's."""
+    i = torch.arange(rotary_dim // 2, dtype=torch.float32, device=device)
+    inv = base_freq ** (-2.0 * i / rotary_dim)
+    return (torch.arange(L, dtype=torch.float32, device=device) + start_pos)[:, None] * inv[None, :]
+
+
+def il_rope(x: torch.Tensor, rotary_dim: int, start_pos: int, base_freq: float) -> torch.Tensor:
+    """Interleaved rotary embedding; x: (B, L, n_heads, head_dim).  Pairs (2i, 2i+1) rotate by angle[l, i]."""
+    ang = _rope_angles(x.shape[1], rotary_dim, start_pos, base_freq, x.device)
+    cos, sin = ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]
+    y = x.float().clone()
+    x0, x1 = y[..., 0:rotary_dim:2].clone(), y[..., 1:rotary_dim:2].clone()
+    y[..., 0:rotary_dim:2] = cos * x0 - sin * x1
+    y[..., 1:rotary_dim:2] = sin * x0 + cos * x1
+    return y.to(x.dtype)
+
+
+def neox_rope(x: torch.Tensor, rotary_dim: int, start_pos: int, base_freq: float) -> torch.Tensor:
+    """NeoX rotary embedding; x: (B, L, n_heads, head_dim).  Pairs (i, i + rotary_dim/2) rotate by angle[l, i]."""
+    ang = _rope_angles(x.shape[1], rotary_dim, start_pos, base_freq, x.device)
+    cos, sin = ang.cos()[None, :, None, :], ang.sin()[None, :, None, :]
+    y = x.float().clone()
+    h = rotary_dim // 2
+    x0, x1 = y[..., :h].clone(), y[..., h:rotary_dim].clone()
+    y[..., :h] = cos * x0 - sin * x1
+    y[..., h:rotary_dim] = sin * x0 + cos * x1
+    return y.to(x.dtype)

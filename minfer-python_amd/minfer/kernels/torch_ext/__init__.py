@@ -8,4 +8,5 @@ except ImportError as e:  # pragma: no cover
         "minfer.kernels.torch_ext._C is not built; run `python minfer-python_amd/build.py` "
         "(hipcc, gfx950) first"
     ) from e
-from .ops import flash_attn, flash_attn_decode, flash_attn_varlen  # noqa: E402,F401
+from .ops import (flash_attn, flash_attn_decode, flash_attn_varlen, il_rope, neox_rope,  # noqa: E402,F401
+                  rope_kv_append)

@@ -1,5 +1,6 @@
-"""Python wrappers and fake (meta) kernels of the attention ops, mirroring the reference's
-wrapper layer (reference: src/minfer/kernels/torch_ext/ops.py:234-266): positional pass-through
+"""Python wrappers and fake (meta) kernels of the attention ops and of the rotary-embedding step
+before them, mirroring the reference's wrapper layer (reference:
+src/minfer/kernels/torch_ext/ops.py:86-126, 234-266): positional pass-through
 to ``torch.ops.minfer.<op>.default``; the result is written into ``out``."""
 import torch
 
@@ -80,3 +81,57 @@ def _(qtype_int, qblock_size, qtype_size, q, k, v, cu_seqlens, max_seqlen, out):
     torch._check(q.device == k.device == v.device == cu_seqlens.device == out.device)
     torch._check(q.device.type == "cuda")
     torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and out.dim() == 4 and cu_seqlens.dim() == 1)
+
+
+
+def il_rope(rotary_dim: int, start_pos: int, freq_base: float, x: torch.Tensor):
+    """Interleaved rotary embedding, in place; x [B,L,n_heads,head_dim], token l at position start_pos + l."""
+    return torch.ops.minfer.il_rope.default(rotary_dim, start_pos, freq_base, x)
+
+
+@torch.library.register_fake("minfer::il_rope")
+def _(rotary_dim, start_pos, freq_base, x):
+    torch._check(x.dtype in _ACT_DTYPES)
+    torch._check(x.dim() == 4)
+    torch._check(x.device.type == "cuda")
+    torch._check(rotary_dim <= x.size(3))
+
+
+def neox_rope(rotary_dim: int, start_pos: int, freq_base: float, x: torch.Tensor):
+    """NeoX (two-halves) rotary embedding, in place; x [B,L,n_heads,head_dim]."""
+    return torch.ops.minfer.neox_rope.default(rotary_dim, start_pos, freq_base, x)
+
+
+@torch.library.register_fake("minfer::neox_rope")
+def _(rotary_dim, start_pos, freq_base, x):
+    torch._check(x.dtype in _ACT_DTYPES)
+    torch._check(x.dim() == 4)
+    torch._check(x.device.type == "cuda")
+    torch._check(rotary_dim <= x.size(3))
+
+
+def rope_kv_append(
+    style: int,
+    rotary_dim: int,
+    freq_base: float,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    positions: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+):
+    """Rotates q [B,L,n_heads,D] in place, writes the rotated k [B,L,n_kv_heads,D] and v into rows
+    positions[b] + l of the caches [B,n_kv_heads,Lmax,D]; style 0 = interleaved, 1 = NeoX; positions
+    int32 [B]."""
+    return torch.ops.minfer.rope_kv_append.default(style, rotary_dim, freq_base, q, k, v, positions, k_cache, v_cache)
+
+
+@torch.library.register_fake("minfer::rope_kv_append")
+def _(style, rotary_dim, freq_base, q, k, v, positions, k_cache, v_cache):
+    torch._check(q.dtype in _ACT_DTYPES)
+    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype)
+    torch._check(positions.dtype == torch.int32)
+    torch._check(q.device.type == "cuda")
+    torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and k_cache.dim() == 4 and v_cache.dim() == 4)
+    torch._check(rotary_dim <= q.size(3))

@@ -1,4 +1,4 @@
-"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c.
+"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c and rope_oracle.c.
 
 Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py may import this
 package.  The shipped operator never does: it launches HIP kernels or raises.
@@ -22,7 +22,7 @@ class _Strides(ctypes.Structure):
 
 
 def build(force=False):
-    """Compile attn_oracle.c into liboracle.so (gcc + OpenMP)."""
+    """Compile attn_oracle.c and rope_oracle.c into liboracle.so (gcc + OpenMP)."""
     so = os.path.join(_HERE, "liboracle.so")
     if force and os.path.exists(so):
         os.remove(so)
@@ -38,7 +38,7 @@ def lib():
             build()
         _LIB = ctypes.CDLL(so)
         for name in ("oracle_flash_attn", "oracle_flash_attn_rows", "oracle_flash_attn_decode",
-                     "oracle_flash_attn_varlen"):
+                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append"):
             getattr(_LIB, name).restype = ctypes.c_int
     return _LIB
 
@@ -130,3 +130,38 @@ def flash_attn_varlen(q, k, v, cu_seqlens):
     if rc != 0:
         raise ValueError(f"oracle_flash_attn_varlen rc={rc}")
     return out
+
+
+ROPE_INTERLEAVED, ROPE_NEOX = 0, 1
+
+
+def rope(style, x, rotary_dim, start_pos, freq_base):
+    """Rotary embedding of x [B,L,H,D] (reference: refs.py:12-47), fp64 arithmetic; returns a new
+    float32 array, unrounded."""
+    x = _f32(x).copy()
+    B, L, H, D = x.shape
+    rc = lib().oracle_rope(ctypes.c_int(style), _ptr(x), *[ctypes.c_int64(v) for v in (B, L, H, D, rotary_dim, start_pos)],
+                           ctypes.c_double(freq_base))
+    if rc != 0:
+        raise ValueError(f"oracle_rope rc={rc}")
+    return x
+
+
+def rope_kv_append(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq_base):
+    """rope(q), rope(k) -> k_cache rows positions[b]+l, v -> v_cache rows (reference: core.py:228-232,
+    cache layout core.py:105-127).  q/k/v [B,L,H*,D], caches [B,Hkv,Lmax,D].  Returns new float32
+    arrays (q, k_cache, v_cache)."""
+    q, k, v = _f32(q).copy(), _f32(k), _f32(v)
+    k_cache, v_cache = _f32(k_cache).copy(), _f32(v_cache).copy()
+    if hasattr(positions, "detach"):
+        positions = positions.detach().to("cpu").numpy()
+    pos = np.ascontiguousarray(np.asarray(positions, dtype=np.int32))
+    B, L, Hq, D = q.shape
+    Hkv, Lmax = k_cache.shape[1], k_cache.shape[2]
+    rc = lib().oracle_rope_kv_append(ctypes.c_int(style), _ptr(q), _ptr(k), _ptr(v), _ptr(pos, ctypes.c_int32),
+                                     _ptr(k_cache), _ptr(v_cache),
+                                     *[ctypes.c_int64(x) for x in (B, L, Hq, Hkv, D, Lmax, rotary_dim)],
+                                     ctypes.c_double(freq_base))
+    if rc != 0:
+        raise ValueError(f"oracle_rope_kv_append rc={rc}")
+    return q, k_cache, v_cache

@@ -8,6 +8,7 @@ LIB_PATH = os.path.join(ROOT, "minfer-python_amd", "lib", "libminfer_attn.so")
 HEADER = os.path.join(ROOT, "include", "minfer_attn.h")
 
 F16, BF16 = 1, 30
+ROPE_INTERLEAVED, ROPE_NEOX = 0, 1
 OK, EINVAL, EWORKSPACE, ELAUNCH = 0, -1, -2, -3
 
 
@@ -40,6 +41,12 @@ def lib():
         L.minfer_flash_attn_varlen.restype = ctypes.c_int
         L.minfer_flash_attn_varlen.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, i64,
                                                ctypes.POINTER(Strides), vp]
+        dbl = ctypes.c_double
+        L.minfer_rope.restype = ctypes.c_int
+        L.minfer_rope.argtypes = [ctypes.c_int, ctypes.c_int, vp, i64, i64, i64, i64, i64, i64, dbl, vp]
+        L.minfer_rope_kv_append.restype = ctypes.c_int
+        L.minfer_rope_kv_append.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
+                                            i64, i64, i64, i64, i64, dbl, vp]
         _lib = L
     return _lib
 
@@ -95,3 +102,18 @@ def flash_attn_varlen(q, k, v, cu_seqlens, max_seqlen, out):
     return lib().minfer_flash_attn_varlen(_dtype_code(q), q.data_ptr(), k.data_ptr(), v.data_ptr(),
                                           cu_seqlens.data_ptr(), cu_seqlens.numel() - 1, max_seqlen, out.data_ptr(),
                                           Hq, k.shape[1], T, D, ctypes.byref(st), _stream())
+
+
+def rope(style, x, rotary_dim, start_pos, freq_base):
+    """In-place rotary embedding of x [B,L,H,D] (contiguous)."""
+    B, L, H, D = x.shape
+    return lib().minfer_rope(_dtype_code(x), style, x.data_ptr(), B, L, H, D, rotary_dim, start_pos, freq_base, _stream())
+
+
+def rope_kv_append(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq_base):
+    """q [B,L,Hq,D] in place; k, v [B,L,Hkv,D] into rows positions[b]+l of the caches [B,Hkv,Lmax,D]."""
+    B, L, Hq, D = q.shape
+    return lib().minfer_rope_kv_append(_dtype_code(q), style, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                       positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), B, L, Hq,
+                                       k.shape[2], D, k_cache.shape[2], k_cache.stride(0), k_cache.stride(1),
+                                       k_cache.stride(2), rotary_dim, freq_base, _stream())

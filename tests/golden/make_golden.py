@@ -9,6 +9,9 @@ from the reference is imported.  Inputs are fp16-representable (q, k ~ N(0,1), v
 the fp16 output format itself does not eat the 2e-3 tolerance) and stored as fp16, so the
 fp16 kernels see exactly the values the expected output was computed from.
 
+The rotary-embedding fixture (rope_small.npz) pins the reference's torch formulation of both styles
+(reference src/minfer/kernels/refs.py:12-47) in float64 on seeded fp16-representable inputs.
+
 Run:  python tests/golden/make_golden.py
 """
 import os
@@ -73,6 +76,28 @@ def make_varlen(name, Hq, Hkv, D, lens, seed):
                         v=v.numpy().astype(np.float16), cu=cu, out=out.numpy().astype(np.float32))
 
 
+def make_rope(name, B, L, H, D, rotary_dim, start_pos, freq_base, seed):
+    """Expected values of both rotary styles from the reference's torch formulation, complex multiplication
+    by exp(i*theta) (reference src/minfer/kernels/refs.py:19-27 and 37-47), evaluated in float64."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(B, L, H, D, generator=g).half().double()
+    f = freq_base ** (-2.0 * torch.arange(rotary_dim // 2, dtype=torch.float64) / rotary_dim)
+    ang = (torch.arange(L, dtype=torch.float64) + start_pos)[:, None] * f[None, :]
+    rot = torch.polar(torch.ones_like(ang), ang)[None, :, None, :]
+    y_il = x.clone()
+    xc = torch.view_as_complex(x[..., :rotary_dim].reshape(B, L, H, rotary_dim // 2, 2).contiguous())
+    y_il[..., :rotary_dim] = torch.view_as_real(xc * rot).flatten(-2)
+    y_neox = x.clone()
+    h = rotary_dim // 2
+    xc = torch.view_as_complex(torch.stack([x[..., :h], x[..., h:rotary_dim]], dim=-1).contiguous())
+    yr = torch.view_as_real(xc * rot)
+    y_neox[..., :h] = yr[..., 0]
+    y_neox[..., h:rotary_dim] = yr[..., 1]
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), x=x.numpy().astype(np.float16), rotary_dim=rotary_dim,
+                        start_pos=start_pos, freq_base=freq_base, y_il=y_il.numpy().astype(np.float32),
+                        y_neox=y_neox.numpy().astype(np.float32))
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
     make("dense_causal_b1_h4_kv2_l16_d64", 1, 4, 2, 16, 64, "causal", 1)
@@ -80,4 +105,5 @@ if __name__ == "__main__":
     make("dense_random_b1_h8_kv1_l70_d64", 1, 8, 1, 70, 64, "random", 3)
     make_decode("decode_b3_h8_kv2_l50_d128", 3, 8, 2, 50, 128, 4)
     make_varlen("varlen_h4_kv2_d64", 4, 2, 64, [5, 1, 33, 70], 5)
+    make_rope("rope_small", 2, 9, 3, 64, 32, 2048, 1e6, 6)
     print("golden vectors written to", HERE)

@@ -74,6 +74,34 @@ def test_validation_rejects_before_launch():
                                       ctypes.byref(st), None) == capi.OK
 
 
+def test_rope_validation_rejects_before_launch():
+    """Fake pointers again: every call must be refused (or be an accepted empty problem) on the host."""
+    L = capi.lib()
+    rope = lambda dtype=capi.F16, style=0, x=0x1000, B=1, Ln=4, H=2, D=128, rd=64, start=0, base=1e4: \
+        L.minfer_rope(dtype, style, x, B, Ln, H, D, rd, start, base, None)
+    assert rope(dtype=7) == capi.EINVAL and "dtype" in capi.last_error()
+    assert rope(style=2) == capi.EINVAL and "style" in capi.last_error()
+    assert rope(rd=130) == capi.EINVAL and "rotary_dim" in capi.last_error()
+    assert rope(rd=7) == capi.EINVAL and "even" in capi.last_error()
+    assert rope(D=512, rd=512) == capi.EINVAL
+    assert rope(base=0.0) == capi.EINVAL and "freq_base" in capi.last_error()
+    assert rope(x=0) == capi.EINVAL
+    assert rope(start=-1) == capi.EINVAL
+    assert rope(start=1 << 31) == capi.EINVAL
+    assert rope(B=0) == capi.OK and rope(rd=0) == capi.OK and capi.last_error() == ""
+
+    app = lambda q=0x1000, k=0x2000, v=0x3000, pos=0x4000, kc=0x5000, vc=0x6000, B=1, Ln=4, Hq=4, Hkv=2, D=128, \
+        Lmax=16, s=(4096, 2048, 128), rd=64, style=0: \
+        L.minfer_rope_kv_append(capi.F16, style, q, k, v, pos, kc, vc, B, Ln, Hq, Hkv, D, Lmax, *s, rd, 1e4, None)
+    assert app(pos=0) == capi.EINVAL and "null" in capi.last_error()
+    assert app(kc=0x5008) == capi.EINVAL and "aligned" in capi.last_error()
+    assert app(s=(4096, 2048, 100)) == capi.EINVAL and "strides" in capi.last_error()
+    assert app(D=100, rd=64) == capi.EINVAL
+    assert app(rd=24, style=1) == capi.EINVAL          # NeoX halves must be whole 16-byte chunks
+    assert app(Hkv=0) == capi.EINVAL
+    assert app(B=0) == capi.OK and app(Ln=0) == capi.OK
+
+
 def test_python_surface_matches_reference_names(kerns):
     from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
     from minfer.kernels import KernelBackend, refs
@@ -88,6 +116,18 @@ def test_python_surface_matches_reference_names(kerns):
     schema = str(torch.ops.minfer.flash_attn.default._schema)
     assert schema == ("minfer::flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, "
                       "Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()")
+    # rotary embedding: names, argument order and schemas of the reference (torch_ext/ops.py:86-126, reg.cpp:25-26)
+    for name in ("il_rope", "neox_rope"):
+        assert list(inspect.signature(getattr(te, name)).parameters) == ["rotary_dim", "start_pos", "freq_base", "x"]
+        assert callable(getattr(kerns, name))
+        assert str(getattr(torch.ops.minfer, name).default._schema) == \
+            f"minfer::{name}(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()"
+    assert callable(kerns.rope_kv_append)
+    x = torch.randn(2, 5, 3, 16).half()
+    import oracle
+    for style, ref in ((0, refs.il_rope), (1, refs.neox_rope)):
+        assert ref(x, 8, 3, 1e4).dtype == torch.float16
+        assert float((ref(x, 8, 3, 1e4).float() - torch.from_numpy(oracle.rope(style, x, 8, 3, 1e4))).abs().max()) < 4e-3
     q = torch.randn(1, 2, 4, 8)
     m = torch.ones(1, 1, 4, 4, dtype=torch.bool).tril()
     assert torch.equal(refs.flash_attn(q, q, q, m), torch.nn.functional.scaled_dot_product_attention(q, q, q, attn_mask=m))
@@ -103,6 +143,14 @@ def test_no_cpu_fallback(kerns):
         kerns.flash_attn_decode(1, 1, 2, q[:, :, :1], q, q, torch.ones(1, dtype=torch.int32), torch.empty_like(q[:, :, :1]))
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.flash_attn_varlen(1, 1, 2, q, q, q, torch.tensor([0, 64], dtype=torch.int32), 64, torch.empty_like(q))
+    x = torch.zeros(1, 4, 2, 128, dtype=torch.float16)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.il_rope(64, 0, 1e4, x)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.neox_rope(64, 0, 1e4, x)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.rope_kv_append(0, 64, 1e4, x, x, x, torch.zeros(1, dtype=torch.int32), torch.zeros(1, 2, 8, 128).half(),
+                             torch.zeros(1, 2, 8, 128).half())
 
 
 def test_workload_generators_are_seeded():
@@ -118,3 +166,9 @@ def test_workload_generators_are_seeded():
     assert len(lens) == 16 and min(lens) >= 128 and max(lens) <= 2048 and q.shape == (1, 64, int(cu[-1]), 128)
     assert workloads.prefill_flops(32, 128, [4096]) == 2 * 128 * 32 * 4096 * 4097
     assert workloads.decode_bytes([10, 20], 32, 8, 128) == 30 * 4096 + 2 * 2 * 32 * 128 * 2
+    x = workloads.rope_input(seed=1, B=1, L=8)
+    assert x.shape == (1, 8, 48, 128) and torch.equal(x, workloads.rope_input(seed=1, B=1, L=8))
+    assert workloads.rope_bytes(8, 4096, 48, 64) == 2 * 8 * 4096 * 48 * 64 * 2
+    q, k, v, pos, kc, vc = workloads.kv_append(seed=0, L=16)
+    assert q.shape == (1, 16, 32, 128) and k.shape == v.shape == (1, 16, 8, 128) and kc.shape == (1, 8, 16, 128)
+    assert workloads.kv_append_bytes(1, 16, 32, 8, 128, 128) == (2 * 16 * 32 * 128 + 4 * 16 * 8 * 128) * 2
