@@ -25,8 +25,10 @@ PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
-PREFILL_TRAFFIC_BYTES = 110289 * 1024
-DECODE_TRAFFIC_BYTES = 1098181 * 1024
+PREFILL_TRAFFIC_BYTES = 107691 * 1024
+DECODE_TRAFFIC_BYTES = 1089627 * 1024
+ROPE_TRAFFIC_BYTES = 393304 * 1024          # il_rope on [8,4096,48,128], rotary 64
+APPEND_TRAFFIC_BYTES = 786577 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
 
 
 class HipEvents:
@@ -99,8 +101,9 @@ def rope_cpu_baseline(torch, workloads, refs):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--steps", type=int, default=500)
+    ap.add_argument("--warmup", type=int, default=300,
+                    help="untimed steps; the GPU needs some 15 ms of continuous work after an idle period to reach its clocks")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay one captured HIP graph per step instead of launching from Python")
     args = ap.parse_args()
@@ -158,7 +161,7 @@ def main():
         step()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    avg_ms, med_ms = ev.time_each(step, stream, max(args.steps, 20))
+    avg_ms, med_ms = ev.time_each(step, stream, min(max(args.steps, 20), 200))
     flops = workloads.prefill_flops(32, 128, [L])
     tflops = flops / (wall_ms * 1e-3) / 1e12
     achieved = flops / (avg_ms * 1e-3) / 1e12
@@ -167,10 +170,10 @@ def main():
     qd, kc, vc, ctx = workloads.decode_cache(seed=0, device=dev)
     outd = torch.zeros_like(qd)
     dstep = lambda: kerns.flash_attn_decode(qt, qb, qs, qd, kc, vc, ctx, outd)
-    for _ in range(args.warmup):
+    for _ in range(max(args.warmup, 100)):
         dstep()
     torch.cuda.synchronize()
-    d_avg_ms, d_med_ms = ev.time_each(dstep, stream, max(args.steps, 20))
+    d_avg_ms, d_med_ms = ev.time_each(dstep, stream, min(max(args.steps, 20), 100))
     dbytes = workloads.decode_bytes(ctx.tolist(), 32, 8, 128)
     d_gbs = dbytes / (d_avg_ms * 1e-3) / 1e9
     del kc, vc
@@ -178,19 +181,19 @@ def main():
     # ---- the step before attention: rotary embedding, alone and fused with the cache append ----
     x = workloads.rope_input(seed=0, device=dev)                      # the reference test's shape
     rstep = lambda: kerns.il_rope(64, 2048, 1e6, x)
-    for _ in range(3):
+    for _ in range(200):
         rstep()
     torch.cuda.synchronize()
-    r_avg_ms, r_med_ms = ev.time_each(rstep, stream, 20)
+    r_avg_ms, r_med_ms = ev.time_each(rstep, stream, 50)
     rbytes = workloads.rope_bytes(8, 4096, 48, 64)
     r_gbs = rbytes / (r_avg_ms * 1e-3) / 1e9
     del x
     aq, ak, av, apos, akc, avc = workloads.kv_append(seed=0, device=dev, B=8, L=4096)
     astep = lambda: kerns.rope_kv_append(1, 128, 5e5, aq, ak, av, apos, akc, avc)
-    for _ in range(3):
+    for _ in range(100):
         astep()
     torch.cuda.synchronize()
-    a_avg_ms, a_med_ms = ev.time_each(astep, stream, 20)
+    a_avg_ms, a_med_ms = ev.time_each(astep, stream, 50)
     abytes = workloads.kv_append_bytes(8, 4096, 32, 8, 128, 128)
     a_gbs = abytes / (a_avg_ms * 1e-3) / 1e9
     del aq, ak, av, akc, avc
@@ -216,11 +219,11 @@ def main():
     rec["rope"] = {"value": r_gbs, "unit": "GB/s", "ms": r_avg_ms, "median_ms": r_med_ms,
                    "workload": "il_rope in place, x [8,4096,48,128] fp16, rotary_dim 64, base 1e6, start_pos 2048 (reference test/kernels.py:76-96)",
                    "roofline": {"bound": "hbm", "achieved": r_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r_gbs / PEAK_HBM_GBS,
-                                "traffic": None, "kernel": "rope_kernel<F16,interleaved,in place>", "algorithmic_bytes": rbytes}}
+                                "traffic": ROPE_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,interleaved,in place>", "algorithmic_bytes": rbytes}}
     rec["rope_kv_append"] = {"value": a_gbs, "unit": "GB/s", "ms": a_avg_ms, "median_ms": a_med_ms,
                              "workload": "NeoX rope(q) in place + rope(k), v appended to the cache: B=8 L=4096 Hq=32 Hkv=8 D=128 fp16, rotary_dim 128, base 5e5",
                              "roofline": {"bound": "hbm", "achieved": a_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a_gbs / PEAK_HBM_GBS,
-                                          "traffic": None, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
+                                          "traffic": APPEND_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
         rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)
