@@ -5,7 +5,7 @@ S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmi
 (4*D*Hq*attended pairs), inputs resident in HBM, every kernel the op launches inside the timed
 region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
 under "decode" with its own HBM roofline, the rotary-embedding step that feeds attention under "rope"
-and "rope_kv_append", and the reference's CPU attention path (torch SDPA in fp32 on the host cores) under
+"rope_kv_append" and "rmsnorm", and the reference's CPU attention path (torch SDPA in fp32 on the host cores) under
 "cpu_baseline".  Prints ONE JSON line.
 """
 import argparse
@@ -197,6 +197,17 @@ def main():
     abytes = workloads.kv_append_bytes(8, 4096, 32, 8, 128, 128)
     a_gbs = abytes / (a_avg_ms * 1e-3) / 1e9
     del aq, ak, av, akc, avc
+    nshape = (8, 4096, 6144)                                          # the reference test's per-token shape
+    nx, nw = workloads.rmsnorm_input(nshape, seed=0, device=dev)
+    nout = torch.empty_like(nx)
+    nstep = lambda: kerns.rmsnorm(1e-6, nx, nw, nout)
+    for _ in range(100):
+        nstep()
+    torch.cuda.synchronize()
+    n_avg_ms, n_med_ms = ev.time_each(nstep, stream, 50)
+    nbytes = workloads.rmsnorm_bytes(nshape)
+    n_gbs = nbytes / (n_avg_ms * 1e-3) / 1e9
+    del nx, nout
 
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
@@ -224,6 +235,10 @@ def main():
                              "workload": "NeoX rope(q) in place + rope(k), v appended to the cache: B=8 L=4096 Hq=32 Hkv=8 D=128 fp16, rotary_dim 128, base 5e5",
                              "roofline": {"bound": "hbm", "achieved": a_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a_gbs / PEAK_HBM_GBS,
                                           "traffic": APPEND_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
+    rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
+                      "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
+                      "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,
+                                   "traffic": None, "kernel": "rmsnorm_rows_kernel<F16,64,16>", "algorithmic_bytes": nbytes}}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
         rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)

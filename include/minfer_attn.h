@@ -130,6 +130,17 @@ int minfer_rope_kv_append(int dtype, int style, void* q, const void* k, const vo
                           int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_row,
                           int64_t rotary_dim, double freq_base, void* stream);
 
+/*
+ * RMS normalisation: in, out are n_vectors contiguous vectors of length dim; w has dim elements;
+ *   out[v, i] = in[v, i] * w[i] / sqrt(mean_i(in[v, :]^2) + eps)      (fp32 arithmetic, one rounding)
+ * The reference's [B,L,hidden] and [B,L,n_heads,head_dim] inputs are both this with dim = |w| and
+ * n_vectors = numel / dim.  in and out may be the same buffer.  Replaces rmsnorm_cuda and its kernel
+ * (reference: rmsnorm/op.cuh:20-70, rmsnorm/kernel.cuh:11-40; oracle refs.py:4-10).  Beyond the reference:
+ * dtype may be MINFER_ATTN_BF16.
+ */
+int minfer_rmsnorm(int dtype, const void* in, const void* w, void* out, int64_t n_vectors, int64_t dim,
+                   double eps, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

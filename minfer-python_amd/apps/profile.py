@@ -106,6 +106,18 @@ def rope_kv_append(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def rmsnorm(backend: str, which: str, workload: str, repeat: int):
+    """The reference test's shapes (reference: test/kernels.py:60-63): per token [8,4096,6144] (default) or,
+    with --workload reference, per head [8,4096,48,128]."""
+    kerns = KernelBackend(backend)
+    x, w = workloads.rmsnorm_input((8, 4096, 48, 128) if workload == "reference" else (8, 4096, 6144), device="cuda")
+    out = torch.empty_like(x)
+    fn = (lambda: kerns.rmsnorm(1e-6, x, w, out)) if which == "minfer" else (lambda: refs.rmsnorm(x, w, 1e-6))
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def copy(backend: str, which: str, workload: str, repeat: int):
     """A plain device-to-device copy of 1 GiB: the known-size kernel that HBM byte counters
     (FETCH_SIZE / WRITE_SIZE) are calibrated against."""
@@ -118,7 +130,7 @@ def copy(backend: str, which: str, workload: str, repeat: int):
 
 if __name__ == "__main__":
     KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
-               "il_rope": il_rope, "rope_kv_append": rope_kv_append, "copy": copy}
+               "il_rope": il_rope, "rope_kv_append": rope_kv_append, "rmsnorm": rmsnorm, "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)

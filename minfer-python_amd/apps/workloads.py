@@ -136,3 +136,27 @@ def rope_bytes(B, L, H, rotary_dim, itemsize=2):
 def kv_append_bytes(B, L, Hq, Hkv, D, rotary_dim, itemsize=2):
     """q's rotary part read and written; k and v read once; their cache rows written once."""
     return (2 * B * L * Hq * rotary_dim + 4 * B * L * Hkv * D) * itemsize
+
+
+def rmsnorm_input(shape=(8, 4096, 6144), seed=0, device="cpu", dtype=torch.float16):
+    """x ~ N(0,1) of `shape`, w ~ N(0,1)/sqrt(shape[-1]) (reference: test/kernels.py:60-69; its two shapes are
+    (8,4096,6144) per token and (8,4096,48,128) per head)."""
+    gen = torch.Generator().manual_seed(seed)
+    w = ((1 / shape[-1] ** 0.5) * torch.randn(shape[-1], generator=gen)).to(dtype)
+    n = 1
+    for s in shape:
+        n *= s
+    x = torch.empty(shape, dtype=dtype)
+    flat = x.view(-1)
+    for lo in range(0, n, 1 << 26):          # in pieces: the fp32 staging of 2e8 elements is large
+        hi = min(n, lo + (1 << 26))
+        flat[lo:hi] = torch.randn(hi - lo, generator=gen).to(dtype)
+    return (x.to(device), w.to(device)) if device != "cpu" else (x, w)
+
+
+def rmsnorm_bytes(shape, itemsize=2):
+    """Every element read once and written once, plus the weight."""
+    n = 1
+    for s in shape:
+        n *= s
+    return (2 * n + shape[-1]) * itemsize

@@ -1,5 +1,5 @@
-// PyTorch (stable ABI) registration of the attention operators, and of the rotary-embedding step
-// that feeds them, in namespace `minfer`.
+// PyTorch (stable ABI) registration of the attention operators, and of the normalisation and
+// rotary-embedding steps that feed them, in namespace `minfer`.
 //
 // This file is the only place where torch types appear: it validates tensors exactly as the
 // reference host function does, turns them into pointers/strides and calls the C ABI of
@@ -243,10 +243,32 @@ void rope_kv_append_hip(int64_t style, int64_t rotary_dim, double freq_base,
              "rope_kv_append");
 }
 
+// Same signature, argument meaning and checks as the reference's rmsnorm_cuda
+// (reference: src/minfer/kernels/torch_ext/csrc/cuda/rmsnorm/op.cuh:20-70); bfloat16 is admitted as well.
+void rmsnorm_hip(double eps,
+                 const Tensor& in,   // [B, L, hidden] or [B, L, n_heads, head_dim]
+                 const Tensor& w,    // [dim]: the vector length that is normalised
+                 Tensor& out) {      // same shape as in
+    STD_TORCH_CHECK(on_gpu(in) && on_gpu(w) && on_gpu(out), "rmsnorm: all tensors must be on the GPU");
+    STD_TORCH_CHECK(in.is_contiguous() && out.is_contiguous() && w.is_contiguous(), "rmsnorm: tensors must be contiguous");
+    const ScalarType t = in.scalar_type();
+    STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, "rmsnorm: input must be float16 or bfloat16");
+    STD_TORCH_CHECK(out.scalar_type() == t && w.scalar_type() == t, "rmsnorm: input, w and out must share one dtype");
+    STD_TORCH_CHECK(in.dim() == 3 || in.dim() == 4, "rmsnorm: input must be 3-D or 4-D");
+    STD_TORCH_CHECK(in.sizes().equals(out.sizes()), "rmsnorm: input and out shapes differ");
+    STD_TORCH_CHECK(w.dim() == 1 && w.size(0) > 0 && (in.size(-1) == w.size(0) || in.size(-1) % w.size(0) == 0),
+                    "rmsnorm: the last dimension must be a multiple of the weight length");
+    const int64_t dim = w.size(0);
+    check_rc(minfer_rmsnorm(t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16, in.const_data_ptr(), w.const_data_ptr(),
+                            out.mutable_data_ptr(), in.numel() / dim, dim, eps, current_stream()),
+             "rmsnorm");
+}
+
 STABLE_TORCH_LIBRARY(minfer, m) {
     // verbatim the reference's schema (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:30)
     m.def("flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()");
-    // verbatim the reference's schemas (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:25-26)
+    // verbatim the reference's schemas (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:24-26)
+    m.def("rmsnorm(float eps, Tensor input, Tensor w, Tensor(a!) out) -> ()");
     m.def("il_rope(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()");
     m.def("neox_rope(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()");
     // extensions in the same style: ints first, inputs, out-parameter last, no return value
@@ -259,6 +281,7 @@ STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-ke
     m.impl("flash_attn", TORCH_BOX(&flash_attn_hip));
     m.impl("flash_attn_decode", TORCH_BOX(&flash_attn_decode_hip));
     m.impl("flash_attn_varlen", TORCH_BOX(&flash_attn_varlen_hip));
+    m.impl("rmsnorm", TORCH_BOX(&rmsnorm_hip));
     m.impl("il_rope", TORCH_BOX(&il_rope_hip));
     m.impl("neox_rope", TORCH_BOX(&neox_rope_hip));
     m.impl("rope_kv_append", TORCH_BOX(&rope_kv_append_hip));

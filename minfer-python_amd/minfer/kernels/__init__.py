@@ -1,13 +1,14 @@
 """Kernel facade, same shape as the reference's (reference: src/minfer/kernels/__init__.py:2-18):
-an attribute bag of callables for one backend.  Only the attention path and the rotary-embedding
-step that feeds it live here."""
+an attribute bag of callables for one backend.  Only the attention path and the normalisation and
+rotary-embedding steps that feed it live here."""
 
 
 class KernelBackend:
     def __init__(self, backend: str):
         if backend == "torch_ext":
             from .torch_ext import (flash_attn, flash_attn_decode, flash_attn_varlen, il_rope, neox_rope,
-                                    rope_kv_append)
+                                    rmsnorm, rope_kv_append)
+            self.rmsnorm = rmsnorm
             self.il_rope = il_rope
             self.neox_rope = neox_rope
             self.rope_kv_append = rope_kv_append

@@ -5,6 +5,11 @@ import torch
 import torch.nn.functional as F
 
 
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    """x: (B, L, n_heads, head_dim) (per head) or (B, L, hidden) (per vector); normalised over the last dimension."""
+    return F.rms_norm(x, (x.shape[-1],), weight=weight, eps=eps)
+
+
 def flash_attn(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
     """SDPA with a bool mask (True = attend).  Q/K/V: (B, n_heads, L, head_dim); K/V must already be
     expanded to n_heads for GQA (``repeat_interleave(n_rep, dim=1)``)."""

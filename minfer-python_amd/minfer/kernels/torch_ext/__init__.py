@@ -9,4 +9,4 @@ except ImportError as e:  # pragma: no cover
         "(hipcc, gfx950) first"
     ) from e
 from .ops import (flash_attn, flash_attn_decode, flash_attn_varlen, il_rope, neox_rope,  # noqa: E402,F401
-                  rope_kv_append)
+                  rmsnorm, rope_kv_append)

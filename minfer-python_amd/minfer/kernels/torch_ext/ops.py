@@ -1,6 +1,6 @@
 """Python wrappers and fake (meta) kernels of the attention ops and of the rotary-embedding step
 before them, mirroring the reference's wrapper layer (reference:
-src/minfer/kernels/torch_ext/ops.py:86-126, 234-266): positional pass-through
+src/minfer/kernels/torch_ext/ops.py:60-126, 234-266): positional pass-through
 to ``torch.ops.minfer.<op>.default``; the result is written into ``out``."""
 import torch
 
@@ -135,3 +135,19 @@ def _(style, rotary_dim, freq_base, q, k, v, positions, k_cache, v_cache):
     torch._check(q.device.type == "cuda")
     torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and k_cache.dim() == 4 and v_cache.dim() == 4)
     torch._check(rotary_dim <= q.size(3))
+
+
+def rmsnorm(eps: float, input: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
+    """RMS normalisation over vectors of length len(w) (the whole hidden dimension, or per head)."""
+    return torch.ops.minfer.rmsnorm.default(eps, input, w, out)
+
+
+@torch.library.register_fake("minfer::rmsnorm")
+def _(eps, input, w, out):
+    torch._check(input.dtype in _ACT_DTYPES)
+    torch._check(w.dtype == input.dtype and out.dtype == input.dtype)
+    torch._check(input.device == w.device == out.device)
+    torch._check(input.device.type == "cuda")
+    torch._check(input.shape == out.shape)
+    torch._check(input.dim() in (3, 4))
+    torch._check(input.size(-1) == w.size(0) or input.size(-1) % w.size(0) == 0)

@@ -1,4 +1,4 @@
-"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c and rope_oracle.c.
+"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c, rope_oracle.c and rmsnorm_oracle.c.
 
 Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py may import this
 package.  The shipped operator never does: it launches HIP kernels or raises.
@@ -22,7 +22,7 @@ class _Strides(ctypes.Structure):
 
 
 def build(force=False):
-    """Compile attn_oracle.c and rope_oracle.c into liboracle.so (gcc + OpenMP)."""
+    """Compile the oracle's C files into liboracle.so (gcc + OpenMP)."""
     so = os.path.join(_HERE, "liboracle.so")
     if force and os.path.exists(so):
         os.remove(so)
@@ -38,7 +38,7 @@ def lib():
             build()
         _LIB = ctypes.CDLL(so)
         for name in ("oracle_flash_attn", "oracle_flash_attn_rows", "oracle_flash_attn_decode",
-                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append"):
+                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append", "oracle_rmsnorm"):
             getattr(_LIB, name).restype = ctypes.c_int
     return _LIB
 
@@ -165,3 +165,15 @@ def rope_kv_append(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq
     if rc != 0:
         raise ValueError(f"oracle_rope_kv_append rc={rc}")
     return q, k_cache, v_cache
+
+
+def rmsnorm(x, w, eps):
+    """x * w / sqrt(mean(x^2 over vectors of len(w)) + eps) (reference: refs.py:4-10, rmsnorm/kernel.cuh:24-38),
+    fp64 arithmetic; returns a new float32 array of x's shape, unrounded."""
+    x, w = _f32(x), _f32(w)
+    dim = w.shape[0]
+    out = np.empty_like(x)
+    rc = lib().oracle_rmsnorm(_ptr(x), _ptr(w), _ptr(out), ctypes.c_int64(x.size // dim), ctypes.c_int64(dim), ctypes.c_double(eps))
+    if rc != 0:
+        raise ValueError(f"oracle_rmsnorm rc={rc}")
+    return out

@@ -47,6 +47,8 @@ def lib():
         L.minfer_rope_kv_append.restype = ctypes.c_int
         L.minfer_rope_kv_append.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
                                             i64, i64, i64, i64, i64, dbl, vp]
+        L.minfer_rmsnorm.restype = ctypes.c_int
+        L.minfer_rmsnorm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, dbl, vp]
         _lib = L
     return _lib
 
@@ -117,3 +119,9 @@ def rope_kv_append(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq
                                        positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), B, L, Hq,
                                        k.shape[2], D, k_cache.shape[2], k_cache.stride(0), k_cache.stride(1),
                                        k_cache.stride(2), rotary_dim, freq_base, _stream())
+
+
+def rmsnorm(x, w, out, eps):
+    """RMS normalisation of contiguous x over vectors of length len(w), into out."""
+    dim = w.shape[0]
+    return lib().minfer_rmsnorm(_dtype_code(x), x.data_ptr(), w.data_ptr(), out.data_ptr(), x.numel() // dim, dim, eps, _stream())

@@ -10,7 +10,8 @@ the fp16 output format itself does not eat the 2e-3 tolerance) and stored as fp1
 fp16 kernels see exactly the values the expected output was computed from.
 
 The rotary-embedding fixture (rope_small.npz) pins the reference's torch formulation of both styles
-(reference src/minfer/kernels/refs.py:12-47) in float64 on seeded fp16-representable inputs.
+(reference src/minfer/kernels/refs.py:12-47) in float64 on seeded fp16-representable inputs, and
+rmsnorm_small.npz the reference's F.rms_norm call (refs.py:10) in float64.
 
 Run:  python tests/golden/make_golden.py
 """
@@ -98,6 +99,17 @@ def make_rope(name, B, L, H, D, rotary_dim, start_pos, freq_base, seed):
                         y_neox=y_neox.numpy().astype(np.float32))
 
 
+def make_rmsnorm(name, shape, eps, seed):
+    """Expected values from the reference's oracle call, F.rms_norm over the last dimension (reference
+    src/minfer/kernels/refs.py:10), evaluated in float64."""
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(*shape, generator=g).half().double()
+    w = ((1 / shape[-1] ** 0.5) * torch.randn(shape[-1], generator=g)).half().double()
+    y = F.rms_norm(x, (shape[-1],), weight=w, eps=eps)
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), x=x.numpy().astype(np.float16), w=w.numpy().astype(np.float16),
+                        eps=eps, y=y.numpy().astype(np.float32))
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
     make("dense_causal_b1_h4_kv2_l16_d64", 1, 4, 2, 16, 64, "causal", 1)
@@ -106,4 +118,5 @@ if __name__ == "__main__":
     make_decode("decode_b3_h8_kv2_l50_d128", 3, 8, 2, 50, 128, 4)
     make_varlen("varlen_h4_kv2_d64", 4, 2, 64, [5, 1, 33, 70], 5)
     make_rope("rope_small", 2, 9, 3, 64, 32, 2048, 1e6, 6)
+    make_rmsnorm("rmsnorm_small", (2, 5, 3, 40), 1e-6, 7)
     print("golden vectors written to", HERE)

@@ -102,10 +102,23 @@ def test_rope_validation_rejects_before_launch():
     assert app(B=0) == capi.OK and app(Ln=0) == capi.OK
 
 
+def test_rmsnorm_validation_rejects_before_launch():
+    L = capi.lib()
+    norm = lambda dtype=capi.F16, x=0x1000, w=0x2000, out=0x3000, n=4, dim=128, eps=1e-6: \
+        L.minfer_rmsnorm(dtype, x, w, out, n, dim, eps, None)
+    assert norm(dtype=3) == capi.EINVAL and "dtype" in capi.last_error()
+    assert norm(dim=0) == capi.EINVAL
+    assert norm(n=-1) == capi.EINVAL
+    assert norm(eps=-1.0) == capi.EINVAL and "eps" in capi.last_error()
+    assert norm(w=0) == capi.EINVAL and "null" in capi.last_error()
+    assert norm(n=0) == capi.OK and capi.last_error() == ""
+
+
 def test_python_surface_matches_reference_names(kerns):
     from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
     from minfer.kernels import KernelBackend, refs
     import minfer.kernels.torch_ext as te
+    import oracle
 
     assert GGMLQuantizationType.F16 == 1 and GGML_QUANT_SIZES[GGMLQuantizationType.F16] == (1, 2)
     assert list(inspect.signature(te.flash_attn).parameters) == [
@@ -123,8 +136,11 @@ def test_python_surface_matches_reference_names(kerns):
         assert str(getattr(torch.ops.minfer, name).default._schema) == \
             f"minfer::{name}(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()"
     assert callable(kerns.rope_kv_append)
+    assert list(inspect.signature(te.rmsnorm).parameters) == ["eps", "input", "w", "out"] and callable(kerns.rmsnorm)
+    assert str(torch.ops.minfer.rmsnorm.default._schema) == "minfer::rmsnorm(float eps, Tensor input, Tensor w, Tensor(a!) out) -> ()"
+    xn, wn = torch.randn(2, 3, 16), torch.randn(16)
+    assert float((refs.rmsnorm(xn, wn, 1e-6) - torch.from_numpy(oracle.rmsnorm(xn, wn, 1e-6))).abs().max()) < 1e-5
     x = torch.randn(2, 5, 3, 16).half()
-    import oracle
     for style, ref in ((0, refs.il_rope), (1, refs.neox_rope)):
         assert ref(x, 8, 3, 1e4).dtype == torch.float16
         assert float((ref(x, 8, 3, 1e4).float() - torch.from_numpy(oracle.rope(style, x, 8, 3, 1e4))).abs().max()) < 4e-3
@@ -144,6 +160,8 @@ def test_no_cpu_fallback(kerns):
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.flash_attn_varlen(1, 1, 2, q, q, q, torch.tensor([0, 64], dtype=torch.int32), 64, torch.empty_like(q))
     x = torch.zeros(1, 4, 2, 128, dtype=torch.float16)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.rmsnorm(1e-6, x, torch.ones(128, dtype=torch.float16), torch.empty_like(x))
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.il_rope(64, 0, 1e4, x)
     with pytest.raises((NotImplementedError, RuntimeError)):
@@ -166,6 +184,9 @@ def test_workload_generators_are_seeded():
     assert len(lens) == 16 and min(lens) >= 128 and max(lens) <= 2048 and q.shape == (1, 64, int(cu[-1]), 128)
     assert workloads.prefill_flops(32, 128, [4096]) == 2 * 128 * 32 * 4096 * 4097
     assert workloads.decode_bytes([10, 20], 32, 8, 128) == 30 * 4096 + 2 * 2 * 32 * 128 * 2
+    xs, ws = workloads.rmsnorm_input((2, 3, 64), seed=5)
+    assert xs.shape == (2, 3, 64) and ws.shape == (64,) and torch.equal(xs, workloads.rmsnorm_input((2, 3, 64), seed=5)[0])
+    assert workloads.rmsnorm_bytes((2, 3, 64)) == (2 * 384 + 64) * 2
     x = workloads.rope_input(seed=1, B=1, L=8)
     assert x.shape == (1, 8, 48, 128) and torch.equal(x, workloads.rope_input(seed=1, B=1, L=8))
     assert workloads.rope_bytes(8, 4096, 48, 64) == 2 * 8 * 4096 * 48 * 64 * 2
