@@ -5,7 +5,7 @@ S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmi
 (4*D*Hq*attended pairs), inputs resident in HBM, every kernel the op launches inside the timed
 region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
 under "decode" with its own HBM roofline, the rotary-embedding step that feeds attention under "rope"
-"rope_kv_append" and "rmsnorm", and the reference's CPU attention path (torch SDPA in fp32 on the host cores) under
+"rope_kv_append", "rmsnorm" and "gemm", and the reference's CPU attention path (torch SDPA in fp32 on the host cores) under
 "cpu_baseline".  Prints ONE JSON line.
 """
 import argparse
@@ -208,6 +208,17 @@ def main():
     nbytes = workloads.rmsnorm_bytes(nshape)
     n_gbs = nbytes / (n_avg_ms * 1e-3) / 1e9
     del nx, nout
+    # ---- projection GEMM: the reference's published HGEMM size, and its QKV projection shape ---------
+    ga, gw, gbias = workloads.gemm_input(4096, 4096, 4096, seed=0, device=dev)
+    gout = torch.empty_like(gbias)
+    gstep = lambda: kerns.gemm(qt, qb, qs, 1.0, 0.0, ga, gw, gbias, gout)
+    for _ in range(100):
+        gstep()
+    torch.cuda.synchronize()
+    g_avg_ms, g_med_ms = ev.time_each(gstep, stream, 50)
+    gflops = workloads.gemm_flops(4096, 4096, 4096)
+    g_tf = gflops / (g_avg_ms * 1e-3) / 1e12
+    del ga, gw, gbias, gout
 
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
@@ -239,6 +250,11 @@ def main():
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,
                                    "traffic": None, "kernel": "rmsnorm_rows_kernel<F16,64,16>", "algorithmic_bytes": nbytes}}
+    rec["gemm"] = {"value": g_tf, "unit": "TFLOP/s", "ms": g_avg_ms, "median_ms": g_med_ms,
+                   "workload": "gemm alpha=1 beta=0, A [1,4096,4096] x W [4096,4096] fp16 (reference README HGEMM table, M=K=N=4096)",
+                   "published_reference_us": 605.3,
+                   "roofline": {"bound": "mfma", "achieved": g_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": g_tf / PEAK_MFMA_TFLOPS,
+                                "traffic": None, "kernel": "gemm_kernel<F16,[K,N],256x256>", "algorithmic_flops": gflops}}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
         rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)

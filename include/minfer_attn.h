@@ -141,6 +141,22 @@ int minfer_rope_kv_append(int dtype, int style, void* q, const void* k, const vo
 int minfer_rmsnorm(int dtype, const void* in, const void* w, void* out, int64_t n_vectors, int64_t dim,
                    double eps, void* stream);
 
+/* Layout of the weight operand of minfer_gemm. */
+#define MINFER_GEMM_B_KN 0   /* B is [K, N]: D = alpha * A B + beta * C     (reference: dispatch_f16_ab)  */
+#define MINFER_GEMM_B_NK 1   /* B is [N, K]: D = alpha * A B^T + beta * C   (reference: dispatch_f16_abt, empty there) */
+
+/*
+ * D[M,N] = alpha * A[M,K] x B + beta * C[M,N], 16-bit operands, fp32 accumulation, one rounding.  lda..ldd
+ * are row strides in elements (ldb: of B as stored).  C may be null when beta == 0 and may alias D.
+ * Replaces gemm_cuda's F16 paths and their kernels (reference: gemm/op.cuh:218-316, gemm/kernels/gemm_f16.cuh;
+ * oracle refs.py:49-51), and is what the QKV projection runs on (reference: qkv/op.cuh, a stub).  The tiled
+ * MFMA kernel needs K % 64 == 0, N % 8 == 0, 16-byte aligned A and B with strides that are multiples of 8 and
+ * 8-byte aligned C and D with strides that are multiples of 4; anything else runs a plain kernel.
+ */
+int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
+                int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                double alpha, double beta, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -118,6 +118,17 @@ def rmsnorm(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def gemm(backend: str, which: str, workload: str, repeat: int):
+    """M=K=N=4096, alpha 1, beta 0: a size of the reference's published HGEMM table (reference: README.md:84-109)."""
+    kerns = KernelBackend(backend)
+    a, w, bias = workloads.gemm_input(4096, 4096, 4096, device="cuda")
+    out = torch.empty_like(bias)
+    fn = (lambda: kerns.gemm(QT, QB, QS, 1.0, 0.0, a, w, bias, out)) if which == "minfer" else (lambda: refs.gemm(a[0], w, bias[0], out[0], 1.0, 0.0))
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def copy(backend: str, which: str, workload: str, repeat: int):
     """A plain device-to-device copy of 1 GiB: the known-size kernel that HBM byte counters
     (FETCH_SIZE / WRITE_SIZE) are calibrated against."""
@@ -130,7 +141,7 @@ def copy(backend: str, which: str, workload: str, repeat: int):
 
 if __name__ == "__main__":
     KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
-               "il_rope": il_rope, "rope_kv_append": rope_kv_append, "rmsnorm": rmsnorm, "copy": copy}
+               "il_rope": il_rope, "rope_kv_append": rope_kv_append, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)

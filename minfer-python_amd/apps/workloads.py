@@ -160,3 +160,17 @@ def rmsnorm_bytes(shape, itemsize=2):
     for s in shape:
         n *= s
     return (2 * n + shape[-1]) * itemsize
+
+
+def gemm_input(M, N, K, seed=0, device="cpu", dtype=torch.float16):
+    """The reference test's recipe (reference: test/kernels.py:133-136): A [1,M,K] ~ N(0,1), weight [K,N] ~
+    N(0,1)/sqrt(K), bias [1,M,N] ~ N(0,1)."""
+    gen = torch.Generator().manual_seed(seed)
+    a = torch.randn(1, M, K, generator=gen).to(dtype)
+    w = ((1 / K ** 0.5) * torch.randn(K, N, generator=gen)).to(dtype)
+    bias = torch.randn(1, M, N, generator=gen).to(dtype)
+    return (a.to(device), w.to(device), bias.to(device)) if device != "cpu" else (a, w, bias)
+
+
+def gemm_flops(M, N, K):
+    return 2 * M * N * K

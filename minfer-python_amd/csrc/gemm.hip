@@ -1,0 +1,283 @@
+// Half-precision GEMM for gfx950: D = alpha * A x B + beta * C with fp32 accumulation on the MFMA units.
+//
+// What the reference computes (reference: src/minfer/kernels/torch_ext/csrc/cuda/gemm/op.cuh:218-316,
+// oracle src/minfer/kernels/refs.py:49-51, tests test/kernels.py:119-216): A is [M, K] activations (leading
+// dims flattened), B is the weight either as [K, N] ("A x B", what its tuned kernel handles) or as [N, K]
+// ("A x B^T", the layout of its QKV projection, whose launcher is empty in the reference), C and D are [M, N].
+//
+// Design.  A workgroup (8 waves, two per SIMD) owns a 256 x 256 tile of D (128 x 128 with 4 waves for problems
+// too small to fill the chip with large tiles) and walks K in steps of 64; the A and B panels of a step (32 KB
+// each) are copied global->LDS without passing through registers, double-buffered, one barrier per step.
+// Every wave owns 128 (64) rows (m) x 64 columns (n) as 4 (2) x 2 accumulator blocks of 32x32
+// and computes the transposed product D^T = B^T A^T, so that a lane ends up with 4 consecutive n of one row m
+// and the epilogue stores 8 bytes per register quadruple: B supplies the MFMA A operand (for the [K, N] layout
+// through LDS transpose reads, the same way the attention kernel reads V^T; for [N, K] through plain 16-byte
+// reads) and A supplies the B operand (16-byte reads).  LDS panels are split into sub-tiles whose geometry
+// and XOR swizzles are those of the attention kernel's K and V tiles, so both read patterns are free of bank
+// conflicts.  Workgroup ids are dealt so that one XCD works on consecutive tiles of a tile row (they share the
+// A panel in that XCD's L2).
+#include <algorithm>
+
+#include "attn_common.h"
+#include "attn_host.h"
+
+namespace minfer_attn {
+
+constexpr int kBK = 64;
+// Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
+// 128 x 128 otherwise.  A wave owns 32*MB rows x 64 columns.
+template <int MB_, int WAVES_N_> struct GemmShape {
+    static constexpr int MB = MB_, WAVES_M = 2, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N;
+    static constexpr int BM = 32 * MB * WAVES_M, BN = 64 * WAVES_N;
+    static constexpr int A_PANEL = BM * 128, B_PANEL = BN * 128;   // bytes of one K step
+};
+using GemmBig = GemmShape<4, 4>;
+using GemmSmall = GemmShape<2, 2>;
+constexpr int kRowTile = 8192;              // sub-tile [64 rows][64 k], 128-byte rows (A, and B as [N, K])
+constexpr int kColTile = 16384;             // sub-tile [64 k][128 n], 256-byte rows (B as [K, N])
+
+struct GemmParams {
+    const void* A; const void* B; const void* C; void* D;
+    int M, N, K;
+    int64_t lda, ldb, ldc, ldd;   // row strides in elements
+    float alpha, beta;
+    int tiles_m, tiles_n, per_xcd;
+};
+
+// swizzles: granule index of a row XORed with a function of the row (see the attention kernel's TileGeom)
+MA_DEV int swz_row_tile(int row) { return (row >> 1) & 7; }        // 128-byte rows, read 32 rows x 16 bytes
+MA_DEV int swz_col_tile(int row) { return (row & 3) << 2; }        // 256-byte rows, read 4 rows x 64 bytes (transposing)
+
+template <class T, bool NT, class SH>
+__global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParams p) {
+    constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB;
+    __shared__ __attribute__((aligned(1024))) char a_lds[2][SH::A_PANEL];
+    __shared__ __attribute__((aligned(1024))) char b_lds[2][SH::B_PANEL];
+
+    const int lane = threadIdx.x & 63, w = wave_id();
+    const int h = lane >> 5, l32 = lane & 31;
+    const int wm = w & 1, wn = w >> 1;   // wave's place in the tile: rows 32*MB*wm .., columns 64*wn ..
+
+    // ---- which tile ----------------------------------------------------------------------------------
+    const int t = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
+    if (t >= p.tiles_m * p.tiles_n) return;
+    const int m0 = (t / p.tiles_n) * kBM, n0 = (t % p.tiles_n) * kBN;
+    const bool full_m = m0 + kBM <= p.M, full_n = n0 + kBN <= p.N;
+
+    const short* Ag = (const short*)p.A;
+    const short* Bg = (const short*)p.B;
+
+    // ---- global -> LDS copies: lane offsets (bytes) from the panel's first element ---------------------
+    // Every wave issues 4 wave-wide copies (1 KB each) per panel and K step; copy q = j*NW + w of a panel covers
+    //   A (and B as [N, K]): rows 8*(q%8) .. +7 of sub-tile q/8 (64 rows of 128 bytes each);
+    //   B as [K, N]:         k rows 4*(q%16) .. +3 of sub-tile q/16 (64 k rows of 256 bytes, 128 columns).
+    uint32_t a_off[4], b_off[4];
+    int a_dst[4], b_dst[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int q = j * NW + w;
+        {
+            const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
+            const int m = min(m0 + 64 * sub + row, p.M - 1) - m0;
+            a_off[j] = (uint32_t)((int64_t)m * p.lda + 8 * (pg ^ swz_row_tile(row))) * 2u;
+            a_dst[j] = sub * kRowTile + 8 * (q & 7) * 128;
+        }
+        if (NT) {
+            const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
+            const int n = min(n0 + 64 * sub + row, p.N - 1) - n0;
+            b_off[j] = (uint32_t)((int64_t)n * p.ldb + 8 * (pg ^ swz_row_tile(row))) * 2u;
+            b_dst[j] = sub * kRowTile + 8 * (q & 7) * 128;
+        } else {
+            const int sub = q >> 4, row = 4 * (q & 15) + (lane >> 4), pg = lane & 15;
+            const int col = min(n0 + 128 * sub + 8 * (pg ^ swz_col_tile(row)), p.N - 8) - n0;
+            b_off[j] = (uint32_t)((int64_t)row * p.ldb + col) * 2u;
+            b_dst[j] = sub * kColTile + 4 * (q & 15) * 256;
+        }
+    }
+    (void)full_m; (void)full_n;
+    auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
+        const short* abase = Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK;
+        const short* bbase = NT ? Bg + (int64_t)n0 * p.ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * p.ldb + n0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            copy16_global_to_lds(abase, a_off[j], &a_lds[stage][a_dst[j]]);
+            copy16_global_to_lds(bbase, b_off[j], &b_lds[stage][b_dst[j]]);
+        }
+    };
+
+    // ---- per-lane LDS read addresses (stage 0; stage, sub-tile and block offsets are immediates) ---------
+    // m fragments (MFMA B operand): tile row 32*MB*wm + 32*mb + l32, i.e. row 32*(mb&1) + l32 of sub-tile
+    // MB*wm/2 + (mb>>1), granule (2kk + h) ^ swizzle
+    uint32_t m_rd[4], n_rd[4];
+    {
+        const int sw = swz_row_tile(l32);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            const uint32_t o = l32 * 128 + 16 * ((2 * kk + h) ^ sw);
+            m_rd[kk] = lds_addr(&a_lds[0][0]) + (MB / 2) * wm * kRowTile + o;
+            if (NT) n_rd[kk] = lds_addr(&b_lds[0][0]) + wn * kRowTile + o;    // n fragments: row 32*nb + l32 of sub-tile wn
+        }
+        if (!NT) {
+            // n fragments through transpose reads of the [k][n] sub-tile wn>>1: per 16-lane group 4 k rows x 16 columns
+            const int blk = lane >> 4, li = lane & 15;
+            const int krow = 8 * h + (li >> 2);   // lane half h contracts k = 16kk + 8h + 0..7, like the 16-byte reads of A
+            const int swv = swz_col_tile(krow);
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) {
+                const int col = 32 * (2 * (wn & 1) + nb) + 16 * (blk & 1) + 4 * (li & 3);
+                n_rd[nb] = lds_addr(&b_lds[0][0]) + (wn >> 1) * kColTile + krow * 256 + 16 * ((col >> 3) ^ swv) + 2 * (col & 7);
+            }
+            n_rd[2] = n_rd[3] = 0;
+        }
+    }
+
+    f32x16 acc[2][MB];
+#pragma unroll
+    for (int nb = 0; nb < 2; ++nb)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.f;
+
+    auto load_frags = [&](auto stage_tag, int kk, s16x8 (&nf)[2], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
+        constexpr int AOFF = decltype(stage_tag)::value * SH::A_PANEL, BOFF = decltype(stage_tag)::value * SH::B_PANEL;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+            if (NT) {
+                nf[nb] = lds_read_b128(n_rd[kk], BOFF + 32 * nb * 128);
+            } else {
+                const s16x4 t0 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk) * 256);
+                const s16x4 t1 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk + 4) * 256);
+                nf[nb] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+            }
+        }
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) mf[mb] = lds_read_b128(m_rd[kk], AOFF + (mb >> 1) * kRowTile + 32 * (mb & 1) * 128);
+    };
+    auto compute = [&](auto stage_tag) __attribute__((always_inline)) {
+        s16x8 nf[2][2], mf[2][MB];
+        load_frags(stage_tag, 0, nf[0], mf[0]);
+#pragma unroll
+        for (int kk = 0; kk < 4; ++kk) {
+            if (kk + 1 < 4) load_frags(stage_tag, kk + 1, nf[(kk + 1) & 1], mf[(kk + 1) & 1]);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+                for (int nb = 0; nb < 2; ++nb) acc[nb][mb] = T::mfma32(nf[kk & 1][nb], mf[kk & 1][mb], acc[nb][mb]);
+        }
+    };
+
+    // ---- main loop: one barrier per K step; the copy of step t+1 is issued right after the barrier that opens
+    // step t, into the stage step t-1 has just vacated --------------------------------------------------
+    const int KT = p.K / kBK;
+    issue(0, 0);
+    for (int kt = 0; kt < KT; kt += 2) {
+        wait_vmcnt<0>();
+        __syncthreads();
+        if (kt + 1 < KT) issue(kt + 1, 1);
+        compute(std::integral_constant<int, 0>{});
+        if (kt + 1 < KT) {
+            wait_vmcnt<0>();
+            __syncthreads();
+            if (kt + 2 < KT) issue(kt + 2, 0);
+            compute(std::integral_constant<int, 1>{});
+        }
+    }
+
+    // ---- epilogue: D = alpha * acc + beta * C; register r of a block is n = 8(r/4) + 4h + r%4, m = l32 ----
+    const short* Cg = (const short*)p.C;
+    short* Dg = (short*)p.D;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = m0 + 32 * MB * wm + 32 * mb + l32;
+        if (m >= p.M) continue;
+#pragma unroll
+        for (int nb = 0; nb < 2; ++nb) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int n = n0 + 64 * wn + 32 * nb + 8 * j + 4 * h;
+                if (n >= p.N) continue;
+                float v[4];
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[nb][mb][4 * j + e];
+                if (p.beta != 0.f) {
+                    const s16x4 c = *reinterpret_cast<const s16x4*>(Cg + (int64_t)m * p.ldc + n);
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+                }
+                uint2 pk;
+                pk.x = T::pack2(v[0], v[1]);
+                pk.y = T::pack2(v[2], v[3]);
+                *reinterpret_cast<uint2*>(Dg + (int64_t)m * p.ldd + n) = pk;
+            }
+        }
+    }
+}
+
+// Any shape and alignment: one thread per element of D, fp32 accumulation.  Small or odd problems only.
+template <class T, bool NT>
+__global__ __launch_bounds__(256) void gemm_plain_kernel(const GemmParams p) {
+    const int64_t total = (int64_t)p.M * p.N;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int m = (int)(i / p.N), n = (int)(i % p.N);
+        const short* a = (const short*)p.A + (int64_t)m * p.lda;
+        const short* b = (const short*)p.B + (NT ? (int64_t)n * p.ldb : (int64_t)n);
+        float s = 0.f;
+        for (int k = 0; k < p.K; ++k) s += T::to_float(a[k]) * T::to_float(b[NT ? k : (int64_t)k * p.ldb]);
+        float v = p.alpha * s;
+        if (p.beta != 0.f) v += p.beta * T::to_float(((const short*)p.C)[(int64_t)m * p.ldc + n]);
+        ((short*)p.D)[(int64_t)m * p.ldd + n] = (short)(T::pack2(v, 0.f) & 0xffffu);
+    }
+}
+
+template <class T, bool NT, class SH>
+static int launch_tiled(GemmParams& p, hipStream_t stream) {
+    p.tiles_m = (p.M + SH::BM - 1) / SH::BM;
+    p.tiles_n = (p.N + SH::BN - 1) / SH::BN;
+    p.per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+    hipLaunchKernelGGL((gemm_kernel<T, NT, SH>), dim3(p.per_xcd * 8), dim3(SH::WAVES * 64), 0, stream, p);
+    return check_launch("gemm_kernel");
+}
+
+template <class T, bool NT>
+static int launch_gemm(GemmParams& p, bool fast, hipStream_t stream) {
+    if (fast) {
+        // large tiles halve the LDS and L2 traffic per flop; they are worth it once they fill most of the chip
+        const int64_t big_tiles = (int64_t)((p.M + GemmBig::BM - 1) / GemmBig::BM) * ((p.N + GemmBig::BN - 1) / GemmBig::BN);
+        return big_tiles >= 160 ? launch_tiled<T, NT, GemmBig>(p, stream) : launch_tiled<T, NT, GemmSmall>(p, stream);
+    }
+    const int grid = (int)std::min<int64_t>(((int64_t)p.M * p.N + 255) / 256, 256 * 16);
+    hipLaunchKernelGGL((gemm_plain_kernel<T, NT>), dim3(grid), dim3(256), 0, stream, p);
+    return check_launch("gemm_plain_kernel");
+}
+
+}  // namespace minfer_attn
+
+using namespace minfer_attn;
+
+MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
+                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                                   double alpha, double beta, void* stream_v) {
+    clear_error();
+    if (dtype != MINFER_ATTN_F16 && dtype != MINFER_ATTN_BF16)
+        return fail(MINFER_ATTN_EINVAL, "gemm: dtype must be MINFER_ATTN_F16 or MINFER_ATTN_BF16");
+    if (b_layout != MINFER_GEMM_B_KN && b_layout != MINFER_GEMM_B_NK)
+        return fail(MINFER_ATTN_EINVAL, "gemm: b_layout must be MINFER_GEMM_B_KN or MINFER_GEMM_B_NK");
+    if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
+        return fail(MINFER_ATTN_EINVAL, "gemm: bad M, N or K");
+    if (!A || !B || !D || (beta != 0.0 && !C)) return fail(MINFER_ATTN_EINVAL, "gemm: null pointer");
+    const bool nt = b_layout == MINFER_GEMM_B_NK;
+    if (lda < K || ldd < N || (beta != 0.0 && ldc < N) || ldb < (nt ? K : N))
+        return fail(MINFER_ATTN_EINVAL, "gemm: a leading dimension is smaller than its row");
+    if (M == 0 || N == 0) return MINFER_ATTN_OK;
+    GemmParams p{};
+    p.A = A; p.B = B; p.C = C; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
+    p.lda = lda; p.ldb = ldb; p.ldc = ldc; p.ldd = ldd; p.alpha = (float)alpha; p.beta = (float)beta;
+    // the tiled kernel moves 16-byte pieces and whole 64-wide K steps, and addresses a panel with 32-bit offsets
+    const bool fast = K > 0 && K % kBK == 0 && N % 8 == 0 && lda % 8 == 0 && ldb % 8 == 0 && ldc % 4 == 0 && ldd % 4 == 0 &&
+                      aligned16(A) && aligned16(B) && ((uintptr_t)D & 7u) == 0 && ((uintptr_t)C & 7u) == 0 &&
+                      (int64_t)GemmBig::BM * lda < (1LL << 30) && (int64_t)std::max<int64_t>(GemmBig::BN, kBK) * ldb < (1LL << 30);
+    hipStream_t stream = (hipStream_t)stream_v;
+    if (dtype == MINFER_ATTN_F16) return nt ? launch_gemm<F16, true>(p, fast, stream) : launch_gemm<F16, false>(p, fast, stream);
+    return nt ? launch_gemm<BF16, true>(p, fast, stream) : launch_gemm<BF16, false>(p, fast, stream);
+}

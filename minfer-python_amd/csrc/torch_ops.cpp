@@ -1,5 +1,5 @@
-// PyTorch (stable ABI) registration of the attention operators, and of the normalisation and
-// rotary-embedding steps that feed them, in namespace `minfer`.
+// PyTorch (stable ABI) registration of the attention operators, and of the normalisation, projection
+// and rotary-embedding steps that feed them, in namespace `minfer`.
 //
 // This file is the only place where torch types appear: it validates tensors exactly as the
 // reference host function does, turns them into pointers/strides and calls the C ABI of
@@ -264,10 +264,82 @@ void rmsnorm_hip(double eps,
              "rmsnorm");
 }
 
+// D = alpha * A B + beta * C.  Same signature, argument meaning and checks as the reference's gemm_cuda for
+// 16-bit weights (reference: src/minfer/kernels/torch_ext/csrc/cuda/gemm/op.cuh:218-297): B stored [in_dim,
+// out_dim] selects A B, B stored [out_dim, in_dim] selects A B^T (the first wins when both fit, as there).
+// Quantised (byte) weights are not implemented here.  bfloat16 is admitted as well.
+void gemm_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size, double alpha, double beta,
+              const Tensor& A,   // [B, L, in_dim]
+              const Tensor& B,   // [in_dim, out_dim] or [out_dim, in_dim]
+              const Tensor& C,   // [B, L, out_dim]
+              Tensor& D) {       // [B, L, out_dim]
+    (void)qblock_size; (void)qtype_size;
+    STD_TORCH_CHECK(qtype_int == 1 || qtype_int == 30, "gemm: only 16-bit weights (qtype F16 = 1, BF16 = 30) are implemented");
+    STD_TORCH_CHECK(on_gpu(A) && on_gpu(B) && on_gpu(C) && on_gpu(D), "gemm: all tensors must be on the GPU");
+    const ScalarType t = A.scalar_type();
+    STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, "gemm: A must be float16 or bfloat16");
+    STD_TORCH_CHECK(B.scalar_type() == t && C.scalar_type() == t && D.scalar_type() == t, "gemm: A, B, C and D must share one dtype");
+    STD_TORCH_CHECK(A.dim() == 3 && B.dim() == 2 && C.dim() == 3 && D.dim() == 3, "gemm: A, C, D must be 3-D and B 2-D");
+    STD_TORCH_CHECK(A.is_contiguous() && B.is_contiguous() && C.is_contiguous() && D.is_contiguous(), "gemm: tensors must be contiguous");
+    const int64_t K = A.size(-1), M = A.numel() / (K > 0 ? K : 1);
+    STD_TORCH_CHECK(B.size(0) == K || B.size(1) == K, "gemm: A and B cannot be multiplied");
+    const bool kn = B.size(0) == K;
+    const int64_t N = kn ? B.size(1) : B.size(0);
+    STD_TORCH_CHECK(A.size(0) * A.size(1) == C.size(0) * C.size(1) && C.size(-1) == N, "gemm: C does not have the shape of A B");
+    STD_TORCH_CHECK(C.sizes().equals(D.sizes()), "gemm: C and D shapes differ");
+    STD_TORCH_CHECK(alpha != 0.0, "gemm: alpha must not be 0");
+    check_rc(minfer_gemm(t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16, kn ? MINFER_GEMM_B_KN : MINFER_GEMM_B_NK,
+                         A.const_data_ptr(), B.const_data_ptr(), C.const_data_ptr(), D.mutable_data_ptr(), M, N, K, K,
+                         kn ? N : K, N, N, alpha, beta, current_stream()),
+             "gemm");
+}
+
+// q_out = x wq^T, k_out = x wk^T, v_out = x wv^T.  The reference's op of this name and signature is a stub
+// (reference: src/minfer/kernels/torch_ext/csrc/cuda/qkv/op.cuh:21-34); what it must compute is fixed by its test
+// (reference: test/kernels.py:173-214): weights stored [out_dim, hidden_dim].  A weight stored
+// [hidden_dim, out_dim] (the layout the stub's comments name) is accepted when its shape says so unambiguously.
+void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int64_t q_qblock_size, int64_t k_qblock_size,
+             int64_t v_qblock_size, int64_t q_qtype_size, int64_t k_qtype_size, int64_t v_qtype_size,
+             const Tensor& x,    // [B, L, hidden_dim]
+             const Tensor& wq,   // [q_dim, hidden_dim]
+             const Tensor& wk,   // [kv_dim, hidden_dim]
+             const Tensor& wv,   // [kv_dim, hidden_dim]
+             Tensor& q_out,      // [B, L, q_dim]
+             Tensor& k_out,      // [B, L, kv_dim]
+             Tensor& v_out) {    // [B, L, kv_dim]
+    (void)q_qblock_size; (void)k_qblock_size; (void)v_qblock_size; (void)q_qtype_size; (void)k_qtype_size; (void)v_qtype_size;
+    STD_TORCH_CHECK((q_qtype_int == 1 || q_qtype_int == 30) && k_qtype_int == q_qtype_int && v_qtype_int == q_qtype_int,
+                    "qkv: only 16-bit weights (qtype F16 = 1, BF16 = 30) are implemented");
+    const ScalarType t = x.scalar_type();
+    STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, "qkv: x must be float16 or bfloat16");
+    STD_TORCH_CHECK(x.dim() == 3 && x.is_contiguous() && on_gpu(x), "qkv: x must be a contiguous 3-D GPU tensor");
+    const int64_t K = x.size(-1), M = x.numel() / (K > 0 ? K : 1);
+    const int dtype = t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16;
+    void* stream = current_stream();
+    const Tensor* ws[3] = {&wq, &wk, &wv};
+    Tensor* outs[3] = {&q_out, &k_out, &v_out};
+    const char* names[3] = {"qkv: q", "qkv: k", "qkv: v"};
+    for (int i = 0; i < 3; ++i) {
+        const Tensor& w = *ws[i];
+        Tensor& o = *outs[i];
+        STD_TORCH_CHECK(on_gpu(w) && on_gpu(o) && w.scalar_type() == t && o.scalar_type() == t, names[i], ": dtype or device mismatch");
+        STD_TORCH_CHECK(w.dim() == 2 && o.dim() == 3 && w.is_contiguous() && o.is_contiguous(), names[i], ": weight must be contiguous 2-D, output contiguous 3-D");
+        const int64_t N = o.size(-1);
+        STD_TORCH_CHECK(o.size(0) == x.size(0) && o.size(1) == x.size(1), names[i], ": output must be [B, L, out_dim]");
+        const bool nk = w.size(0) == N && w.size(1) == K;
+        STD_TORCH_CHECK(nk || (w.size(0) == K && w.size(1) == N), names[i], ": weight must be [out_dim, hidden_dim] (or [hidden_dim, out_dim])");
+        check_rc(minfer_gemm(dtype, nk ? MINFER_GEMM_B_NK : MINFER_GEMM_B_KN, x.const_data_ptr(), w.const_data_ptr(), nullptr,
+                             o.mutable_data_ptr(), M, N, K, K, nk ? K : N, N, N, 1.0, 0.0, stream),
+                 names[i]);
+    }
+}
+
 STABLE_TORCH_LIBRARY(minfer, m) {
     // verbatim the reference's schema (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:30)
     m.def("flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()");
-    // verbatim the reference's schemas (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:24-26)
+    // verbatim the reference's schemas (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:24-29)
+    m.def("gemm(int qtype_int, int qblock_size, int qtype_size, float alpha, float beta, Tensor A, Tensor B, Tensor C, Tensor(a!) out) -> ()");
+    m.def("qkv(int q_qtype_int, int k_qtype_int, int v_qtype_int, int q_qblock_size, int k_qblock_size, int v_qblock_size, int q_qtype_size, int k_qtype_size, int v_qtype_size, Tensor x, Tensor wq, Tensor wk, Tensor wv, Tensor(a!) q_out, Tensor(a!) k_out, Tensor(a!) v_out) -> ()");
     m.def("rmsnorm(float eps, Tensor input, Tensor w, Tensor(a!) out) -> ()");
     m.def("il_rope(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()");
     m.def("neox_rope(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()");
@@ -282,6 +354,8 @@ STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-ke
     m.impl("flash_attn_decode", TORCH_BOX(&flash_attn_decode_hip));
     m.impl("flash_attn_varlen", TORCH_BOX(&flash_attn_varlen_hip));
     m.impl("rmsnorm", TORCH_BOX(&rmsnorm_hip));
+    m.impl("gemm", TORCH_BOX(&gemm_hip));
+    m.impl("qkv", TORCH_BOX(&qkv_hip));
     m.impl("il_rope", TORCH_BOX(&il_rope_hip));
     m.impl("neox_rope", TORCH_BOX(&neox_rope_hip));
     m.impl("rope_kv_append", TORCH_BOX(&rope_kv_append_hip));

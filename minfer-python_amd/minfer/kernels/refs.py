@@ -10,6 +10,11 @@ def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
     return F.rms_norm(x, (x.shape[-1],), weight=weight, eps=eps)
 
 
+def gemm(input: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, out: torch.Tensor, alpha: float, beta: float):
+    """alpha * input @ weight + beta * bias -> out; all 2-D (squeeze 3-D activations first)."""
+    torch.addmm(bias, input, weight, beta=beta, alpha=alpha, out=out)
+
+
 def flash_attn(Q: torch.Tensor, K: torch.Tensor, V: torch.Tensor, mask: torch.Tensor) -> torch.Tensor:
     """SDPA with a bool mask (True = attend).  Q/K/V: (B, n_heads, L, head_dim); K/V must already be
     expanded to n_heads for GQA (``repeat_interleave(n_rep, dim=1)``)."""

@@ -8,5 +8,5 @@ except ImportError as e:  # pragma: no cover
         "minfer.kernels.torch_ext._C is not built; run `python minfer-python_amd/build.py` "
         "(hipcc, gfx950) first"
     ) from e
-from .ops import (flash_attn, flash_attn_decode, flash_attn_varlen, il_rope, neox_rope,  # noqa: E402,F401
-                  rmsnorm, rope_kv_append)
+from .ops import (flash_attn, flash_attn_decode, flash_attn_varlen, gemm, il_rope, neox_rope,  # noqa: E402,F401
+                  qkv, rmsnorm, rope_kv_append)

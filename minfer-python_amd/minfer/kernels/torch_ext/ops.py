@@ -1,6 +1,6 @@
 """Python wrappers and fake (meta) kernels of the attention ops and of the rotary-embedding step
 before them, mirroring the reference's wrapper layer (reference:
-src/minfer/kernels/torch_ext/ops.py:60-126, 234-266): positional pass-through
+src/minfer/kernels/torch_ext/ops.py:60-266): positional pass-through
 to ``torch.ops.minfer.<op>.default``; the result is written into ``out``."""
 import torch
 
@@ -151,3 +151,43 @@ def _(eps, input, w, out):
     torch._check(input.shape == out.shape)
     torch._check(input.dim() in (3, 4))
     torch._check(input.size(-1) == w.size(0) or input.size(-1) % w.size(0) == 0)
+
+
+def gemm(qtype_int: int, qblock_size: int, qtype_size: int, alpha: float, beta: float,
+         A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, D: torch.Tensor):
+    """D = alpha * A B + beta * C; A [B,L,in_dim], weight B [in_dim,out_dim] (or [out_dim,in_dim]: A B^T), C and D
+    [B,L,out_dim]."""
+    return torch.ops.minfer.gemm.default(qtype_int, qblock_size, qtype_size, alpha, beta, A, B, C, D)
+
+
+@torch.library.register_fake("minfer::gemm")
+def _(qtype_int, qblock_size, qtype_size, alpha, beta, A, B, C, D):
+    torch._check(A.dtype in _ACT_DTYPES)
+    torch._check(B.dtype == A.dtype and C.dtype == A.dtype and D.dtype == A.dtype)
+    torch._check(A.device == B.device == C.device == D.device)
+    torch._check(A.device.type == "cuda")
+    torch._check(A.dim() == 3 and B.dim() == 2 and C.dim() == 3 and D.dim() == 3)
+    torch._check(A.size(0) * A.size(1) == C.size(0) * C.size(1))
+    torch._check(B.size(-1) == C.size(-1) or B.size(0) == C.size(-1))
+    torch._check(C.shape == D.shape)
+    torch._check(alpha != 0.0)
+
+
+def qkv(q_qtype_int: int, k_qtype_int: int, v_qtype_int: int, q_qblock_size: int, k_qblock_size: int, v_qblock_size: int,
+        q_qtype_size: int, k_qtype_size: int, v_qtype_size: int,
+        x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor,
+        q_out: torch.Tensor, k_out: torch.Tensor, v_out: torch.Tensor):
+    """The three projections q_out = x wq^T, k_out = x wk^T, v_out = x wv^T; x [B,L,hidden], weights [out,hidden]."""
+    return torch.ops.minfer.qkv.default(q_qtype_int, k_qtype_int, v_qtype_int, q_qblock_size, k_qblock_size, v_qblock_size,
+                                        q_qtype_size, k_qtype_size, v_qtype_size, x, wq, wk, wv, q_out, k_out, v_out)
+
+
+@torch.library.register_fake("minfer::qkv")
+def _(q_qtype_int, k_qtype_int, v_qtype_int, q_qblock_size, k_qblock_size, v_qblock_size, q_qtype_size, k_qtype_size,
+      v_qtype_size, x, wq, wk, wv, q_out, k_out, v_out):
+    torch._check(x.dtype in _ACT_DTYPES)
+    torch._check(all(t.dtype == x.dtype for t in (wq, wk, wv, q_out, k_out, v_out)))
+    torch._check(x.device == wq.device == wk.device == wv.device == q_out.device == k_out.device == v_out.device)
+    torch._check(x.device.type == "cuda")
+    torch._check(x.dim() == 3 and q_out.dim() == 3 and k_out.dim() == 3 and v_out.dim() == 3)
+    torch._check(wq.dim() == 2 and wk.dim() == 2 and wv.dim() == 2)

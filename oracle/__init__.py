@@ -1,4 +1,5 @@
-"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c, rope_oracle.c and rmsnorm_oracle.c.
+"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c, rope_oracle.c, rmsnorm_oracle.c and
+gemm_oracle.c.
 
 Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py may import this
 package.  The shipped operator never does: it launches HIP kernels or raises.
@@ -38,7 +39,7 @@ def lib():
             build()
         _LIB = ctypes.CDLL(so)
         for name in ("oracle_flash_attn", "oracle_flash_attn_rows", "oracle_flash_attn_decode",
-                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append", "oracle_rmsnorm"):
+                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append", "oracle_rmsnorm", "oracle_gemm"):
             getattr(_LIB, name).restype = ctypes.c_int
     return _LIB
 
@@ -176,4 +177,24 @@ def rmsnorm(x, w, eps):
     rc = lib().oracle_rmsnorm(_ptr(x), _ptr(w), _ptr(out), ctypes.c_int64(x.size // dim), ctypes.c_int64(dim), ctypes.c_double(eps))
     if rc != 0:
         raise ValueError(f"oracle_rmsnorm rc={rc}")
+    return out
+
+
+GEMM_B_KN, GEMM_B_NK = 0, 1
+
+
+def gemm(a, b, c, alpha, beta, b_layout=GEMM_B_KN):
+    """alpha * A @ B + beta * C with B stored [K,N] (b_layout 0) or [N,K] (1); a [..., K] with leading dims
+    flattened (reference: gemm/op.cuh:284-297, refs.py:49-51); fp64 sums; returns float32 [M, N], unrounded."""
+    a, b = _f32(a), _f32(b)
+    K = a.shape[-1]
+    a2 = np.ascontiguousarray(a.reshape(-1, K))
+    M = a2.shape[0]
+    N = b.shape[1] if b_layout == GEMM_B_KN else b.shape[0]
+    c2 = np.ascontiguousarray(_f32(c).reshape(M, N)) if c is not None else None
+    out = np.empty((M, N), dtype=np.float32)
+    rc = lib().oracle_gemm(ctypes.c_int(b_layout), _ptr(a2), _ptr(b), _ptr(c2) if c2 is not None else None, _ptr(out),
+                           *[ctypes.c_int64(x) for x in (M, N, K)], ctypes.c_double(alpha), ctypes.c_double(beta))
+    if rc != 0:
+        raise ValueError(f"oracle_gemm rc={rc}")
     return out

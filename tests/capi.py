@@ -9,6 +9,7 @@ HEADER = os.path.join(ROOT, "include", "minfer_attn.h")
 
 F16, BF16 = 1, 30
 ROPE_INTERLEAVED, ROPE_NEOX = 0, 1
+GEMM_B_KN, GEMM_B_NK = 0, 1
 OK, EINVAL, EWORKSPACE, ELAUNCH = 0, -1, -2, -3
 
 
@@ -49,6 +50,8 @@ def lib():
                                             i64, i64, i64, i64, i64, dbl, vp]
         L.minfer_rmsnorm.restype = ctypes.c_int
         L.minfer_rmsnorm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, dbl, vp]
+        L.minfer_gemm.restype = ctypes.c_int
+        L.minfer_gemm.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, dbl, dbl, vp]
         _lib = L
     return _lib
 
@@ -125,3 +128,13 @@ def rmsnorm(x, w, out, eps):
     """RMS normalisation of contiguous x over vectors of length len(w), into out."""
     dim = w.shape[0]
     return lib().minfer_rmsnorm(_dtype_code(x), x.data_ptr(), w.data_ptr(), out.data_ptr(), x.numel() // dim, dim, eps, _stream())
+
+
+def gemm(a, b, c, d, alpha, beta, b_layout=GEMM_B_KN):
+    """d[M,N] = alpha * a[M,K] x b + beta * c; 2-D tensors with unit stride on their last dimension; b is
+    [K,N] (GEMM_B_KN) or [N,K] (GEMM_B_NK); c may be None when beta == 0."""
+    M, K = a.shape
+    N = d.shape[1]
+    return lib().minfer_gemm(_dtype_code(a), b_layout, a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None,
+                             d.data_ptr(), M, N, K, a.stride(0), b.stride(0), c.stride(0) if c is not None else N, d.stride(0),
+                             alpha, beta, _stream())

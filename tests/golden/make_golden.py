@@ -11,7 +11,8 @@ fp16 kernels see exactly the values the expected output was computed from.
 
 The rotary-embedding fixture (rope_small.npz) pins the reference's torch formulation of both styles
 (reference src/minfer/kernels/refs.py:12-47) in float64 on seeded fp16-representable inputs, and
-rmsnorm_small.npz the reference's F.rms_norm call (refs.py:10) in float64.
+rmsnorm_small.npz the reference's F.rms_norm call (refs.py:10) in float64, gemm_small.npz its torch.addmm call
+(refs.py:49-51) in float64.
 
 Run:  python tests/golden/make_golden.py
 """
@@ -110,6 +111,18 @@ def make_rmsnorm(name, shape, eps, seed):
                         eps=eps, y=y.numpy().astype(np.float32))
 
 
+def make_gemm(name, M, N, K, alpha, beta, seed):
+    """Expected values from the reference's oracle call torch.addmm (reference src/minfer/kernels/refs.py:49-51)
+    evaluated in float64; inputs drawn as in the reference's test (reference test/kernels.py:133-136)."""
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(M, K, generator=g).half().double()
+    b = ((1 / K ** 0.5) * torch.randn(K, N, generator=g)).half().double()
+    c = torch.randn(M, N, generator=g).half().double()
+    d = torch.addmm(c, a, b, beta=beta, alpha=alpha)
+    np.savez_compressed(os.path.join(HERE, name + ".npz"), a=a.numpy().astype(np.float16), b=b.numpy().astype(np.float16),
+                        c=c.numpy().astype(np.float16), alpha=alpha, beta=beta, d=d.numpy().astype(np.float32))
+
+
 if __name__ == "__main__":
     torch.set_num_threads(1)
     make("dense_causal_b1_h4_kv2_l16_d64", 1, 4, 2, 16, 64, "causal", 1)
@@ -119,4 +132,5 @@ if __name__ == "__main__":
     make_varlen("varlen_h4_kv2_d64", 4, 2, 64, [5, 1, 33, 70], 5)
     make_rope("rope_small", 2, 9, 3, 64, 32, 2048, 1e6, 6)
     make_rmsnorm("rmsnorm_small", (2, 5, 3, 40), 1e-6, 7)
+    make_gemm("gemm_small", 70, 72, 128, 2.0, 3.0, 8)
     print("golden vectors written to", HERE)

@@ -1,0 +1,152 @@
+"""GPU parity tests (-m gpu) of the GEMM kernels and of the gemm / qkv operators, through the C ABI and the
+registered torch ops, against the fp64 CPU oracle on identical seeded inputs.
+
+Tolerance: the reference's tests allow atol 6e-1 (gemm) and 2e-1 (qkv) (reference: test/kernels.py:145,
+212-214).  Here every element must lie within 0.51 units in the last place of the output format of the
+oracle's exact value, plus 2^-17 of the largest magnitude of the result for the fp32 accumulation (which
+shows only where a sum of a few hundred terms cancels to something far smaller than its terms)."""
+import os
+
+import numpy as np
+import pytest
+import torch
+
+import capi
+import oracle
+import workloads
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+MANT = {torch.float16: 10, torch.bfloat16: 7}
+MIN_EXP = {torch.float16: -14, torch.bfloat16: -126}
+KN, NK = capi.GEMM_B_KN, capi.GEMM_B_NK
+
+
+def assert_close(got, exact, dtype, what=""):
+    got = got.float().cpu().numpy().astype(np.float64)
+    exact = exact.astype(np.float64)
+    e = np.floor(np.log2(np.maximum(np.abs(exact), 2.0 ** MIN_EXP[dtype])))
+    bound = 0.51 * 2.0 ** (e - MANT[dtype]) + 2.0 ** -17 * float(np.abs(exact).max())
+    err = np.abs(got - exact)
+    worst = np.unravel_index(np.argmax(err - bound), err.shape)
+    assert not (err > bound).any(), (f"{what}: {(err > bound).sum()} elements out of bound; at {worst} got {got[worst]!r}, "
+                                     f"exact {float(exact[worst])!r}")
+
+
+def make(M, N, K, layout, dtype, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(M, K, generator=g).to(dtype)
+    b = ((1 / K ** 0.5) * torch.randn((K, N) if layout == KN else (N, K), generator=g)).to(dtype)
+    c = torch.randn(M, N, generator=g).to(dtype)
+    return a, b, c
+
+
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K,alpha,beta", [
+    (256, 256, 64, 1.0, 0.0),        # four tiles of the 128 x 128 kernel, one K step
+    (512, 384, 256, 2.0, 3.0),
+    (300, 264, 192, 0.5, 2.0),       # ragged rows and columns (N a multiple of 8 only)
+    (100, 72, 64, 1.0, 1.0),
+    (1, 128, 128, 1.0, 0.0),         # a single row (decode-time projection)
+    (4096, 4096, 128, 1.0, 1.0),     # enough tiles for the 256 x 256 kernel
+    (3000, 4104, 64, 2.0, 0.0),      # the same with ragged edges
+    (33, 17, 50, 1.0, 1.0),          # nothing tileable: plain kernel
+    (64, 64, 72, 1.0, 0.0),          # K not a multiple of 64: plain kernel
+])
+def test_gemm_matches_oracle(layout, dtype, M, N, K, alpha, beta):
+    a, b, c = make(M, N, K, layout, dtype, M + N + K)
+    if M * N * K <= 1 << 26:
+        exact = oracle.gemm(a, b, c, alpha, beta, layout)
+        rows = slice(None)
+    else:       # the oracle is a scalar CPU program: a sample of rows at this size
+        rows = torch.tensor(sorted({0, 1, 255, 256, 257, M // 2, M - 257, M - 2, M - 1} | set(range(1000, 1064))))
+        exact = oracle.gemm(a[rows], b, c[rows], alpha, beta, layout)
+    d = torch.full((M, N), float("nan"), dtype=dtype, device=DEV)
+    assert capi.gemm(a.to(DEV), b.to(DEV), c.to(DEV), d, alpha, beta, layout) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert_close(d[rows], exact, dtype, "gemm")
+    if not isinstance(rows, slice):   # the whole result against an fp32 torch evaluation of the same expression
+        ref = alpha * (a.to(DEV).float() @ (b.to(DEV).float() if layout == KN else b.to(DEV).float().T)) + beta * c.to(DEV).float()
+        assert float((d.float() - ref).abs().max()) <= 2.0 ** -MANT[dtype] * float(ref.abs().max())
+
+
+def test_gemm_golden_strided_and_in_place():
+    z = np.load(os.path.join(os.path.dirname(__file__), "golden", "gemm_small.npz"))
+    a, b, c = (torch.from_numpy(z[k]).to(DEV) for k in "abc")
+    alpha, beta = float(z["alpha"]), float(z["beta"])
+    d = torch.empty_like(c)
+    assert capi.gemm(a, b, c, d, alpha, beta) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert_close(d, z["d"], torch.float16, "golden")
+    # C aliasing D
+    d2 = c.clone()
+    assert capi.gemm(a, b, d2, d2, alpha, beta) == capi.OK
+    torch.cuda.synchronize()
+    assert torch.equal(d2, d)
+    # row strides larger than the rows (views of wider buffers), beta = 0 with no C
+    big_a = torch.randn(70, 200, device=DEV).half()
+    big_d = torch.full((70, 96), float("nan"), dtype=torch.float16, device=DEV)
+    av, dv = big_a[:, 8:136], big_d[:, 16:88]
+    assert capi.gemm(av, b, None, dv, 1.0, 0.0) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert_close(dv, oracle.gemm(av.cpu().contiguous(), b.cpu(), None, 1.0, 0.0), torch.float16, "strided")
+    assert torch.isnan(big_d[:, :16]).all() and torch.isnan(big_d[:, 88:]).all()
+
+
+@pytest.mark.parametrize("S", [1024, 2048])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (2.0, 3.0)])
+def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
+    """The reference's test recipe (test/kernels.py:119-147): A [1,S,S] ~ N(0,1), weight [S,S] ~ N(0,1)/sqrt(S), bias
+    ~ N(0,1), through the op with the reference's signature; sampled rows against the oracle, everything against
+    the reference's own expression at its own tolerance."""
+    a, w, bias = workloads.gemm_input(S, S, S, seed=S, device=DEV)
+    out = torch.zeros_like(bias)
+    assert kerns.gemm(1, 1, 2, alpha, beta, a, w, bias, out) is None
+    torch.cuda.synchronize()
+    rows = torch.arange(0, S, S // 16)
+    assert_close(out[0, rows], oracle.gemm(a[0, rows].cpu(), w.cpu(), bias[0, rows].cpu(), alpha, beta), torch.float16, "op")
+    assert torch.allclose((alpha * (a @ w) + beta * bias).float(), out.float(), atol=6e-1)
+    d = torch.empty(S, S, dtype=torch.float16, device=DEV)
+    assert capi.gemm(a[0], w, bias[0], d, alpha, beta) == capi.OK
+    torch.cuda.synchronize()
+    assert torch.equal(d, out[0])
+
+
+def test_qkv_op_and_reference_checks(kerns):
+    """The QKV recipe of the reference's test at a smaller batch (test/kernels.py:173-214: hidden 6144, 48 query and
+    8 KV heads of 128): x @ W^T for the three weights stored [out, hidden]."""
+    B, L, hidden, q_dim, kv_dim = 2, 512, 6144, 48 * 128, 8 * 128
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(B, L, hidden, generator=g).half().to(DEV)
+    wq, wk, wv = (((1 / hidden ** 0.5) * torch.randn(n, hidden, generator=g)).half().to(DEV) for n in (q_dim, kv_dim, kv_dim))
+    q, k, v = (torch.zeros(B, L, n, dtype=torch.float16, device=DEV) for n in (q_dim, kv_dim, kv_dim))
+    assert kerns.qkv(1, 1, 1, 1, 1, 1, 2, 2, 2, x, wq, wk, wv, q, k, v) is None
+    torch.cuda.synchronize()
+    rows = torch.arange(0, B * L, 64)
+    xs = x.view(B * L, hidden)[rows].cpu()
+    for out, w, name in ((q, wq, "q"), (k, wk, "k"), (v, wv, "v")):
+        assert_close(out.view(B * L, -1)[rows], oracle.gemm(xs, w.cpu(), None, 1.0, 0.0, oracle.GEMM_B_NK), torch.float16, name)
+        assert torch.allclose((x @ w.T).float(), out.float(), atol=2e-1)
+    # weights stored [hidden, out] are recognised by their shape
+    k2 = torch.zeros_like(k)
+    kerns.qkv(1, 1, 1, 1, 1, 1, 2, 2, 2, x, wq, wk.T.contiguous(), wv, q, k2, v)
+    torch.cuda.synchronize()
+    assert float((k2.float() - k.float()).abs().max()) <= 4e-3
+    with pytest.raises(RuntimeError):
+        kerns.qkv(1, 1, 1, 1, 1, 1, 2, 2, 2, x, wq, wk[:, :100].contiguous(), wv, q, k, v)
+    with pytest.raises(RuntimeError):
+        kerns.qkv(2, 2, 2, 32, 32, 32, 18, 18, 18, x, wq, wk, wv, q, k, v)          # quantised weights: not implemented
+    # gemm's reference checks (gemm/op.cuh:229-273)
+    a, w, bias = workloads.gemm_input(64, 64, 64, seed=1, device=DEV)
+    out = torch.zeros_like(bias)
+    with pytest.raises(RuntimeError):
+        kerns.gemm(1, 1, 2, 0.0, 1.0, a, w, bias, out)                              # alpha == 0
+    with pytest.raises(RuntimeError):
+        kerns.gemm(1, 1, 2, 1.0, 0.0, a[0], w, bias, out)                           # A must be 3-D
+    with pytest.raises(RuntimeError):
+        kerns.gemm(1, 1, 2, 1.0, 0.0, a, w[:, :32], bias, out)                      # not contiguous / wrong shape
+    with pytest.raises(RuntimeError):
+        kerns.gemm(1, 1, 2, 1.0, 0.0, a, w.float(), bias, out)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        kerns.gemm(1, 1, 2, 1.0, 0.0, a.cpu(), w.cpu(), bias.cpu(), out.cpu())

@@ -114,6 +114,20 @@ def test_rmsnorm_validation_rejects_before_launch():
     assert norm(n=0) == capi.OK and capi.last_error() == ""
 
 
+def test_gemm_validation_rejects_before_launch():
+    L = capi.lib()
+    gemm = lambda dtype=capi.F16, layout=0, a=0x1000, b=0x2000, c=0x3000, d=0x4000, M=64, N=64, K=64, lda=64, ldb=64, \
+        ldc=64, ldd=64, alpha=1.0, beta=1.0: L.minfer_gemm(dtype, layout, a, b, c, d, M, N, K, lda, ldb, ldc, ldd, alpha, beta, None)
+    assert gemm(dtype=2) == capi.EINVAL and "dtype" in capi.last_error()
+    assert gemm(layout=2) == capi.EINVAL and "b_layout" in capi.last_error()
+    assert gemm(M=-1) == capi.EINVAL
+    assert gemm(a=0) == capi.EINVAL and "null" in capi.last_error()
+    assert gemm(c=0) == capi.EINVAL                      # beta != 0 needs C
+    assert gemm(lda=32) == capi.EINVAL and "leading" in capi.last_error()
+    assert gemm(N=128, ldd=64) == capi.EINVAL
+    assert gemm(M=0) == capi.OK and gemm(N=0) == capi.OK and capi.last_error() == ""
+
+
 def test_python_surface_matches_reference_names(kerns):
     from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
     from minfer.kernels import KernelBackend, refs
@@ -136,6 +150,17 @@ def test_python_surface_matches_reference_names(kerns):
         assert str(getattr(torch.ops.minfer, name).default._schema) == \
             f"minfer::{name}(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()"
     assert callable(kerns.rope_kv_append)
+    assert list(inspect.signature(te.gemm).parameters) == ["qtype_int", "qblock_size", "qtype_size", "alpha", "beta", "A", "B", "C", "D"]
+    assert str(torch.ops.minfer.gemm.default._schema) == ("minfer::gemm(int qtype_int, int qblock_size, int qtype_size, float alpha, "
+                                                          "float beta, Tensor A, Tensor B, Tensor C, Tensor(a!) out) -> ()")
+    assert list(inspect.signature(te.qkv).parameters)[9:] == ["x", "wq", "wk", "wv", "q_out", "k_out", "v_out"]
+    assert str(torch.ops.minfer.qkv.default._schema).endswith("Tensor x, Tensor wq, Tensor wk, Tensor wv, Tensor(a!) q_out, "
+                                                              "Tensor(a!) k_out, Tensor(a!) v_out) -> ()")
+    assert callable(kerns.gemm) and callable(kerns.qkv)
+    ga, gw, gb = torch.randn(5, 7), torch.randn(7, 3), torch.randn(5, 3)
+    go = torch.empty(5, 3)
+    refs.gemm(ga, gw, gb, go, 2.0, 3.0)
+    assert float((go - torch.from_numpy(oracle.gemm(ga, gw, gb, 2.0, 3.0))).abs().max()) < 1e-5
     assert list(inspect.signature(te.rmsnorm).parameters) == ["eps", "input", "w", "out"] and callable(kerns.rmsnorm)
     assert str(torch.ops.minfer.rmsnorm.default._schema) == "minfer::rmsnorm(float eps, Tensor input, Tensor w, Tensor(a!) out) -> ()"
     xn, wn = torch.randn(2, 3, 16), torch.randn(16)
@@ -162,6 +187,11 @@ def test_no_cpu_fallback(kerns):
     x = torch.zeros(1, 4, 2, 128, dtype=torch.float16)
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.rmsnorm(1e-6, x, torch.ones(128, dtype=torch.float16), torch.empty_like(x))
+    h = torch.zeros(1, 4, 64, dtype=torch.float16)
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.gemm(1, 1, 2, 1.0, 0.0, h, torch.zeros(64, 64, dtype=torch.float16), h, torch.empty_like(h))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.qkv(1, 1, 1, 1, 1, 1, 2, 2, 2, h, *[torch.zeros(64, 64, dtype=torch.float16)] * 3, *[torch.empty_like(h) for _ in range(3)])
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.il_rope(64, 0, 1e4, x)
     with pytest.raises((NotImplementedError, RuntimeError)):
@@ -184,6 +214,8 @@ def test_workload_generators_are_seeded():
     assert len(lens) == 16 and min(lens) >= 128 and max(lens) <= 2048 and q.shape == (1, 64, int(cu[-1]), 128)
     assert workloads.prefill_flops(32, 128, [4096]) == 2 * 128 * 32 * 4096 * 4097
     assert workloads.decode_bytes([10, 20], 32, 8, 128) == 30 * 4096 + 2 * 2 * 32 * 128 * 2
+    ga, gw, gb = workloads.gemm_input(8, 16, 32, seed=2)
+    assert ga.shape == (1, 8, 32) and gw.shape == (32, 16) and gb.shape == (1, 8, 16) and workloads.gemm_flops(8, 16, 32) == 8192
     xs, ws = workloads.rmsnorm_input((2, 3, 64), seed=5)
     assert xs.shape == (2, 3, 64) and ws.shape == (64,) and torch.equal(xs, workloads.rmsnorm_input((2, 3, 64), seed=5)[0])
     assert workloads.rmsnorm_bytes((2, 3, 64)) == (2 * 384 + 64) * 2
