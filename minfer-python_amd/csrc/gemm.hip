@@ -7,7 +7,8 @@
 //
 // Design.  A workgroup (8 waves, two per SIMD) owns a 256 x 256 tile of D (128 x 128 with 4 waves for problems
 // too small to fill the chip with large tiles) and walks K in steps of 64; the A and B panels of a step (32 KB
-// each) are copied global->LDS without passing through registers, double-buffered, one barrier per step.
+// each) are copied global->LDS without passing through registers, double-buffered, one barrier per step
+// (placed inside the step, so that the matrix pipe keeps running across step boundaries).
 // Every wave owns 128 (64) rows (m) x 64 columns (n) as 4 (2) x 2 accumulator blocks of 32x32
 // and computes the transposed product D^T = B^T A^T, so that a lane ends up with 4 consecutive n of one row m
 // and the epilogue stores 8 bytes per register quadruple: B supplies the MFMA A operand (for the [K, N] layout
@@ -154,34 +155,44 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) mf[mb] = lds_read_b128(m_rd[kk], AOFF + (mb >> 1) * kRowTile + 32 * (mb & 1) * 128);
     };
-    auto compute = [&](auto stage_tag) __attribute__((always_inline)) {
-        s16x8 nf[2][2], mf[2][MB];
-        load_frags(stage_tag, 0, nf[0], mf[0]);
-#pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            if (kk + 1 < 4) load_frags(stage_tag, kk + 1, nf[(kk + 1) & 1], mf[(kk + 1) & 1]);
-#pragma unroll
-            for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-                for (int nb = 0; nb < 2; ++nb) acc[nb][mb] = T::mfma32(nf[kk & 1][nb], mf[kk & 1][mb], acc[nb][mb]);
-        }
-    };
-
-    // ---- main loop: one barrier per K step; the copy of step t+1 is issued right after the barrier that opens
-    // step t, into the stage step t-1 has just vacated --------------------------------------------------
+    // ---- main loop ---------------------------------------------------------------------------------------
+    // Fragments are double-buffered in registers: while the 8 (4) MFMAs of one 16-wide k slice run, the fragments
+    // of the next slice are read from LDS.  The workgroup's only barrier per K step sits between the third and
+    // the last slice: a wave arrives when it has read the last fragments of the current stage and its own share
+    // of the next stage's copy has landed; after the barrier it issues the copy of the step after next into the
+    // stage just vacated and reads the next step's first fragments, all of which overlaps with the last slice's
+    // MFMAs, so the matrix pipe does not drain at step boundaries.
     const int KT = p.K / kBK;
-    issue(0, 0);
-    for (int kt = 0; kt < KT; kt += 2) {
-        wait_vmcnt<0>();
+    s16x8 nf[2][2], mf[2][MB];
+    auto mfmas = [&](int buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int nb = 0; nb < 2; ++nb) acc[nb][mb] = T::mfma32(nf[buf][nb], mf[buf][mb], acc[nb][mb]);
+    };
+    auto step = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        load_frags(stage_tag, 1, nf[1], mf[1]);
+        mfmas(0);
+        load_frags(stage_tag, 2, nf[0], mf[0]);
+        mfmas(1);
+        load_frags(stage_tag, 3, nf[1], mf[1]);
+        mfmas(0);
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read everything it needs from this stage
+        wait_vmcnt<0>();                                       // and its share of the next stage has landed
         __syncthreads();
-        if (kt + 1 < KT) issue(kt + 1, 1);
-        compute(std::integral_constant<int, 0>{});
-        if (kt + 1 < KT) {
-            wait_vmcnt<0>();
-            __syncthreads();
-            if (kt + 2 < KT) issue(kt + 2, 0);
-            compute(std::integral_constant<int, 1>{});
-        }
+        if (kt + 2 < KT) issue(kt + 2, STAGE);
+        if (kt + 1 < KT) load_frags(std::integral_constant<int, STAGE ^ 1>{}, 0, nf[0], mf[0]);
+        mfmas(1);
+    };
+    issue(0, 0);
+    if (KT > 1) issue(1, 1);
+    if (KT > 1) wait_vmcnt<8>(); else wait_vmcnt<0>();   // the 8 copies of step 0 retire first
+    __syncthreads();
+    load_frags(std::integral_constant<int, 0>{}, 0, nf[0], mf[0]);
+    for (int kt = 0; kt < KT; kt += 2) {
+        step(std::integral_constant<int, 0>{}, kt);
+        if (kt + 1 < KT) step(std::integral_constant<int, 1>{}, kt + 1);
     }
 
     // ---- epilogue: D = alpha * acc + beta * C; register r of a block is n = 8(r/4) + 4h + r%4, m = l32 ----
