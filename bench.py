@@ -25,10 +25,12 @@ PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
-PREFILL_TRAFFIC_BYTES = 107691 * 1024
+PREFILL_TRAFFIC_BYTES = 107374 * 1024
 DECODE_TRAFFIC_BYTES = 1089627 * 1024
-ROPE_TRAFFIC_BYTES = 393304 * 1024          # il_rope on [8,4096,48,128], rotary 64
+ROPE_TRAFFIC_BYTES = 393306 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786577 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
+NORM_TRAFFIC_BYTES = 786708 * 1024          # rmsnorm on [8,4096,6144]
+GEMM_TRAFFIC_BYTES = 328543 * 1024          # gemm 4096^3 (B is re-read by each of the 8 XCDs)
 
 
 class HipEvents:
@@ -249,12 +251,12 @@ def main():
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,
-                                   "traffic": None, "kernel": "rmsnorm_rows_kernel<F16,64,16>", "algorithmic_bytes": nbytes}}
+                                   "traffic": NORM_TRAFFIC_BYTES, "kernel": "rmsnorm_rows_kernel<F16,64,16>", "algorithmic_bytes": nbytes}}
     rec["gemm"] = {"value": g_tf, "unit": "TFLOP/s", "ms": g_avg_ms, "median_ms": g_med_ms,
                    "workload": "gemm alpha=1 beta=0, A [1,4096,4096] x W [4096,4096] fp16 (reference README HGEMM table, M=K=N=4096)",
                    "published_reference_us": 605.3,
                    "roofline": {"bound": "mfma", "achieved": g_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": g_tf / PEAK_MFMA_TFLOPS,
-                                "traffic": None, "kernel": "gemm_kernel<F16,[K,N],256x256>", "algorithmic_flops": gflops}}
+                                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_kernel<F16,[K,N],256x256>", "algorithmic_flops": gflops}}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
         rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)
