@@ -31,6 +31,8 @@ ROPE_TRAFFIC_BYTES = 393306 * 1024          # il_rope on [8,4096,48,128], rotary
 APPEND_TRAFFIC_BYTES = 786577 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
 NORM_TRAFFIC_BYTES = 786708 * 1024          # rmsnorm on [8,4096,6144]
 GEMM_TRAFFIC_BYTES = 328543 * 1024          # gemm 4096^3 (B is re-read by each of the 8 XCDs)
+DECODE_Q8_TRAFFIC_BYTES = None              # decode over Q8_0 caches
+APPEND_Q8_TRAFFIC_BYTES = None              # rope_kv_append into Q8_0 caches
 
 
 class HipEvents:
@@ -178,7 +180,19 @@ def main():
     d_avg_ms, d_med_ms = ev.time_each(dstep, stream, min(max(args.steps, 20), 100))
     dbytes = workloads.decode_bytes(ctx.tolist(), 32, 8, 128)
     d_gbs = dbytes / (d_avg_ms * 1e-3) / 1e9
+    # the same decode over Q8_0 caches (34 bytes per 32 values), quantised on the device from the fp16 caches
+    q8 = GGMLQuantizationType.Q8_0
+    q8b, q8s = GGML_QUANT_SIZES[q8]
+    kq8, vq8 = workloads.q8_0_rows(kc), workloads.q8_0_rows(vc)
     del kc, vc
+    d8step = lambda: kerns.flash_attn_decode(q8, q8b, q8s, qd, kq8, vq8, ctx, outd)
+    for _ in range(max(args.warmup, 100)):
+        d8step()
+    torch.cuda.synchronize()
+    d8_avg_ms, d8_med_ms = ev.time_each(d8step, stream, min(max(args.steps, 20), 100))
+    d8bytes = workloads.decode_bytes_q8_0(ctx.tolist(), 32, 8, 128)
+    d8_gbs = d8bytes / (d8_avg_ms * 1e-3) / 1e9
+    del kq8, vq8
 
     # ---- the step before attention: rotary embedding, alone and fused with the cache append ----
     x = workloads.rope_input(seed=0, device=dev)                      # the reference test's shape
@@ -198,7 +212,17 @@ def main():
     a_avg_ms, a_med_ms = ev.time_each(astep, stream, 50)
     abytes = workloads.kv_append_bytes(8, 4096, 32, 8, 128, 128)
     a_gbs = abytes / (a_avg_ms * 1e-3) / 1e9
-    del aq, ak, av, akc, avc
+    del akc, avc
+    akq = torch.zeros(8, 8, 4096, 128 // 32 * 34, dtype=torch.uint8, device=dev)
+    avq = torch.zeros_like(akq)
+    a8step = lambda: kerns.rope_kv_append(1, 128, 5e5, aq, ak, av, apos, akq, avq)
+    for _ in range(100):
+        a8step()
+    torch.cuda.synchronize()
+    a8_avg_ms, a8_med_ms = ev.time_each(a8step, stream, 50)
+    a8bytes = workloads.kv_append_bytes_q8_0(8, 4096, 32, 8, 128, 128)
+    a8_gbs = a8bytes / (a8_avg_ms * 1e-3) / 1e9
+    del aq, ak, av, akq, avq
     nshape = (8, 4096, 6144)                                          # the reference test's per-token shape
     nx, nw = workloads.rmsnorm_input(nshape, seed=0, device=dev)
     nout = torch.empty_like(nx)
@@ -240,6 +264,17 @@ def main():
                                 "kernel": "decode_split_kernel<F16,128> + decode_combine_kernel",
                                 "algorithmic_bytes": dbytes}},
     }
+    rec["decode_q8_0"] = {"value": d8_gbs, "unit": "GB/s", "ms": d8_avg_ms, "median_ms": d8_med_ms,
+                          "speedup_over_fp16_cache": d_avg_ms / d8_avg_ms,
+                          "workload": "the decode workload over Q8_0 caches, uint8 [64,8,8192,136] (34-byte blocks of 32 values), q/out fp16",
+                          "roofline": {"bound": "hbm", "achieved": d8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
+                                       "frac": d8_gbs / PEAK_HBM_GBS, "traffic": DECODE_Q8_TRAFFIC_BYTES,
+                                       "kernel": "decode_split_q8_kernel<128> + decode_combine_kernel",
+                                       "algorithmic_bytes": d8bytes}}
+    rec["rope_kv_append_q8_0"] = {"value": a8_gbs, "unit": "GB/s", "ms": a8_avg_ms, "median_ms": a8_med_ms,
+                                  "workload": "the rope_kv_append workload into Q8_0 caches, uint8 [8,8,4096,136]",
+                                  "roofline": {"bound": "hbm", "achieved": a8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a8_gbs / PEAK_HBM_GBS,
+                                               "traffic": APPEND_Q8_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,neox,fused append,Q8_0>", "algorithmic_bytes": a8bytes}}
     rec["rope"] = {"value": r_gbs, "unit": "GB/s", "ms": r_avg_ms, "median_ms": r_med_ms,
                    "workload": "il_rope in place, x [8,4096,48,128] fp16, rotary_dim 64, base 1e6, start_pos 2048 (reference test/kernels.py:76-96)",
                    "roofline": {"bound": "hbm", "achieved": r_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r_gbs / PEAK_HBM_GBS,

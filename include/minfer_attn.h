@@ -27,6 +27,7 @@ extern "C" {
  * (reference: src/minfer/const.py:4-35: F16 = 1, BF16 = 30). */
 #define MINFER_ATTN_F16 1
 #define MINFER_ATTN_BF16 30
+#define MINFER_ATTN_F32 0    /* only as the float side of minfer_quant_q8_0 / minfer_dequant_q8_0 */
 
 #define MINFER_ATTN_OK 0
 #define MINFER_ATTN_EINVAL (-1)    /* shape, stride, dtype or alignment rejected        */
@@ -156,6 +157,59 @@ int minfer_rmsnorm(int dtype, const void* in, const void* w, void* out, int64_t 
 int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
                 double alpha, double beta, void* stream);
+
+/*
+ * Q8_0 blocks: 32 consecutive values of a row as an fp16 scale d followed by 32 int8, 34 bytes, no padding
+ * (reference: src/minfer/kernels/torch_ext/csrc/common/types.hpp:141-146; GGML type 8, sizes const.py:46).
+ */
+#define MINFER_Q8_0 8
+#define MINFER_Q8_0_BLOCK 32        /* values per block */
+#define MINFER_Q8_0_BLOCK_BYTES 34  /* bytes per block  */
+
+/*
+ * Quantises n_rows contiguous rows of k values (k a multiple of 32) into rows of k/32 blocks: per block
+ * d = max|x| / 127, q = roundf(x / d) (ties away from zero; all zero when d is), d stored as fp16.
+ * x is fp32 (MINFER_ATTN_F32), fp16 or bf16, 16-byte aligned; y 2-byte aligned.  Replaces quant_cpu's Q8_0
+ * case, which runs on the host (reference: csrc/quants/op.cpp:156-196, csrc/quants/impl.cpp:1169-1193), byte
+ * for byte on fp32 input.
+ */
+int minfer_quant_q8_0(int src_dtype, const void* x, void* y, int64_t n_rows, int64_t k, void* stream);
+
+/*
+ * The inverse: y[i] = (T)(q[i] * (float)d), T fp32 (MINFER_ATTN_F32) or fp16; x 2-byte aligned, y 16-byte
+ * aligned.  Replaces dequant_cuda's Q8_0 case and its kernel (reference: cuda/quants/op.cuh,
+ * cuda/quants/kernel.cuh:10-40, cuda/quants/impls.cuh:121-143), bit for bit.
+ */
+int minfer_dequant_q8_0(int dst_dtype, const void* x, void* y, int64_t n_rows, int64_t k, void* stream);
+
+/*
+ * minfer_flash_attn_decode over Q8_0 caches: q and out are fp16 [B,Hq,1,D] with element strides st->q0, q1 and
+ * st->o0, o1; k_cache and v_cache are [B,Hkv,Lmax] rows of D/32 blocks, 2-byte aligned, with st->kv0 and
+ * st->kv1 the BYTE strides of their first two dims (even) and st->kv2 = D/32 * 34 (rows are dense).  The kernel
+ * reads whole aligned 16-byte pieces, so up to 15 bytes on either side of a (sequence, head)'s rows, inside the
+ * same 16-byte lines, are read and ignored.  Every
+ * block is dequantised to fp16 exactly as minfer_dequant_q8_0 does and the result is that of
+ * minfer_flash_attn_decode on the dequantised cache; workspace as for minfer_flash_attn_decode.  This is what
+ * the reference's unused (qtype_int, qblock_size, qtype_size) operator arguments are for (reference:
+ * cuda/flash_attn/op.cuh:22-24); it has no kernel for it.
+ */
+int minfer_flash_attn_decode_q8_0(const void* q, const void* k_cache, const void* v_cache,
+                                  const int32_t* ctx_lens, void* out, int64_t B, int64_t Hq, int64_t Hkv,
+                                  int64_t Lmax, int64_t D, const minfer_attn_strides* st, void* workspace,
+                                  size_t workspace_bytes, void* stream);
+
+/*
+ * minfer_rope_kv_append into Q8_0 caches: q is rotated in place as there; the rotated k and v, rounded to
+ * `dtype` as an fp16/bf16 cache would hold them, are quantised as minfer_quant_q8_0 does and written to row
+ * positions[b] + l of caches laid out as minfer_flash_attn_decode_q8_0 reads them (cache_stride_b,
+ * cache_stride_h in bytes, even; rows dense).  D must be a multiple of 32 and rotary_dim of 32 (interleaved)
+ * or 64 (NeoX); q, k, v 16-byte aligned, caches 2-byte aligned.  No counterpart in the reference.
+ */
+int minfer_rope_kv_append_q8_0(int dtype, int style, void* q, const void* k, const void* v,
+                               const int32_t* positions, void* k_cache, void* v_cache,
+                               int64_t B, int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
+                               int64_t cache_stride_b, int64_t cache_stride_h,
+                               int64_t rotary_dim, double freq_base, void* stream);
 
 #ifdef __cplusplus
 }

@@ -63,6 +63,28 @@ def flash_attn_decode(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def flash_attn_decode_q8_0(backend: str, which: str, workload: str, repeat: int):
+    """The decode workload over Q8_0 caches (quantised on the device from the same fp16 caches); `ref` attends the
+    dequantised caches with the fp16 decode op."""
+    kerns = KernelBackend(backend)
+    q, kc, vc, ctx = workloads.decode_cache(device="cuda")
+    out = torch.zeros_like(q)
+    q8 = GGMLQuantizationType.Q8_0
+    kq, vq = workloads.q8_0_rows(kc), workloads.q8_0_rows(vc)
+    if which == "minfer":
+        del kc, vc
+        fn = lambda: kerns.flash_attn_decode(q8, *GGML_QUANT_SIZES[q8], q, kq, vq, ctx, out)
+    else:
+        k16, v16 = torch.empty_like(kc), torch.empty_like(vc)
+        kerns._dequant(q8, *GGML_QUANT_SIZES[q8], kq.view(-1, kq.shape[-1]), k16.view(-1, 128))
+        kerns._dequant(q8, *GGML_QUANT_SIZES[q8], vq.view(-1, vq.shape[-1]), v16.view(-1, 128))
+        fn = lambda: kerns.flash_attn_decode(QT, QB, QS, q, k16, v16, ctx, out)
+    with torch.no_grad():
+        for _ in range(repeat):
+            fn()
+    torch.cuda.synchronize()
+
+
 def flash_attn_varlen(backend: str, which: str, workload: str, repeat: int):
     kerns = KernelBackend(backend)
     q, k, v, cu = workloads.ragged_prefill(device="cuda")
@@ -106,6 +128,39 @@ def rope_kv_append(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def rope_kv_append_q8_0(backend: str, which: str, workload: str, repeat: int):
+    """rope_kv_append at the same shape into Q8_0 caches."""
+    kerns = KernelBackend(backend)
+    q, k, v, pos, kc, vc = workloads.kv_append(device="cuda", B=8, L=4096)
+    kq = torch.zeros(kc.shape[:-1] + (kc.shape[-1] // 32 * 34,), dtype=torch.uint8, device="cuda")
+    vq = torch.zeros_like(kq)
+    if which == "minfer":
+        fn = lambda: kerns.rope_kv_append(1, 128, 5e5, q, k, v, pos, kq, vq)
+    else:
+        q8 = GGMLQuantizationType.Q8_0
+
+        def fn():
+            kerns.rope_kv_append(1, 128, 5e5, q, k, v, pos, kc, vc)
+            kerns._quant(q8, *GGML_QUANT_SIZES[q8], kc.view(-1, 128), kq.view(-1, kq.shape[-1]))
+            kerns._quant(q8, *GGML_QUANT_SIZES[q8], vc.view(-1, 128), vq.view(-1, vq.shape[-1]))
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
+def quant(backend: str, which: str, workload: str, repeat: int):
+    """The reference test's larger shape (reference: test/kernels.py:25): fp32 [16384, 6144] into Q8_0 rows and back."""
+    kerns = KernelBackend(backend)
+    q8 = GGMLQuantizationType.Q8_0
+    x = torch.randn(16384, 6144, device="cuda")
+    y = torch.empty(16384, 6144 // 32 * 34, dtype=torch.uint8, device="cuda")
+    back = torch.empty_like(x)
+    for _ in range(repeat):
+        kerns._quant(q8, *GGML_QUANT_SIZES[q8], x, y)
+        kerns._dequant(q8, *GGML_QUANT_SIZES[q8], y, back)
+    torch.cuda.synchronize()
+
+
 def rmsnorm(backend: str, which: str, workload: str, repeat: int):
     """The reference test's shapes (reference: test/kernels.py:60-63): per token [8,4096,6144] (default) or,
     with --workload reference, per head [8,4096,48,128]."""
@@ -141,7 +196,8 @@ def copy(backend: str, which: str, workload: str, repeat: int):
 
 if __name__ == "__main__":
     KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
-               "il_rope": il_rope, "rope_kv_append": rope_kv_append, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
+               "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "il_rope": il_rope, "rope_kv_append": rope_kv_append,
+               "rope_kv_append_q8_0": rope_kv_append_q8_0, "quant": quant, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)

@@ -75,6 +75,24 @@ def decode_cache(seed=0, device="cpu", B=64, Hq=32, Hkv=8, Lmax=8192, D=128, dty
     return q, kc, vc, ctx
 
 
+def q8_0_rows(x):
+    """Device tensor [..., D] (D a multiple of 32) -> its rows as Q8_0 blocks, uint8 [..., D/32*34], quantised on the
+    device by the library's own quantiser (reference format: common/types.hpp:141-146)."""
+    from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
+    from minfer.kernels import KernelBackend
+    qt = GGMLQuantizationType.Q8_0
+    D = x.shape[-1]
+    y = torch.empty(x.shape[:-1] + (D // 32 * 34,), dtype=torch.uint8, device=x.device)
+    KernelBackend("torch_ext")._quant(qt, *GGML_QUANT_SIZES[qt], x.reshape(-1, D), y.view(-1, D // 32 * 34))
+    return y
+
+
+def decode_bytes_q8_0(ctx_lens, Hq, Hkv, D):
+    """K and V rows of D/32 34-byte blocks read once per KV head, plus fp16 q and out."""
+    B = len(ctx_lens)
+    return int(sum(int(c) for c in ctx_lens)) * Hkv * (D // 32 * 34) * 2 + 2 * B * Hq * D * 2
+
+
 def ragged_prefill(seed=0, device="cpu", n_seqs=16, len_lo=128, len_hi=2048, Hq=64, Hkv=8, D=128,
                    dtype=torch.float16, scale=1.0):
     """Packed sequences with lengths uniform in [len_lo, len_hi]: q [1,Hq,T,D], k/v [1,Hkv,T,D] ~ N(0,1),
@@ -136,6 +154,11 @@ def rope_bytes(B, L, H, rotary_dim, itemsize=2):
 def kv_append_bytes(B, L, Hq, Hkv, D, rotary_dim, itemsize=2):
     """q's rotary part read and written; k and v read once; their cache rows written once."""
     return (2 * B * L * Hq * rotary_dim + 4 * B * L * Hkv * D) * itemsize
+
+
+def kv_append_bytes_q8_0(B, L, Hq, Hkv, D, rotary_dim, itemsize=2):
+    """As kv_append_bytes, with the cache rows written as D/32 blocks of 34 bytes."""
+    return B * L * (2 * Hq * rotary_dim * itemsize + 2 * Hkv * D * itemsize + 2 * Hkv * (D // 32 * 34))
 
 
 def rmsnorm_input(shape=(8, 4096, 6144), seed=0, device="cpu", dtype=torch.float16):

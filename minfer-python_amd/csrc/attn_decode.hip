@@ -18,8 +18,19 @@
 //
 // Every (sequence, head, chunk) writes an un-normalised fp32 partial (O, max, sum) to the
 // workspace; the combine kernel merges the chunks of a row with the usual log-sum-exp weights.
+//
+// Q8_0 caches (decode_split_q8_kernel): a cache row is D/32 blocks of 34 bytes, an fp16 scale d followed by
+// 32 int8 (reference: src/minfer/kernels/torch_ext/csrc/common/types.hpp:141-146), so blocks start on 2-byte
+// boundaries.  Global memory is read in aligned 16-byte pieces all the same (2-byte-aligned wide loads run at a
+// fraction of the rate): a wave's ring holds 32-row groups as the flat run of aligned pieces that covers them,
+// the pieces are dropped into the wave's LDS area, and every lane picks its own blocks out of it with 2-byte
+// aligned LDS reads.  A block becomes the 32 fp16 values (half)(q * d) the reference's dequantiser produces
+// (reference: cuda/quants/impls.cuh:121-143).  K needs no further LDS pass: lane (key, quad) holds values
+// D/4 * quad .. of its key, which is a valid MFMA contraction order as long as Q^T is loaded in the same
+// order.  V is parked as fp16 rows and read back transposed, as on the fp16 path.
 #include "attn_common.h"
 #include "attn_host.h"
+#include "quant_q8.h"
 
 namespace minfer_attn {
 
@@ -270,6 +281,277 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     }
 }
 
+// ---- decode over Q8_0 caches -----------------------------------------------------------------------
+#ifndef MINFER_DECODE_STAGES_Q8
+#define MINFER_DECODE_STAGES_Q8 2
+#endif
+constexpr int kDecodeStagesQ8 = MINFER_DECODE_STAGES_Q8;   // ring depth, in 32-row groups
+constexpr int kGroupRowsQ8 = 32;
+
+template <int D> struct DecodeGeomQ8 {
+    static constexpr int BPR = D / 32;                        // blocks per cache row
+    static constexpr int ROWB = BPR * 34;                     // bytes per cache row
+    static constexpr int RAWB = kGroupRowsQ8 * ROWB;          // bytes of a group's K (or V) rows, a multiple of 16
+    static constexpr int NG = (RAWB + 14 + 15) / 16;          // aligned 16-byte pieces that cover them (base any even address)
+    static constexpr int NL = (NG + 63) / 64;                 // wave-wide loads per group and tensor
+    static constexpr int RAW_LDS = NG * 16;
+    static constexpr int RB = D * 2;                          // bytes of a parked fp16 row
+    static constexpr int PARK = kGroupRowsQ8 * RB;
+    static constexpr int PS = D + 4;                          // floats per head in a wave's partial result
+    static constexpr int PART = 16 * PS * 4;
+    static constexpr int WAVE_LDS = (2 * RAW_LDS + PARK > PART ? 2 * RAW_LDS + PARK : PART);
+};
+
+// kv0/kv1 of DecodeParams are byte strides here; q and out are fp16.
+template <int D>
+__global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD) void decode_split_q8_kernel(const DecodeParams p) {
+    using T = F16;
+    using GEO = DecodeGeom<D>;
+    using Q = DecodeGeomQ8<D>;
+    constexpr int RB = Q::RB, BPR = Q::BPR, ROWB = Q::ROWB, NL = Q::NL, NG = Q::NG;
+    constexpr int KC = D / 32;   // 32-wide contraction steps of K Q^T
+    constexpr int DB = D / 16;   // 16-row blocks of O^T
+    constexpr int NS = kDecodeStagesQ8;
+    constexpr int PS = Q::PS;
+    constexpr int GR = kGroupRowsQ8;
+
+    __shared__ __attribute__((aligned(1024))) char lds[kDecodeWaves][(Q::WAVE_LDS + 1023) / 1024 * 1024];
+
+    const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
+    const int l16 = lane & 15, quad = lane >> 4;
+    const int per_chunk = p.Hkv * p.n_hg;
+    const int y = blockIdx.x % per_chunk;
+    const int g = y % p.Hkv, hg = y / p.Hkv;
+    int b, split, ctx_raw;
+    if (!locate_chunk(p, blockIdx.x / per_chunk, lane, b, split, ctx_raw)) return;   // past the last chunk
+
+    const int ctx = min(max(ctx_raw, 0), p.Lmax);
+    const int row_lo = split * p.chunk;                      // a multiple of 64
+    const int row_hi = min(row_lo + p.chunk, ctx);
+    const int n_groups = (row_hi - row_lo + GR - 1) / GR;
+    const int my_groups = (n_groups - w + kDecodeWaves - 1) / kDecodeWaves;  // groups w, w+4, ...
+    auto group_of = [&](int t) { return w + t * kDecodeWaves; };
+    auto wave_has_work = [&](int ww) { return ww < n_groups; };
+
+    const int heads_here = min(16, p.n_rep - hg * 16);
+    const int head0 = g * p.n_rep + hg * 16;
+    char* raw_k = lds[w];
+    char* raw_v = lds[w] + Q::RAW_LDS;
+    char* park_v = lds[w] + 2 * Q::RAW_LDS;
+
+    // The (sequence, KV head)'s rows start at kb; pieces are counted from the 16-byte boundary at or below it.
+    // (plain pointer arithmetic, so that the loads below stay global-memory loads)
+    const char* kb = (const char*)p.k + ((int64_t)b * p.kv0 + (int64_t)g * p.kv1);
+    const char* vb = (const char*)p.v + ((int64_t)b * p.kv0 + (int64_t)g * p.kv1);
+    const int pre_k = (int)((uintptr_t)kb & 15), pre_v = (int)((uintptr_t)vb & 15);   // even, wave-uniform
+    const char* kb16 = kb - pre_k;
+    const char* vb16 = vb - pre_v;
+    // last piece that holds a byte of the chunk's rows, relative to the aligned base
+    const int64_t last_k = ((int64_t)pre_k + (int64_t)row_hi * ROWB - 1) & ~(int64_t)15;
+    const int64_t last_v = ((int64_t)pre_v + (int64_t)row_hi * ROWB - 1) & ~(int64_t)15;
+
+    // ---- Q^T fragments (B operand): column = head l16; step s takes d = D/4 * quad + 8s + 0..7, the order in
+    // which the K fragments below come out of a lane's share of its key's row
+    s16x8 qf[KC];
+    {
+        const bool valid = l16 < heads_here;
+        const short* src = (const short*)p.q + (int64_t)b * p.q0 + (int64_t)(head0 + (valid ? l16 : 0)) * p.q1 + (D / 4) * quad;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) {
+            s16x8 x = *reinterpret_cast<const s16x8*>(src + 8 * c);
+            if (!valid) x = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            qf[c] = x;
+        }
+    }
+
+    // ring of groups in flight: piece 64j + lane of the group's K bytes and of its V bytes
+    struct Stage { u32x4 k[NL], v[NL]; };
+    Stage ring[NS];
+    // Pieces past the chunk's last one re-read that one (and land on its LDS slot again); ring slots past the
+    // wave's last group have every lane re-read one piece of the last group, which costs one cache line.  The
+    // loop body stays straight-line code that way, which lets the compiler's wait counts keep NS-1 groups in flight.
+    auto piece_offset = [&](int t, int j, int64_t last, int64_t& group_off) {
+        const bool real = group_of(t) < n_groups;
+        const int grp = min(group_of(t), n_groups - 1);
+        group_off = (int64_t)(row_lo + grp * GR) * ROWB;              // a multiple of 16, wave-uniform
+        // the group's own pieces only (they are what its LDS area holds), and none past the chunk's last one
+        const int rel_last = real ? (int)min(last - group_off, (int64_t)16 * (NG - 1)) : 0;   // >= 0
+        return min(16 * (64 * j + lane), rel_last);
+    };
+    auto load_group = [&](int t, Stage& st) {
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            int64_t goff;
+            const int off = piece_offset(t, j, last_k, goff);
+            st.k[j] = *reinterpret_cast<const u32x4*>(kb16 + goff + off);
+        }
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            int64_t goff;
+            const int off = piece_offset(t, j, last_v, goff);
+            st.v[j] = *reinterpret_cast<const u32x4*>(vb16 + goff + off);
+        }
+    };
+#pragma unroll
+    for (int s = 0; s < NS; ++s) load_group(s, ring[s]);
+
+    f32x4 o_acc[DB];
+#pragma unroll
+    for (int db = 0; db < DB; ++db) o_acc[db] = f32x4{0.f, 0.f, 0.f, 0.f};
+    float m_ref = -INFINITY, l_sum = 0.f;
+    const float c2 = p.scale_log2;
+    constexpr float kLazyLog2 = 6.f;
+
+    // A block sits at an even offset of a raw area and is read as the aligned words that cover it (2-byte aligned
+    // LDS reads stall for tens of cycles): whether it starts on a word or in the middle of one is a property of
+    // the lane, fixed for the whole kernel (rows and 64-block strides are multiples of 4 bytes).
+    const bool k_odd = ((pre_k + (D == 128 ? quad : quad >> 1) * 34) & 2) != 0;
+    const bool v_odd = ((pre_v + lane * 34) & 2) != 0;
+    const uint32_t k_sel_a = k_odd ? kQ8SelOddA : kQ8SelEvenA, k_sel_b = k_odd ? kQ8SelOddB : kQ8SelEvenB;
+    const uint32_t v_sel_a = v_odd ? kQ8SelOddA : kQ8SelEvenA, v_sel_b = v_odd ? kQ8SelOddB : kQ8SelEvenB;
+    // the block's scale from its first memory word (zero for rows past the chunk's end, whose bytes were never loaded)
+    auto scale_of = [&](uint32_t w0, bool odd, bool row_ok) {
+        const uint16_t bits = (uint16_t)(odd ? w0 >> 16 : w0);
+        const _Float16 dh = row_ok ? __builtin_bit_cast(_Float16, bits) : (_Float16)0.f;
+        return h16x2{dh, dh};
+    };
+
+    auto consume = [&](int t, const Stage& st) {
+        const int r0 = row_lo + group_of(t) * GR;
+        int64_t goff;
+        // ---- the group's pieces into the wave's raw areas ----------------------------------------------
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            const int off = piece_offset(t, j, last_k, goff);
+            *reinterpret_cast<u32x4*>(raw_k + off) = st.k[j];
+        }
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            const int off = piece_offset(t, j, last_v, goff);
+            *reinterpret_cast<u32x4*>(raw_v + off) = st.v[j];
+        }
+        // ---- S^T = K Q^T for the two 16-key halves: lane gets head l16, keys 16h + 4*quad + r ---------------
+        f32x4 s[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = 16 * h + l16;
+            // the lane's share of its key's row: D/4 values starting at D/4 * quad (one block at D = 128, half a block at 64)
+            const int at = pre_k + row * ROWB + (D == 128 ? quad : quad >> 1) * 34;
+            const uint32_t* wp = reinterpret_cast<const uint32_t*>(raw_k + (at & ~3));
+            const h16x2 d2 = scale_of(wp[0], k_odd, r0 + row < row_hi);
+            constexpr int NW = D / 16;                       // quant words of the lane's share
+            const uint32_t* qp = wp + (D == 128 ? 0 : 4 * (quad & 1));
+            uint32_t wq[NW + 1];
+#pragma unroll
+            for (int i = 0; i <= NW; ++i) wq[i] = qp[i];
+            s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KC; ++c)
+                s[h] = T::mfma16(dequant8_shifted(wq[2 * c], wq[2 * c + 1], wq[2 * c + 2], k_sel_a, k_sel_b, d2), qf[c], s[h]);
+            const int key0 = r0 + 16 * h + 4 * quad;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s[h][r] = (key0 + r < row_hi) ? s[h][r] : -INFINITY;
+        }
+        // ---- V: every lane dequantises GR * BPR / 64 blocks and parks them as fp16 rows (swizzled) ----------
+#pragma unroll
+        for (int i = 0; i < GR * BPR / 64; ++i) {
+            const int idx = 64 * i + lane, row = idx / BPR, c = idx % BPR;
+            const int at = pre_v + idx * 34;
+            const uint32_t* wp = reinterpret_cast<const uint32_t*>(raw_v + (at & ~3));
+            uint32_t wv[9];
+#pragma unroll
+            for (int j = 0; j < 9; ++j) wv[j] = wp[j];
+            const h16x2 d2 = scale_of(wv[0], v_odd, r0 + row < row_hi);
+            char* rowp = park_v + row * RB;
+            const int sw = GEO::swz_v(row);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                *reinterpret_cast<s16x8*>(rowp + 16 * ((4 * c + j) ^ sw)) =
+                    dequant8_shifted(wv[2 * j], wv[2 * j + 1], wv[2 * j + 2], v_sel_a, v_sel_b, d2);
+        }
+        // ---- online softmax over this group's 32 keys ----------------------------------------------------
+        float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])), fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));
+        mx = fmaxf(mx, __shfl_xor(mx, 16));
+        mx = fmaxf(mx, __shfl_xor(mx, 32));
+        const bool grow = (mx - m_ref) * c2 > kLazyLog2 || (m_ref == -INFINITY && mx > -INFINITY);
+        if (__any(grow)) {
+            const float m_new = grow ? mx : m_ref;
+            const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2((m_ref - m_new) * c2);
+            m_ref = m_new;
+            l_sum *= alpha;
+#pragma unroll
+            for (int db = 0; db < DB; ++db) o_acc[db] *= alpha;
+        }
+        const float mc = (m_ref == -INFINITY) ? 0.f : m_ref * c2;
+        uint4 pu;
+        {
+            uint32_t pk[4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                pk[2 * h] = T::pack2(fast_exp2(fmaf(s[h][0], c2, -mc)), fast_exp2(fmaf(s[h][1], c2, -mc)));
+                pk[2 * h + 1] = T::pack2(fast_exp2(fmaf(s[h][2], c2, -mc)), fast_exp2(fmaf(s[h][3], c2, -mc)));
+            }
+            pu = uint4{pk[0], pk[1], pk[2], pk[3]};
+            l_sum = T::add_pair(pk[3], T::add_pair(pk[2], T::add_pair(pk[1], T::add_pair(pk[0], l_sum))));   // the rounded weights
+        }
+        const s16x8 pfrag = __builtin_bit_cast(s16x8, pu);   // contraction index j: key 4*quad + j (j < 4), 16 + 4*quad + j - 4
+        // ---- O^T += V^T P^T over the 32 keys: A = V^T block (row d = 16db + l16), same key order ---------------
+        {
+            const int row = 4 * quad + (l16 >> 2);
+            const char* rowp = park_v + row * RB;
+            const int sw = GEO::swz_v(row);         // rows 16 apart share a swizzle
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const int dcol = 16 * db + 4 * (l16 & 3);
+                const int at = 16 * ((dcol >> 3) ^ sw) + 2 * (dcol & 7);
+                const s16x4 a0 = lds_read_tr16(rowp + at);
+                const s16x4 a1 = lds_read_tr16(rowp + 16 * RB + at);
+                const s16x8 a = {a0[0], a0[1], a0[2], a0[3], a1[0], a1[1], a1[2], a1[3]};
+                o_acc[db] = T::mfma16(a, pfrag, o_acc[db]);
+            }
+        }
+    };
+
+    for (int t0 = 0; t0 < my_groups; t0 += NS) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            consume(t0 + s, ring[s]);
+            load_group(t0 + s + NS, ring[s]);
+        }
+    }
+
+    // ---- merge the four waves' partial results through LDS (over the wave's own areas), write the chunk's partial
+    l_sum += __shfl_xor(l_sum, 16);
+    l_sum += __shfl_xor(l_sum, 32);
+    float* mine = reinterpret_cast<float*>(lds[w]);   // [16 heads][PS]
+    if (l16 < heads_here) {
+#pragma unroll
+        for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(mine + l16 * PS + 16 * db + 4 * quad) = o_acc[db];
+        if (quad == 0) { mine[l16 * PS + D] = m_ref; mine[l16 * PS + D + 1] = l_sum; }
+    }
+    __syncthreads();
+    for (int idx = tid; idx < heads_here * D; idx += kDecodeWaves * 64) {
+        const int hh = idx / D, d = idx % D;
+        float M = -INFINITY;
+#pragma unroll
+        for (int ww = 0; ww < kDecodeWaves; ++ww)
+            if (wave_has_work(ww)) M = fmaxf(M, reinterpret_cast<const float*>(lds[ww])[hh * PS + D]);
+        float o = 0.f, l = 0.f;
+#pragma unroll
+        for (int ww = 0; ww < kDecodeWaves; ++ww) {
+            const float* src = reinterpret_cast<const float*>(lds[ww]) + hh * PS;
+            if (wave_has_work(ww) && src[D] > -INFINITY) {
+                const float wgt = fast_exp2((src[D] - M) * c2);
+                o += src[d] * wgt;
+                l += src[D + 1] * wgt;
+            }
+        }
+        const int64_t slot = ((int64_t)b * p.Hq + head0 + hh) * p.S + split;
+        p.part_o[slot * D + d] = o;
+        if (d == 0) { p.part_ml[slot * 2] = M; p.part_ml[slot * 2 + 1] = l; }
+    }
+}
+
 // out[b,h,:] = sum_s O_s w_s / sum_s l_s w_s with w_s = 2^((m_s - max m) * scale_log2).
 // One wave per (sequence, head) row; lane s holds chunk s's (max, sum), every lane owns D/64
 // output elements.  grid ceil(B*Hq/4), 256 threads.
@@ -359,6 +641,15 @@ static int launch_decode(const DecodeParams& p, void* out, int64_t o0, int64_t o
     return check_launch("decode_combine_kernel");
 }
 
+template <int D>
+static int launch_decode_q8(const DecodeParams& p, void* out, int64_t o0, int64_t o1, hipStream_t stream) {
+    const int64_t grid = (int64_t)p.B * p.S * p.Hkv * p.n_hg;
+    hipLaunchKernelGGL((decode_split_q8_kernel<D>), dim3((unsigned)grid), dim3(kDecodeWaves * 64), 0, stream, p);
+    if (int rc = check_launch("decode_split_q8_kernel")) return rc;
+    hipLaunchKernelGGL((decode_combine_kernel<F16, D>), dim3((p.B * p.Hq + 3) / 4), dim3(256), 0, stream, p, out, o0, o1);
+    return check_launch("decode_combine_kernel");
+}
+
 }  // namespace minfer_attn
 
 using namespace minfer_attn;
@@ -368,22 +659,17 @@ MINFER_ATTN_EXPORT size_t minfer_flash_attn_decode_workspace_bytes(int64_t B, in
     return decode_ws_bytes(B, Hq, Lmax, D);
 }
 
-MINFER_ATTN_EXPORT int minfer_flash_attn_decode(int dtype, const void* q, const void* k_cache, const void* v_cache,
-                                        const int32_t* ctx_lens, void* out, int64_t B, int64_t Hq, int64_t Hkv,
-                                        int64_t Lmax, int64_t D, const minfer_attn_strides* st, void* workspace,
-                                        size_t workspace_bytes, void* stream_v) {
-    clear_error();
-    if (int rc = check_common(dtype, q, k_cache, v_cache, out, Hq, Hkv, D, st)) return rc;
+// Fills the launch parameters both decode entry points share; returns an error code or MINFER_ATTN_OK.
+static int fill_decode(DecodeParams& p, const void* q, const void* k_cache, const void* v_cache, const int32_t* ctx_lens,
+                       int64_t B, int64_t Hq, int64_t Hkv, int64_t Lmax, int64_t D, const minfer_attn_strides* st,
+                       void* workspace, size_t workspace_bytes) {
     if (!ctx_lens) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: ctx_lens is null");
     if (B < 0 || Lmax < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: negative B or Lmax");
-    if (B == 0) return MINFER_ATTN_OK;
     if (B > 65535 || Hq > 65535) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: B or n_heads > 65535 unsupported");
     if (Lmax > (1 << 30)) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: Lmax too large");
+    if (B == 0) return MINFER_ATTN_OK;
     if (!workspace || workspace_bytes < decode_ws_bytes(B, Hq, Lmax, D) || !aligned16(workspace))
         return fail(MINFER_ATTN_EWORKSPACE, "flash_attn_decode: workspace too small or misaligned (see minfer_flash_attn_decode_workspace_bytes)");
-    hipStream_t stream = (hipStream_t)stream_v;
-
-    DecodeParams p{};
     p.q = q; p.k = k_cache; p.v = v_cache; p.ctx = ctx_lens;
     p.q0 = st->q0; p.q1 = st->q1; p.kv0 = st->kv0; p.kv1 = st->kv1; p.kv2 = st->kv2;
     p.B = (int)B; p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.n_rep = (int)(Hq / Hkv); p.Lmax = (int)Lmax;
@@ -397,8 +683,47 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode(int dtype, const void* q, const 
     const size_t o_bytes = (size_t)B * Hq * p.S * D * 4;
     p.part_o = (float*)workspace;
     p.part_ml = (float*)((char*)workspace + (o_bytes + 255) / 256 * 256);
+    return MINFER_ATTN_OK;
+}
+
+MINFER_ATTN_EXPORT int minfer_flash_attn_decode(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                                        const int32_t* ctx_lens, void* out, int64_t B, int64_t Hq, int64_t Hkv,
+                                        int64_t Lmax, int64_t D, const minfer_attn_strides* st, void* workspace,
+                                        size_t workspace_bytes, void* stream_v) {
+    clear_error();
+    if (int rc = check_common(dtype, q, k_cache, v_cache, out, Hq, Hkv, D, st)) return rc;
+    DecodeParams p{};
+    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes)) return rc;
+    if (B == 0) return MINFER_ATTN_OK;
+    hipStream_t stream = (hipStream_t)stream_v;
 
     if (dtype == MINFER_ATTN_F16)
         return D == 128 ? launch_decode<F16, 128>(p, out, st->o0, st->o1, stream) : launch_decode<F16, 64>(p, out, st->o0, st->o1, stream);
     return D == 128 ? launch_decode<BF16, 128>(p, out, st->o0, st->o1, stream) : launch_decode<BF16, 64>(p, out, st->o0, st->o1, stream);
+}
+
+MINFER_ATTN_EXPORT int minfer_flash_attn_decode_q8_0(const void* q, const void* k_cache, const void* v_cache,
+                                             const int32_t* ctx_lens, void* out, int64_t B, int64_t Hq, int64_t Hkv,
+                                             int64_t Lmax, int64_t D, const minfer_attn_strides* st, void* workspace,
+                                             size_t workspace_bytes, void* stream_v) {
+    clear_error();
+    if (D != 64 && D != 128) return fail(MINFER_ATTN_EINVAL, "head_dim must be 64 or 128");
+    if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0)
+        return fail(MINFER_ATTN_EINVAL, "n_heads must be a positive multiple of n_kv_heads");
+    if (!st) return fail(MINFER_ATTN_EINVAL, "strides is null");
+    if (!q || !k_cache || !v_cache || !out) return fail(MINFER_ATTN_EINVAL, "q, k_cache, v_cache and out must be non-null");
+    if (!aligned16(q) || !aligned16(out)) return fail(MINFER_ATTN_EINVAL, "q and out must be 16-byte aligned");
+    if (st->q0 % 8 || st->q1 % 8 || st->o0 % 8 || st->o1 % 8 || st->q0 < 0 || st->q1 < 0 || st->o0 < 0 || st->o1 < 0)
+        return fail(MINFER_ATTN_EINVAL, "strides of q and out must be non-negative multiples of 8 elements");
+    if (((uintptr_t)k_cache | (uintptr_t)v_cache) & 1u)
+        return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_q8_0: caches must be 2-byte aligned");
+    if (st->kv2 != D / 32 * 34)
+        return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_q8_0: cache rows must be dense (row stride = D/32 * 34 bytes)");
+    if (st->kv0 < 0 || st->kv1 < 0 || st->kv0 % 2 || st->kv1 % 2)
+        return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_q8_0: cache strides must be non-negative even byte counts");
+    DecodeParams p{};
+    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes)) return rc;
+    if (B == 0) return MINFER_ATTN_OK;
+    hipStream_t stream = (hipStream_t)stream_v;
+    return D == 128 ? launch_decode_q8<128>(p, out, st->o0, st->o1, stream) : launch_decode_q8<64>(p, out, st->o0, st->o1, stream);
 }

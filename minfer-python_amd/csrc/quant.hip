@@ -1,0 +1,132 @@
+// Q8_0 block quantisation for gfx950: rows of floats <-> rows of 34-byte blocks.
+//
+// A block holds 32 consecutive values of a row as an fp16 scale d followed by 32 int8
+// (reference: src/minfer/kernels/torch_ext/csrc/common/types.hpp:141-146).  Quantising (reference:
+// csrc/quants/impl.cpp:1169-1193, CPU only there): amax = max |x|, d = amax / 127, id = d ? 1 / d : 0,
+// q = roundf(x * id) (ties away from zero), d stored rounded to fp16.  Dequantising (reference:
+// cuda/quants/impls.cuh:121-143, csrc/quants/impl.cpp:1152-1167): y = (T)(q * (float)d).  Both are exact
+// restatements: IEEE division, one rounding per step, so the bytes equal the reference's.
+//
+// HBM-bound byte movers.  Four lanes share a block, eight values each (the amax goes through two
+// lane exchanges), so a wave reads 2 KB (fp32) or 1 KB (fp16) of contiguous input per step and writes 544
+// contiguous bytes; blocks start on 2-byte boundaries, which global accesses on this target allow.
+#include <algorithm>
+
+#include "attn_common.h"
+#include "attn_host.h"
+#include "quant_q8.h"
+
+namespace minfer_attn {
+
+constexpr int kQuantThreads = 256;
+
+// x: n_blocks * 32 values, contiguous; y: n_blocks * 34 bytes.  SRC: 0 fp32, 1 fp16, 2 bf16.
+template <int SRC>
+__global__ __launch_bounds__(kQuantThreads) void quant_q8_0_kernel(const void* x, char* y, int64_t n_blocks) {
+    const int64_t n_pieces = n_blocks * 4;
+    for (int64_t i = (int64_t)blockIdx.x * kQuantThreads + threadIdx.x; i < ((n_pieces + 3) & ~(int64_t)3);
+         i += (int64_t)gridDim.x * kQuantThreads) {
+        const bool on = i < n_pieces;   // a block's four lanes are on or off together (n_pieces is a multiple of 4)
+        float f[8];
+        if (SRC == 0) {
+            const f32x4* src = (const f32x4*)x + 2 * i;
+            const f32x4 a = on ? src[0] : f32x4{0.f, 0.f, 0.f, 0.f};
+            const f32x4 b = on ? src[1] : f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) { f[j] = a[j]; f[4 + j] = b[j]; }
+        } else {
+            const s16x8 a = on ? ((const s16x8*)x)[i] : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 8; ++j) f[j] = SRC == 1 ? F16::to_float(a[j]) : BF16::to_float(a[j]);
+        }
+        uint16_t d_bits;
+        const uint2 q = quant8_q8_0(f, d_bits);
+        if (on) {
+            char* blk = y + (i >> 2) * 34;
+            store_q8_piece(blk, (int)(i & 3) * 8, q, d_bits);
+        }
+    }
+}
+
+// x: n_blocks * 34 bytes; y: n_blocks * 32 values.  DST: 0 fp32, 1 fp16.
+template <int DST>
+__global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kernel(const char* x, void* y, int64_t n_blocks) {
+    const int64_t n_pieces = n_blocks * 4;
+    for (int64_t i = (int64_t)blockIdx.x * kQuantThreads + threadIdx.x; i < n_pieces; i += (int64_t)gridDim.x * kQuantThreads) {
+        const char* blk = (const char*)__builtin_assume_aligned(x + (i >> 2) * 34, 2);
+        uint16_t d_bits;
+        uint2 q;
+        __builtin_memcpy(&d_bits, blk, 2);
+        __builtin_memcpy(&q, blk + 2 + 8 * (i & 3), 8);
+        if (DST == 1) {
+            const _Float16 dh = __builtin_bit_cast(_Float16, d_bits);
+            const h16x2 d2 = {dh, dh};
+            ((s16x8*)y)[i] = dequant8(q.x, q.y, d2);
+        } else {
+            const float d = (float)__builtin_bit_cast(_Float16, d_bits);
+            f32x4 a, b;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                a[j] = (float)(int8_t)(q.x >> (8 * j)) * d;
+                b[j] = (float)(int8_t)(q.y >> (8 * j)) * d;
+            }
+            f32x4* dst = (f32x4*)y + 2 * i;
+            dst[0] = a;
+            dst[1] = b;
+        }
+    }
+}
+
+static int check_rows(const char* op, const void* x, const void* y, int64_t n_rows, int64_t k) {
+    char msg[160];
+    auto bad = [&](const char* what) {
+        snprintf(msg, sizeof msg, "%s: %s", op, what);
+        return fail(MINFER_ATTN_EINVAL, msg);
+    };
+    if (n_rows < 0 || k < 0) return bad("negative size");
+    if (k % 32 != 0) return bad("row length must be a multiple of 32 (the Q8_0 block)");
+    if (!x || !y) return bad("null pointer");
+    if (n_rows > 0 && k > 0 && n_rows > (INT64_C(1) << 56) / k) return bad("problem too large");
+    return MINFER_ATTN_OK;
+}
+
+static int grid_for(int64_t n_pieces) {
+    return (int)std::min<int64_t>((n_pieces + kQuantThreads - 1) / kQuantThreads, 256 * 32);
+}
+
+}  // namespace minfer_attn
+
+using namespace minfer_attn;
+
+MINFER_ATTN_EXPORT int minfer_quant_q8_0(int src_dtype, const void* x, void* y, int64_t n_rows, int64_t k, void* stream_v) {
+    clear_error();
+    if (src_dtype != MINFER_ATTN_F32 && src_dtype != MINFER_ATTN_F16 && src_dtype != MINFER_ATTN_BF16)
+        return fail(MINFER_ATTN_EINVAL, "quant_q8_0: source dtype must be MINFER_ATTN_F32, MINFER_ATTN_F16 or MINFER_ATTN_BF16");
+    if (int rc = check_rows("quant_q8_0", x, y, n_rows, k)) return rc;
+    if (!aligned16(x)) return fail(MINFER_ATTN_EINVAL, "quant_q8_0: x must be 16-byte aligned");
+    if ((uintptr_t)y & 1u) return fail(MINFER_ATTN_EINVAL, "quant_q8_0: y must be 2-byte aligned");
+    const int64_t n_blocks = n_rows * (k / 32);
+    if (n_blocks == 0) return MINFER_ATTN_OK;
+    hipStream_t stream = (hipStream_t)stream_v;
+    const dim3 grid(grid_for(n_blocks * 4)), block(kQuantThreads);
+    if (src_dtype == MINFER_ATTN_F32) hipLaunchKernelGGL((quant_q8_0_kernel<0>), grid, block, 0, stream, x, (char*)y, n_blocks);
+    else if (src_dtype == MINFER_ATTN_F16) hipLaunchKernelGGL((quant_q8_0_kernel<1>), grid, block, 0, stream, x, (char*)y, n_blocks);
+    else hipLaunchKernelGGL((quant_q8_0_kernel<2>), grid, block, 0, stream, x, (char*)y, n_blocks);
+    return check_launch("quant_q8_0_kernel");
+}
+
+MINFER_ATTN_EXPORT int minfer_dequant_q8_0(int dst_dtype, const void* x, void* y, int64_t n_rows, int64_t k, void* stream_v) {
+    clear_error();
+    if (dst_dtype != MINFER_ATTN_F32 && dst_dtype != MINFER_ATTN_F16)
+        return fail(MINFER_ATTN_EINVAL, "dequant_q8_0: destination dtype must be MINFER_ATTN_F32 or MINFER_ATTN_F16");
+    if (int rc = check_rows("dequant_q8_0", x, y, n_rows, k)) return rc;
+    if (!aligned16(y)) return fail(MINFER_ATTN_EINVAL, "dequant_q8_0: y must be 16-byte aligned");
+    if ((uintptr_t)x & 1u) return fail(MINFER_ATTN_EINVAL, "dequant_q8_0: x must be 2-byte aligned");
+    const int64_t n_blocks = n_rows * (k / 32);
+    if (n_blocks == 0) return MINFER_ATTN_OK;
+    hipStream_t stream = (hipStream_t)stream_v;
+    const dim3 grid(grid_for(n_blocks * 4)), block(kQuantThreads);
+    if (dst_dtype == MINFER_ATTN_F32) hipLaunchKernelGGL((dequant_q8_0_kernel<0>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+    else hipLaunchKernelGGL((dequant_q8_0_kernel<1>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+    return check_launch("dequant_q8_0_kernel");
+}

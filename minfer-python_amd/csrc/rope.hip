@@ -16,11 +16,14 @@
 // The fused producer does what the model does right before attention (reference: src/minfer/core.py:228-232,
 // cache layout core.py:105-127): rotate q in place, rotate k while copying it into the KV cache
 // [B, n_kv_heads, Lmax, head_dim] at row positions[b] + l, copy v into the cache.  k is read once and never
-// written back, the cache row is written once.
+// written back, the cache row is written once.  With Q8_0 caches (Q8 = true; rows of D/32 blocks of 34 bytes,
+// strides in bytes) the rotated k and the v values are quantised on the way, from the values an fp16/bf16 cache
+// would have held: the four lanes that hold a block's 32 values agree on its scale through two lane exchanges.
 #include <algorithm>
 
 #include "attn_common.h"
 #include "attn_host.h"
+#include "quant_q8.h"
 
 namespace minfer_attn {
 
@@ -33,7 +36,7 @@ struct RopeParams {
     void* x;                  // [B, L, H, D], rotated in place (q of the fused producer)
     const void* k;            // fused: [B, L, Hkv, D]
     const void* v;            // fused: [B, L, Hkv, D]
-    void* k_cache;            // fused: [B, Hkv, Lmax, D] with element strides c0, c1, c2
+    void* k_cache;            // fused: [B, Hkv, Lmax, D] with element strides c0, c1, c2 (Q8_0: byte strides)
     void* v_cache;
     const int32_t* positions; // fused: [B] first cache row of each sequence; otherwise null
     int64_t c0, c1, c2;
@@ -65,8 +68,9 @@ MA_DEV f32x2 table_entry(double inv_freq, int pos) {
 // head hd covers elements 8c..8c+7 (pairs 4c..4c+3), rd/8 chunks per head; NeoX style, chunk c covers
 // elements 8c..8c+7 and their partners rd/2 + 8c.., rd/16 chunks per head.  Sections, in order: q rotary,
 // then (fused only) k rotary, k tail (elements rd..D-1, copied), v (copied).
-template <class T, int STYLE, bool FUSED>
+template <class T, int STYLE, bool FUSED, bool Q8 = false>
 __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) {
+    static_assert(FUSED || !Q8, "only the fused producer writes a cache");
     __shared__ f32x2 tab[2][kMaxPairs];
     const int tid = threadIdx.x;
     const int half_rd = p.rd >> 1;
@@ -88,14 +92,18 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
         short* xq = (short*)p.x + (int64_t)tok * p.H * p.D;
         const short* xk = FUSED ? (const short*)p.k + (int64_t)tok * p.Hkv * p.D : nullptr;
         const short* xv = FUSED ? (const short*)p.v + (int64_t)tok * p.Hkv * p.D : nullptr;
-        short* ck = FUSED ? (short*)p.k_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
-        short* cv = FUSED ? (short*)p.v_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
+        // the token's cache row of head 0: element pointers, or byte pointers (Q8_0)
+        short* ck = FUSED && !Q8 ? (short*)p.k_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
+        short* cv = FUSED && !Q8 ? (short*)p.v_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
+        char* qk = Q8 ? (char*)p.k_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
+        char* qv = Q8 ? (char*)p.v_cache + (int64_t)b * p.c0 + (int64_t)pos * p.c2 : nullptr;
 
         // Where chunk t of the token lives: kind 0 rotate, 1 copy, 2 nothing.  Evaluated once to request the
         // chunk and again to store it (the index is made opaque in between), so that only the loaded data
         // stays in registers across the barrier.
-        auto locate = [&](int t, const short*& src, short*& dst, int& kind, int& chunk) __attribute__((always_inline)) {
-            src = xq; dst = xq; kind = 2; chunk = 0;
+        // For a Q8_0 cache, crow is the (row, head) the chunk belongs to and elem its first element there.
+        auto locate = [&](int t, const short*& src, short*& dst, int& kind, int& chunk, char*& crow, int& elem) __attribute__((always_inline)) {
+            src = xq; dst = xq; kind = 2; chunk = 0; crow = nullptr; elem = 0;
             if (t < n_q) {
                 const int hd = t / cph; chunk = t - hd * cph;
                 src = dst = xq + hd * p.D + 8 * chunk;
@@ -105,19 +113,22 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
                 if (t < n_kr) {
                     const int hd = t / cph; chunk = t - hd * cph;
                     src = xk + hd * p.D + 8 * chunk;
-                    dst = ck + hd * p.c1 + 8 * chunk;
+                    if (Q8) { crow = qk + hd * p.c1; elem = 8 * chunk; }
+                    else dst = ck + hd * p.c1 + 8 * chunk;
                     kind = 0;
                 } else if (t < n_kr + n_kt) {
                     t -= n_kr;
                     const int hd = t / tail, c = t - hd * tail;
                     src = xk + hd * p.D + p.rd + 8 * c;
-                    dst = ck + hd * p.c1 + p.rd + 8 * c;
+                    if (Q8) { crow = qk + hd * p.c1; elem = p.rd + 8 * c; }
+                    else dst = ck + hd * p.c1 + p.rd + 8 * c;
                     kind = 1;
                 } else {
                     t -= n_kr + n_kt;
                     const int per = p.D >> 3, hd = t / per, c = t - hd * per;
                     src = xv + hd * p.D + 8 * c;
-                    dst = cv + hd * p.c1 + 8 * c;
+                    if (Q8) { crow = qv + hd * p.c1; elem = 8 * c; }
+                    else dst = cv + hd * p.c1 + 8 * c;
                     kind = 1;
                 }
             }
@@ -128,20 +139,33 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
         auto request = [&](int t0) __attribute__((always_inline)) {
 #pragma unroll
             for (int u = 0; u < UN; ++u) {
-                const short* src; short* dst; int kind, chunk;
-                locate(t0 + u * kRopeThreads, src, dst, kind, chunk);
+                const short* src; short* dst; int kind, chunk, elem; char* crow;
+                locate(t0 + u * kRopeThreads, src, dst, kind, chunk, crow, elem);
                 lo[u] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
                 if (kind != 2) lo[u] = *reinterpret_cast<const s16x8*>(src);
                 hi[u] = lo[u];
                 if (STYLE == ROPE_NEOX && kind == 0) hi[u] = *reinterpret_cast<const s16x8*>(src + half_rd);
             }
         };
+        // 8 values to their place: as they are, or (Q8_0 cache) quantised with the block's three other lanes
+        auto put = [&](short* dst, char* crow, int elem, s16x8 val) __attribute__((always_inline)) {
+            if (Q8 && crow) {
+                float f[8];
+#pragma unroll
+                for (int j = 0; j < 8; ++j) f[j] = T::to_float(val[j]);
+                uint16_t d_bits;
+                const uint2 q = quant8_q8_0(f, d_bits);
+                store_q8_piece(crow + (elem >> 5) * 34, elem & 31, q, d_bits);
+            } else {
+                *reinterpret_cast<s16x8*>(dst) = val;
+            }
+        };
         auto finish = [&](int t0) __attribute__((always_inline)) {
             asm volatile("" : "+v"(t0));
 #pragma unroll
             for (int u = 0; u < UN; ++u) {
-                const short* src; short* dst; int kind, chunk;
-                locate(t0 + u * kRopeThreads, src, dst, kind, chunk);
+                const short* src; short* dst; int kind, chunk, elem; char* crow;
+                locate(t0 + u * kRopeThreads, src, dst, kind, chunk, crow, elem);
                 if (kind == 2) continue;
                 s16x8 a = lo[u];
                 if (kind == 0) {
@@ -162,10 +186,10 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
                             a[j] = (short)(pk & 0xffffu);
                             b[j] = (short)(pk >> 16);
                         }
-                        *reinterpret_cast<s16x8*>(dst + half_rd) = b;
+                        put(dst + half_rd, crow, elem + half_rd, b);
                     }
                 }
-                *reinterpret_cast<s16x8*>(dst) = a;
+                put(dst, crow, elem, a);
             }
         };
         // first batch of chunks requested, then the token's table while those loads are in flight
@@ -222,16 +246,16 @@ static bool vector_ok(int style, int64_t D, int64_t rd) {
     return D % 8 == 0 && rd % (style == ROPE_IL ? 8 : 16) == 0;
 }
 
-template <bool FUSED>
+template <bool FUSED, bool Q8 = false>
 static int launch_rope(int dtype, int style, const RopeParams& p, hipStream_t stream) {
     const int tokens = p.B * p.L;
     const int grid = std::min(tokens, 256 * 16);
     if (dtype == MINFER_ATTN_F16) {
-        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<F16, ROPE_IL, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
-        else hipLaunchKernelGGL((rope_kernel<F16, ROPE_NEOX, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<F16, ROPE_IL, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_kernel<F16, ROPE_NEOX, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
     } else {
-        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<BF16, ROPE_IL, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
-        else hipLaunchKernelGGL((rope_kernel<BF16, ROPE_NEOX, FUSED>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<BF16, ROPE_IL, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_kernel<BF16, ROPE_NEOX, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
     }
     return check_launch("rope_kernel");
 }
@@ -285,4 +309,28 @@ MINFER_ATTN_EXPORT int minfer_rope_kv_append(int dtype, int style, void* q, cons
     p.Hkv = (int)Hkv; p.Lmax = (int)Lmax;
     p.c0 = cache_stride_b; p.c1 = cache_stride_h; p.c2 = cache_stride_row;
     return launch_rope<true>(dtype, style, p, (hipStream_t)stream_v);
+}
+
+MINFER_ATTN_EXPORT int minfer_rope_kv_append_q8_0(int dtype, int style, void* q, const void* k, const void* v,
+                                                  const int32_t* positions, void* k_cache, void* v_cache, int64_t B,
+                                                  int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
+                                                  int64_t cache_stride_b, int64_t cache_stride_h, int64_t rotary_dim,
+                                                  double freq_base, void* stream_v) {
+    clear_error();
+    RopeParams p{};
+    if (int rc = fill_rope(p, dtype, style, B, L, Hq, D, rotary_dim, freq_base, "rope_kv_append_q8_0")) return rc;
+    if (!q || !k || !v || !positions || !k_cache || !v_cache) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_q8_0: null pointer");
+    if (Hkv <= 0 || Hkv > 65535 || Lmax < 0 || Lmax > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_q8_0: bad n_kv_heads or Lmax");
+    // a block's 32 values must sit in four neighbouring 8-value chunks of one kind
+    if (D % 32 != 0 || rotary_dim % (style == ROPE_IL ? 32 : 64) != 0)
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append_q8_0: head_dim must be a multiple of 32 and rotary_dim of 32 (interleaved) or 64 (NeoX)");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v)) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_q8_0: q, k and v must be 16-byte aligned");
+    if (((uintptr_t)k_cache | (uintptr_t)v_cache) & 1u) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_q8_0: caches must be 2-byte aligned");
+    if (cache_stride_b % 2 || cache_stride_h % 2 || cache_stride_b < 0 || cache_stride_h < 0)
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append_q8_0: cache strides must be non-negative even byte counts");
+    if (B == 0 || L == 0) return MINFER_ATTN_OK;
+    p.x = q; p.k = k; p.v = v; p.k_cache = k_cache; p.v_cache = v_cache; p.positions = positions;
+    p.Hkv = (int)Hkv; p.Lmax = (int)Lmax;
+    p.c0 = cache_stride_b; p.c1 = cache_stride_h; p.c2 = D / 32 * 34;
+    return launch_rope<true, true>(dtype, style, p, (hipStream_t)stream_v);
 }

@@ -110,6 +110,42 @@ void flash_attn_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size,
              "flash_attn");
 }
 
+// Decode over Q8_0 caches: uint8 [B, n_kv_heads, Lmax, HEAD_DIM/32 * 34], selected by the operator's
+// (qtype_int, qblock_size, qtype_size) = (8, 32, 34) (reference: the unused leading arguments of
+// flash_attn_cuda, cuda/flash_attn/op.cuh:22-24; sizes src/minfer/const.py:46).
+static void flash_attn_decode_q8_0(int64_t qblock_size, int64_t qtype_size, const Tensor& q, const Tensor& k_cache,
+                                   const Tensor& v_cache, const Tensor& ctx_lens, Tensor& out) {
+    STD_TORCH_CHECK(qblock_size == MINFER_Q8_0_BLOCK && qtype_size == MINFER_Q8_0_BLOCK_BYTES,
+                    "flash_attn_decode: Q8_0 has qblock_size 32 and qtype_size 34");
+    STD_TORCH_CHECK(q.dim() == 4 && k_cache.dim() == 4 && v_cache.dim() == 4 && out.dim() == 4 && ctx_lens.dim() == 1,
+                    "flash_attn_decode: q, k_cache, v_cache, out must be 4-D and ctx_lens 1-D");
+    STD_TORCH_CHECK(q.scalar_type() == ScalarType::Half && out.scalar_type() == ScalarType::Half,
+                    "flash_attn_decode: q and out must be float16 over Q8_0 caches");
+    STD_TORCH_CHECK(k_cache.scalar_type() == ScalarType::Byte && v_cache.scalar_type() == ScalarType::Byte,
+                    "flash_attn_decode: Q8_0 caches must be uint8");
+    STD_TORCH_CHECK(q.stride(-1) == 1 && k_cache.stride(-1) == 1 && v_cache.stride(-1) == 1 && out.stride(-1) == 1,
+                    "flash_attn_decode: tensors must be contiguous in their last dimension");
+    STD_TORCH_CHECK(k_cache.stride(0) == v_cache.stride(0) && k_cache.stride(1) == v_cache.stride(1) &&
+                    k_cache.stride(2) == v_cache.stride(2), "flash_attn_decode: k_cache and v_cache must share strides");
+    STD_TORCH_CHECK(ctx_lens.scalar_type() == ScalarType::Int && ctx_lens.is_contiguous(),
+                    "flash_attn_decode: ctx_lens must be contiguous int32");
+    STD_TORCH_CHECK(q.sizes().equals(out.sizes()), "flash_attn_decode: q and out shapes differ");
+    STD_TORCH_CHECK(k_cache.sizes().equals(v_cache.sizes()), "flash_attn_decode: cache shapes differ");
+    const int64_t B = q.size(0), Hq = q.size(1), Hkv = k_cache.size(1), Lmax = k_cache.size(2), D = q.size(3);
+    STD_TORCH_CHECK(D == 128 || D == 64, "flash_attn_decode: head_dim must be 128 or 64");
+    STD_TORCH_CHECK(q.size(2) == 1 && B == k_cache.size(0) && B == ctx_lens.size(0) &&
+                    k_cache.size(3) == D / 32 * 34 && k_cache.stride(2) == k_cache.size(3),
+                    "flash_attn_decode: expected q [B,Hq,1,D], caches [B,Hkv,Lmax,D/32*34] with dense rows, ctx_lens [B]");
+    if (B == 0) return;
+    const minfer_attn_strides st = strides_of(q, k_cache, out);   // a byte tensor's strides are byte strides
+    const size_t ws_bytes = minfer_flash_attn_decode_workspace_bytes(B, Hq, Lmax, D);
+    Tensor ws = byte_workspace(q, ws_bytes);
+    check_rc(minfer_flash_attn_decode_q8_0(q.const_data_ptr(), k_cache.const_data_ptr(), v_cache.const_data_ptr(),
+                                           static_cast<const int32_t*>(ctx_lens.const_data_ptr()), out.mutable_data_ptr(),
+                                           B, Hq, Hkv, Lmax, D, &st, ws.mutable_data_ptr(), ws_bytes, current_stream()),
+             "flash_attn_decode");
+}
+
 // Decode over a KV cache laid out like the reference's cache (reference: src/minfer/core.py:105-127).
 void flash_attn_decode_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size,
                            const Tensor& q,         // [B, n_heads, 1, HEAD_DIM]
@@ -117,9 +153,14 @@ void flash_attn_decode_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype
                            const Tensor& v_cache,   // [B, n_kv_heads, Lmax, HEAD_DIM]
                            const Tensor& ctx_lens,  // [B] int32
                            Tensor& out) {           // [B, n_heads, 1, HEAD_DIM]
-    (void)qtype_int; (void)qblock_size; (void)qtype_size;
     STD_TORCH_CHECK(on_gpu(q) && on_gpu(k_cache) && on_gpu(v_cache) && on_gpu(ctx_lens) && on_gpu(out),
                     "flash_attn_decode: all tensors must be on the GPU");
+    if (qtype_int == MINFER_Q8_0) {
+        flash_attn_decode_q8_0(qblock_size, qtype_size, q, k_cache, v_cache, ctx_lens, out);
+        return;
+    }
+    // any other value describes caches of q's own type, as the reference's callers pass it (F16 = 1)
+    STD_TORCH_CHECK(k_cache.scalar_type() != ScalarType::Byte, "flash_attn_decode: byte caches need qtype_int = 8 (Q8_0)");
     STD_TORCH_CHECK(q.dim() == 4 && k_cache.dim() == 4 && v_cache.dim() == 4 && out.dim() == 4 && ctx_lens.dim() == 1,
                     "flash_attn_decode: q, k_cache, v_cache, out must be 4-D and ctx_lens 1-D");
     STD_TORCH_CHECK(q.stride(-1) == 1 && k_cache.stride(-1) == 1 && v_cache.stride(-1) == 1 && out.stride(-1) == 1,
@@ -224,17 +265,29 @@ void rope_kv_append_hip(int64_t style, int64_t rotary_dim, double freq_base,
                     "rope_kv_append: q, k, v and the caches must be 4-D and positions 1-D");
     STD_TORCH_CHECK(q.is_contiguous() && k.is_contiguous() && v.is_contiguous(), "rope_kv_append: q, k and v must be contiguous");
     STD_TORCH_CHECK(style == MINFER_ROPE_INTERLEAVED || style == MINFER_ROPE_NEOX, "rope_kv_append: style must be 0 (interleaved) or 1 (NeoX)");
-    const int dtype = dtype_code(q, k, v, k_cache, "rope_kv_append");
-    STD_TORCH_CHECK(v_cache.scalar_type() == q.scalar_type(), "rope_kv_append: caches must share q's dtype");
+    const bool q8 = k_cache.scalar_type() == ScalarType::Byte;   // Q8_0 caches: [B, n_kv_heads, Lmax, head_dim/32 * 34] bytes
+    const int dtype = dtype_code(q, k, v, q8 ? q : k_cache, "rope_kv_append");
+    STD_TORCH_CHECK(v_cache.scalar_type() == k_cache.scalar_type(), "rope_kv_append: caches must share q's dtype, or both be uint8 (Q8_0)");
     STD_TORCH_CHECK(positions.scalar_type() == ScalarType::Int && positions.is_contiguous(), "rope_kv_append: positions must be contiguous int32");
     STD_TORCH_CHECK(k.sizes().equals(v.sizes()) && k_cache.sizes().equals(v_cache.sizes()), "rope_kv_append: k/v or cache shapes differ");
     STD_TORCH_CHECK(k_cache.stride(-1) == 1 && v_cache.stride(-1) == 1 && k_cache.stride(0) == v_cache.stride(0) &&
                     k_cache.stride(1) == v_cache.stride(1) && k_cache.stride(2) == v_cache.stride(2),
                     "rope_kv_append: caches must be contiguous in head_dim and share strides");
     STD_TORCH_CHECK(q.size(0) == k.size(0) && q.size(1) == k.size(1) && q.size(3) == k.size(3) && q.size(0) == k_cache.size(0) &&
-                    k.size(2) == k_cache.size(1) && q.size(3) == k_cache.size(3) && positions.size(0) == q.size(0),
-                    "rope_kv_append: expected q [B,L,Hq,D], k/v [B,L,Hkv,D], caches [B,Hkv,Lmax,D], positions [B]");
+                    k.size(2) == k_cache.size(1) && positions.size(0) == q.size(0) &&
+                    k_cache.size(3) == (q8 ? q.size(3) / 32 * 34 : q.size(3)) && (!q8 || q.size(3) % 32 == 0),
+                    "rope_kv_append: expected q [B,L,Hq,D], k/v [B,L,Hkv,D], caches [B,Hkv,Lmax,D] (or [B,Hkv,Lmax,D/32*34] bytes), positions [B]");
     STD_TORCH_CHECK(rotary_dim <= q.size(3), "rope_kv_append: rotary_dim exceeds head_dim");
+    if (q8) {
+        STD_TORCH_CHECK(k_cache.stride(2) == k_cache.size(3), "rope_kv_append: Q8_0 cache rows must be dense");
+        check_rc(minfer_rope_kv_append_q8_0(dtype, (int)style, q.mutable_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
+                                            static_cast<const int32_t*>(positions.const_data_ptr()), k_cache.mutable_data_ptr(),
+                                            v_cache.mutable_data_ptr(), q.size(0), q.size(1), q.size(2), k.size(2), q.size(3),
+                                            k_cache.size(2), k_cache.stride(0), k_cache.stride(1), rotary_dim, freq_base,
+                                            current_stream()),
+                 "rope_kv_append");
+        return;
+    }
     check_rc(minfer_rope_kv_append(dtype, (int)style, q.mutable_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
                                    static_cast<const int32_t*>(positions.const_data_ptr()), k_cache.mutable_data_ptr(),
                                    v_cache.mutable_data_ptr(), q.size(0), q.size(1), q.size(2), k.size(2), q.size(3),
@@ -334,8 +387,45 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
     }
 }
 
+// Same signatures and checks as the reference's dequant_cuda and quant_cpu (reference:
+// src/minfer/kernels/torch_ext/csrc/cuda/quants/op.cuh:25-78, csrc/quants/op.cpp:156-196), for the one block
+// format on this path, Q8_0; the quantiser runs on the device here.  x and y are 2-D, rows are whole blocks.
+void dequant_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size, const Tensor& x, Tensor& y) {
+    STD_TORCH_CHECK(qtype_int == MINFER_Q8_0, "dequant: only Q8_0 (qtype 8) is built here, got qtype ", qtype_int);
+    STD_TORCH_CHECK(qblock_size == MINFER_Q8_0_BLOCK && qtype_size == MINFER_Q8_0_BLOCK_BYTES, "dequant: Q8_0 has qblock_size 32 and qtype_size 34");
+    STD_TORCH_CHECK(on_gpu(x) && on_gpu(y), "dequant: x and y must be on the GPU");
+    STD_TORCH_CHECK(x.dim() == 2 && y.dim() == 2);
+    STD_TORCH_CHECK(x.size(0) == y.size(0), "x and y must have the same number of rows");
+    STD_TORCH_CHECK(x.scalar_type() == ScalarType::Byte, "x must be uint8 (byte)");
+    STD_TORCH_CHECK(y.scalar_type() == ScalarType::Float || y.scalar_type() == ScalarType::Half, "y must be float32 or float16");
+    STD_TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+    STD_TORCH_CHECK(y.is_contiguous(), "y must be contiguous");
+    STD_TORCH_CHECK(y.size(1) % 32 == 0 && x.size(1) == y.size(1) / 32 * 34, "dequant: x rows must hold y.size(1)/32 blocks of 34 bytes");
+    check_rc(minfer_dequant_q8_0(y.scalar_type() == ScalarType::Float ? MINFER_ATTN_F32 : MINFER_ATTN_F16, x.const_data_ptr(),
+                                 y.mutable_data_ptr(), y.size(0), y.size(1), current_stream()),
+             "dequant");
+}
+
+void quant_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size, const Tensor& x, Tensor& y) {
+    STD_TORCH_CHECK(qtype_int == MINFER_Q8_0, "quant: only Q8_0 (qtype 8) is built here, got qtype ", qtype_int);
+    STD_TORCH_CHECK(qblock_size == MINFER_Q8_0_BLOCK && qtype_size == MINFER_Q8_0_BLOCK_BYTES, "quant: Q8_0 has qblock_size 32 and qtype_size 34");
+    STD_TORCH_CHECK(on_gpu(x) && on_gpu(y), "quant: x and y must be on the GPU");
+    STD_TORCH_CHECK(x.dim() == 2 && y.dim() == 2);
+    STD_TORCH_CHECK(x.size(0) == y.size(0), "x and y must have same number of rows");
+    const ScalarType t = x.scalar_type();
+    STD_TORCH_CHECK(t == ScalarType::Float || t == ScalarType::Half || t == ScalarType::BFloat16, "x must be float32 (or float16 / bfloat16)");
+    STD_TORCH_CHECK(y.scalar_type() == ScalarType::Byte, "y must be uint8 (byte)");
+    STD_TORCH_CHECK(x.is_contiguous(), "x must be contiguous");
+    STD_TORCH_CHECK(y.is_contiguous(), "y must be contiguous");
+    STD_TORCH_CHECK(x.size(1) % 32 == 0 && y.size(1) == x.size(1) / 32 * 34, "quant: y rows must hold x.size(1)/32 blocks of 34 bytes");
+    const int src = t == ScalarType::Float ? MINFER_ATTN_F32 : t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16;
+    check_rc(minfer_quant_q8_0(src, x.const_data_ptr(), y.mutable_data_ptr(), x.size(0), x.size(1), current_stream()), "quant");
+}
+
 STABLE_TORCH_LIBRARY(minfer, m) {
     // verbatim the reference's schema (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:30)
+    m.def("dequant(int qtype, int qblock_size, int qtype_size, Tensor x, Tensor(a!) y) -> ()");
+    m.def("quant(int qtype, int qblock_size, int qtype_size, Tensor x, Tensor(a!) y) -> ()");
     m.def("flash_attn(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor(a!) mask, Tensor(a!) out) -> ()");
     // verbatim the reference's schemas (reference: src/minfer/kernels/torch_ext/csrc/reg.cpp:24-29)
     m.def("gemm(int qtype_int, int qblock_size, int qtype_size, float alpha, float beta, Tensor A, Tensor B, Tensor C, Tensor(a!) out) -> ()");
@@ -350,6 +440,8 @@ STABLE_TORCH_LIBRARY(minfer, m) {
 }
 
 STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-key name for ROCm devices too
+    m.impl("dequant", TORCH_BOX(&dequant_hip));
+    m.impl("quant", TORCH_BOX(&quant_hip));
     m.impl("flash_attn", TORCH_BOX(&flash_attn_hip));
     m.impl("flash_attn_decode", TORCH_BOX(&flash_attn_decode_hip));
     m.impl("flash_attn_varlen", TORCH_BOX(&flash_attn_varlen_hip));

@@ -1,13 +1,15 @@
 """Kernel facade, same shape as the reference's (reference: src/minfer/kernels/__init__.py:2-18):
-an attribute bag of callables for one backend.  Only the attention path and the normalisation,
-projection and rotary-embedding steps that feed it live here."""
+an attribute bag of callables for one backend.  Only the attention path, the normalisation,
+projection and rotary-embedding steps that feed it, and the Q8_0 quantisers of its KV cache live here."""
 
 
 class KernelBackend:
     def __init__(self, backend: str):
         if backend == "torch_ext":
-            from .torch_ext import (flash_attn, flash_attn_decode, flash_attn_varlen, gemm, il_rope, neox_rope,
-                                    qkv, rmsnorm, rope_kv_append)
+            from .torch_ext import (_dequant, _quant, flash_attn, flash_attn_decode, flash_attn_varlen, gemm, il_rope,
+                                    neox_rope, qkv, rmsnorm, rope_kv_append)
+            self._dequant = _dequant
+            self._quant = _quant
             self.rmsnorm = rmsnorm
             self.gemm = gemm
             self.qkv = qkv

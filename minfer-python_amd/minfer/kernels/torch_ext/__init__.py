@@ -10,3 +10,4 @@ except ImportError as e:  # pragma: no cover
     ) from e
 from .ops import (flash_attn, flash_attn_decode, flash_attn_varlen, gemm, il_rope, neox_rope,  # noqa: E402,F401
                   qkv, rmsnorm, rope_kv_append)
+from .ops import dequant as _dequant, quant as _quant  # noqa: E402,F401  (reference: torch_ext/__init__.py:2)

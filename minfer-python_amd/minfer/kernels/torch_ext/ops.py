@@ -5,6 +5,37 @@ to ``torch.ops.minfer.<op>.default``; the result is written into ``out``."""
 import torch
 
 _ACT_DTYPES = (torch.float16, torch.bfloat16)
+_Q8_0 = 8   # GGML type number of the one block format built here: 32 values in 34 bytes
+
+
+def dequant(qtype: int, qblock_size: int, qtype_size: int, x: torch.Tensor, y: torch.Tensor):
+    """Dequantises the rows of x (uint8 [M, N/32*34], Q8_0 blocks) into y (float32 or float16 [M, N]);
+    qblock_size is the number of values per block, qtype_size its bytes (reference: ops.py:8-21)."""
+    return torch.ops.minfer.dequant.default(qtype, qblock_size, qtype_size, x, y)
+
+
+@torch.library.register_fake("minfer::dequant")
+def _(qtype, qblock_size, qtype_size, x, y):
+    torch._check(x.dtype == torch.uint8)
+    torch._check(y.dtype in (torch.float32, torch.float16))
+    torch._check(x.device == y.device)
+    torch._check(x.device.type == "cuda")
+    torch._check(x.size(0) == y.size(0))
+
+
+def quant(qtype: int, qblock_size: int, qtype_size: int, x: torch.Tensor, y: torch.Tensor):
+    """Quantises the rows of x (float32 [M, N]; float16/bfloat16 also taken) into y (uint8 [M, N/32*34], Q8_0
+    blocks), on the device (reference: ops.py:33-46, CPU only there)."""
+    return torch.ops.minfer.quant.default(qtype, qblock_size, qtype_size, x, y)
+
+
+@torch.library.register_fake("minfer::quant")
+def _(qtype, qblock_size, qtype_size, x, y):
+    torch._check(x.dtype in (torch.float32, torch.float16, torch.bfloat16))
+    torch._check(y.dtype == torch.uint8)
+    torch._check(x.device == y.device)
+    torch._check(x.device.type == "cuda")
+    torch._check(x.size(0) == y.size(0))
 
 
 def flash_attn(
@@ -43,14 +74,16 @@ def flash_attn_decode(
     out: torch.Tensor,
 ):
     """Single-token decode: q/out [B,n_heads,1,D] against caches [B,n_kv_heads,Lmax,D]; query b
-    attends cache rows 0..ctx_lens[b]-1 (ctx_lens int32 [B])."""
+    attends cache rows 0..ctx_lens[b]-1 (ctx_lens int32 [B]).  With (qtype_int, qblock_size, qtype_size) =
+    (8, 32, 34) the caches are Q8_0 blocks, uint8 [B,n_kv_heads,Lmax,D/32*34], and q/out float16."""
     return torch.ops.minfer.flash_attn_decode.default(qtype_int, qblock_size, qtype_size, q, k_cache, v_cache, ctx_lens, out)
 
 
 @torch.library.register_fake("minfer::flash_attn_decode")
 def _(qtype_int, qblock_size, qtype_size, q, k_cache, v_cache, ctx_lens, out):
-    torch._check(q.dtype in _ACT_DTYPES)
-    torch._check(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and out.dtype == q.dtype)
+    torch._check(q.dtype in _ACT_DTYPES and out.dtype == q.dtype)
+    cache_dtype = torch.uint8 if qtype_int == _Q8_0 else q.dtype
+    torch._check(k_cache.dtype == cache_dtype and v_cache.dtype == cache_dtype)
     torch._check(ctx_lens.dtype == torch.int32)
     torch._check(q.device == k_cache.device == v_cache.device == ctx_lens.device == out.device)
     torch._check(q.device.type == "cuda")
@@ -123,14 +156,15 @@ def rope_kv_append(
 ):
     """Rotates q [B,L,n_heads,D] in place, writes the rotated k [B,L,n_kv_heads,D] and v into rows
     positions[b] + l of the caches [B,n_kv_heads,Lmax,D]; style 0 = interleaved, 1 = NeoX; positions
-    int32 [B]."""
+    int32 [B].  uint8 caches [B,n_kv_heads,Lmax,D/32*34] receive the rows as Q8_0 blocks."""
     return torch.ops.minfer.rope_kv_append.default(style, rotary_dim, freq_base, q, k, v, positions, k_cache, v_cache)
 
 
 @torch.library.register_fake("minfer::rope_kv_append")
 def _(style, rotary_dim, freq_base, q, k, v, positions, k_cache, v_cache):
     torch._check(q.dtype in _ACT_DTYPES)
-    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and k_cache.dtype == q.dtype and v_cache.dtype == q.dtype)
+    torch._check(k.dtype == q.dtype and v.dtype == q.dtype)
+    torch._check(k_cache.dtype in (q.dtype, torch.uint8) and v_cache.dtype == k_cache.dtype)
     torch._check(positions.dtype == torch.int32)
     torch._check(q.device.type == "cuda")
     torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and k_cache.dim() == 4 and v_cache.dim() == 4)

@@ -1,5 +1,5 @@
-"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c, rope_oracle.c, rmsnorm_oracle.c and
-gemm_oracle.c.
+"""TEST INFRASTRUCTURE ONLY: ctypes access to the CPU oracle in attn_oracle.c, rope_oracle.c, rmsnorm_oracle.c,
+gemm_oracle.c and quant_oracle.c.
 
 Only tests/, __graft_entry__.smoke() and the cpu_baseline leg of bench.py may import this
 package.  The shipped operator never does: it launches HIP kernels or raises.
@@ -39,8 +39,13 @@ def lib():
             build()
         _LIB = ctypes.CDLL(so)
         for name in ("oracle_flash_attn", "oracle_flash_attn_rows", "oracle_flash_attn_decode",
-                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append", "oracle_rmsnorm", "oracle_gemm"):
+                     "oracle_flash_attn_varlen", "oracle_rope", "oracle_rope_kv_append", "oracle_rmsnorm", "oracle_gemm",
+                     "oracle_quant_q8_0", "oracle_dequant_q8_0", "oracle_dequant_q8_0_f16"):
             getattr(_LIB, name).restype = ctypes.c_int
+        _LIB.oracle_f32_to_f16.restype = ctypes.c_uint16
+        _LIB.oracle_f32_to_f16.argtypes = [ctypes.c_float]
+        _LIB.oracle_f16_to_f32.restype = ctypes.c_float
+        _LIB.oracle_f16_to_f32.argtypes = [ctypes.c_uint16]
     return _LIB
 
 
@@ -198,3 +203,94 @@ def gemm(a, b, c, alpha, beta, b_layout=GEMM_B_KN):
     if rc != 0:
         raise ValueError(f"oracle_gemm rc={rc}")
     return out
+
+
+Q8_0_BLOCK, Q8_0_BLOCK_BYTES = 32, 34
+
+
+def quant_q8_0(x):
+    """Rows of floats [..., k] -> rows of Q8_0 blocks, uint8 [..., k/32*34] (reference:
+    csrc/quants/impl.cpp:1169-1193)."""
+    x = _f32(x)
+    k = x.shape[-1]
+    y = np.empty(x.shape[:-1] + (k // 32 * 34,), dtype=np.uint8)
+    rc = lib().oracle_quant_q8_0(_ptr(x), _ptr(y, ctypes.c_uint8), ctypes.c_int64(x.size // max(k, 1)), ctypes.c_int64(k))
+    if rc != 0:
+        raise ValueError(f"oracle_quant_q8_0 rc={rc}")
+    return y
+
+
+def dequant_q8_0(y, dtype=np.float32):
+    """Rows of Q8_0 blocks, uint8 [..., nb*34] -> values [..., nb*32] as float32 (q * d) or float16
+    ((half)(q * d)) (reference: csrc/quants/impl.cpp:1152-1167, cuda/quants/impls.cuh:121-143)."""
+    if hasattr(y, "detach"):
+        y = y.detach().to("cpu").numpy()
+    y = np.ascontiguousarray(np.asarray(y, dtype=np.uint8))
+    nbytes = y.shape[-1]
+    if nbytes % 34 != 0:
+        raise ValueError("row bytes must be a multiple of 34")
+    k = nbytes // 34 * 32
+    n_rows = y.size // max(nbytes, 1)
+    if np.dtype(dtype) == np.float16:
+        out = np.empty(y.shape[:-1] + (k,), dtype=np.uint16)
+        rc = lib().oracle_dequant_q8_0_f16(_ptr(y, ctypes.c_uint8), _ptr(out, ctypes.c_uint16), ctypes.c_int64(n_rows), ctypes.c_int64(k))
+        out = out.view(np.float16)
+    else:
+        out = np.empty(y.shape[:-1] + (k,), dtype=np.float32)
+        rc = lib().oracle_dequant_q8_0(_ptr(y, ctypes.c_uint8), _ptr(out), ctypes.c_int64(n_rows), ctypes.c_int64(k))
+    if rc != 0:
+        raise ValueError(f"oracle_dequant_q8_0 rc={rc}")
+    return out
+
+
+def flash_attn_decode_q8_0(q, k_cache_q8, v_cache_q8, ctx_lens):
+    """Decode attention over Q8_0 caches (uint8 [B,Hkv,Lmax,D/32*34]): the caches are dequantised to fp16 as
+    the reference's device dequantiser does, then attended as fp16 caches are."""
+    return flash_attn_decode(q, dequant_q8_0(k_cache_q8, np.float16), dequant_q8_0(v_cache_q8, np.float16), ctx_lens)
+
+
+_REF = None
+
+
+def ref_quants():
+    """The reference's own quantiser source compiled into oracle/_ref/libref_quants.so (make -C oracle ref), or
+    None when that library has not been built.  Returns (quant, dequant_f32, dequant_f16) taking numpy arrays."""
+    global _REF
+    so = os.path.join(_HERE, "_ref", "libref_quants.so")
+    if not os.path.exists(so):
+        return None
+    if _REF is None:
+        L = ctypes.CDLL(so)
+        qf = getattr(L, "_ZN6minfer4impl14quant_row_q8_0EPKfPhl")
+        d32 = getattr(L, "_ZN6minfer4impl16dequant_row_q8_0IfEEvPKhPT_l")
+        d16 = getattr(L, "_ZN6minfer4impl16dequant_row_q8_0IN3c104HalfEEEvPKhPT_l")
+        for f in (qf, d32, d16):
+            f.restype = None
+
+        def quant(x):
+            x = _f32(x)
+            k = x.shape[-1]
+            y = np.empty(x.shape[:-1] + (k // 32 * 34,), dtype=np.uint8)
+            qf(_ptr(x), _ptr(y, ctypes.c_uint8), ctypes.c_int64(x.size))   # rows are whole blocks: one long row
+            return y
+
+        def dequant32(y):
+            y = np.ascontiguousarray(y, dtype=np.uint8)
+            out = np.empty(y.shape[:-1] + (y.shape[-1] // 34 * 32,), dtype=np.float32)
+            d32(_ptr(y, ctypes.c_uint8), _ptr(out), ctypes.c_int64(out.size))
+            return out
+
+        def dequant16(y):
+            y = np.ascontiguousarray(y, dtype=np.uint8)
+            out = np.empty(y.shape[:-1] + (y.shape[-1] // 34 * 32,), dtype=np.uint16)
+            d16(_ptr(y, ctypes.c_uint8), _ptr(out, ctypes.c_uint16), ctypes.c_int64(out.size))
+            return out.view(np.float16)
+
+        _REF = (quant, dequant32, dequant16)
+    return _REF
+
+
+def build_ref():
+    """Compile oracle/_ref from the reference's source tree (only where that tree exists)."""
+    if os.path.isdir("/root/reference"):
+        subprocess.run(["make", "-C", _HERE, "ref"], check=True, stdout=subprocess.DEVNULL)

@@ -7,7 +7,8 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LIB_PATH = os.path.join(ROOT, "minfer-python_amd", "lib", "libminfer_attn.so")
 HEADER = os.path.join(ROOT, "include", "minfer_attn.h")
 
-F16, BF16 = 1, 30
+F16, BF16, F32 = 1, 30, 0
+Q8_0, Q8_0_BLOCK, Q8_0_BLOCK_BYTES = 8, 32, 34
 ROPE_INTERLEAVED, ROPE_NEOX = 0, 1
 GEMM_B_KN, GEMM_B_NK = 0, 1
 OK, EINVAL, EWORKSPACE, ELAUNCH = 0, -1, -2, -3
@@ -52,6 +53,16 @@ def lib():
         L.minfer_rmsnorm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, dbl, vp]
         L.minfer_gemm.restype = ctypes.c_int
         L.minfer_gemm.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, dbl, dbl, vp]
+        L.minfer_quant_q8_0.restype = ctypes.c_int
+        L.minfer_quant_q8_0.argtypes = [ctypes.c_int, vp, vp, i64, i64, vp]
+        L.minfer_dequant_q8_0.restype = ctypes.c_int
+        L.minfer_dequant_q8_0.argtypes = [ctypes.c_int, vp, vp, i64, i64, vp]
+        L.minfer_flash_attn_decode_q8_0.restype = ctypes.c_int
+        L.minfer_flash_attn_decode_q8_0.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
+                                                    ctypes.POINTER(Strides), vp, sz, vp]
+        L.minfer_rope_kv_append_q8_0.restype = ctypes.c_int
+        L.minfer_rope_kv_append_q8_0.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
+                                                 i64, i64, i64, i64, i64, dbl, vp]
         _lib = L
     return _lib
 
@@ -62,7 +73,7 @@ def last_error():
 
 def _dtype_code(t):
     import torch
-    return {torch.float16: F16, torch.bfloat16: BF16}[t.dtype]
+    return {torch.float16: F16, torch.bfloat16: BF16, torch.float32: F32}[t.dtype]
 
 
 def _strides(q, k, o):
@@ -138,3 +149,38 @@ def gemm(a, b, c, d, alpha, beta, b_layout=GEMM_B_KN):
     return lib().minfer_gemm(_dtype_code(a), b_layout, a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None,
                              d.data_ptr(), M, N, K, a.stride(0), b.stride(0), c.stride(0) if c is not None else N, d.stride(0),
                              alpha, beta, _stream())
+
+
+def quant_q8_0(x, y):
+    """Rows of contiguous x [n, k] (fp32, fp16 or bf16) into rows of Q8_0 blocks y, uint8 [n, k/32*34]."""
+    k = x.shape[-1]
+    return lib().minfer_quant_q8_0(_dtype_code(x), x.data_ptr(), y.data_ptr(), x.numel() // max(k, 1), k, _stream())
+
+
+def dequant_q8_0(x, y):
+    """Rows of Q8_0 blocks x, uint8 [n, k/32*34], into contiguous y [n, k] (fp32 or fp16)."""
+    k = y.shape[-1]
+    return lib().minfer_dequant_q8_0(_dtype_code(y), x.data_ptr(), y.data_ptr(), y.numel() // max(k, 1), k, _stream())
+
+
+def flash_attn_decode_q8_0(q, k_cache, v_cache, ctx_lens, out, workspace=None):
+    """q, out fp16 [B,Hq,1,D]; caches uint8 [B,Hkv,Lmax,D/32*34] (dims 0, 1 may be strided)."""
+    import torch
+    B, Hq, _, D = q.shape
+    Hkv, Lmax = k_cache.shape[1], k_cache.shape[2]
+    need = lib().minfer_flash_attn_decode_workspace_bytes(B, Hq, Lmax, D)
+    if workspace is None:
+        workspace = torch.empty(need, dtype=torch.uint8, device=q.device)
+    st = _strides(q, k_cache, out)   # a uint8 tensor's strides are byte strides
+    return lib().minfer_flash_attn_decode_q8_0(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                               ctx_lens.data_ptr(), out.data_ptr(), B, Hq, Hkv, Lmax, D,
+                                               ctypes.byref(st), workspace.data_ptr(), workspace.numel(), _stream())
+
+
+def rope_kv_append_q8_0(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq_base):
+    """As rope_kv_append, into Q8_0 caches, uint8 [B,Hkv,Lmax,D/32*34] with dense rows."""
+    B, L, Hq, D = q.shape
+    return lib().minfer_rope_kv_append_q8_0(_dtype_code(q), style, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                            positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), B, L, Hq,
+                                            k.shape[2], D, k_cache.shape[2], k_cache.stride(0), k_cache.stride(1),
+                                            rotary_dim, freq_base, _stream())

@@ -128,6 +128,48 @@ def test_gemm_validation_rejects_before_launch():
     assert gemm(M=0) == capi.OK and gemm(N=0) == capi.OK and capi.last_error() == ""
 
 
+def test_q8_0_validation_rejects_before_launch():
+    L = capi.lib()
+    quant = lambda dtype=capi.F32, x=0x1000, y=0x2000, n=4, k=128: L.minfer_quant_q8_0(dtype, x, y, n, k, None)
+    assert quant(dtype=8) == capi.EINVAL and "dtype" in capi.last_error()
+    assert quant(k=100) == capi.EINVAL and "multiple of 32" in capi.last_error()
+    assert quant(x=0) == capi.EINVAL and "null" in capi.last_error()
+    assert quant(x=0x1004) == capi.EINVAL and quant(y=0x2001) == capi.EINVAL and quant(n=-1) == capi.EINVAL
+    assert quant(n=0) == capi.OK and quant(k=0) == capi.OK and capi.last_error() == ""
+    dequant = lambda dtype=capi.F16, x=0x1000, y=0x2000, n=4, k=128: L.minfer_dequant_q8_0(dtype, x, y, n, k, None)
+    assert dequant(dtype=capi.BF16) == capi.EINVAL and "dtype" in capi.last_error()   # the reference dequantises to float or half
+    assert dequant(k=31) == capi.EINVAL and dequant(y=0x2002) == capi.EINVAL and dequant(x=0x1001) == capi.EINVAL
+    assert dequant(n=0) == capi.OK
+
+    def dec(B=2, Hq=8, Hkv=2, Lmax=64, D=128, q=0x1000, k=0x2000, v=0x3000, ctx=0x4000, out=0x5000, ws=0x6000, ws_bytes=None, **st):
+        s = dict(q0=Hq * D, q1=D, q2=D, kv0=Hkv * Lmax * (D // 32 * 34), kv1=Lmax * (D // 32 * 34), kv2=D // 32 * 34,
+                 o0=Hq * D, o1=D, o2=D)
+        s.update(st)
+        need = L.minfer_flash_attn_decode_workspace_bytes(B, Hq, Lmax, D)
+        return L.minfer_flash_attn_decode_q8_0(q, k, v, ctx, out, B, Hq, Hkv, Lmax, D, ctypes.byref(capi.Strides(**s)), ws,
+                                               need if ws_bytes is None else ws_bytes, None)
+    assert dec(D=96) == capi.EINVAL and "head_dim" in capi.last_error()
+    assert dec(Hq=7) == capi.EINVAL
+    assert dec(k=0x2001) == capi.EINVAL and "2-byte" in capi.last_error()
+    assert dec(kv2=256) == capi.EINVAL and "dense" in capi.last_error()
+    assert dec(kv1=64 * 136 + 1) == capi.EINVAL and "even" in capi.last_error()
+    assert dec(ctx=0) == capi.EINVAL and dec(q=0x1008) == capi.EINVAL
+    assert dec(ws_bytes=16) == capi.EWORKSPACE
+    assert dec(B=0) == capi.OK and capi.last_error() == ""
+
+    def app(dtype=capi.F16, style=0, q=0x1000, k=0x2000, v=0x3000, pos=0x4000, kc=0x5000, vc=0x6000, B=1, Ln=4, Hq=8, Hkv=2, D=128,
+            Lmax=16, c0=None, c1=None, rd=128, base=1e4):
+        row = D // 32 * 34
+        return L.minfer_rope_kv_append_q8_0(dtype, style, q, k, v, pos, kc, vc, B, Ln, Hq, Hkv, D, Lmax,
+                                            Hkv * Lmax * row if c0 is None else c0, Lmax * row if c1 is None else c1, rd, base, None)
+    assert app(D=80, rd=0) == capi.EINVAL and "multiple of 32" in capi.last_error()
+    assert app(rd=48) == capi.EINVAL                      # a block must not straddle the rotary part's end
+    assert app(rd=96, style=1) == capi.EINVAL             # NeoX halves must be whole blocks
+    assert app(kc=0x5001) == capi.EINVAL and app(c1=137) == capi.EINVAL and app(pos=0) == capi.EINVAL
+    assert app(dtype=capi.F32) == capi.EINVAL
+    assert app(B=0) == capi.OK and app(Ln=0) == capi.OK
+
+
 def test_python_surface_matches_reference_names(kerns):
     from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
     from minfer.kernels import KernelBackend, refs
@@ -150,6 +192,14 @@ def test_python_surface_matches_reference_names(kerns):
         assert str(getattr(torch.ops.minfer, name).default._schema) == \
             f"minfer::{name}(int rotary_dim, int start_pos, float freq_base, Tensor(a!) x) -> ()"
     assert callable(kerns.rope_kv_append)
+    # the quantisers: private names, argument order and schemas of the reference (kernels/__init__.py:5-7,
+    # torch_ext/ops.py:8-46, reg.cpp:22-23); Q8_0 numbered and sized as there (const.py:11, :46)
+    assert GGMLQuantizationType.Q8_0 == 8 and GGML_QUANT_SIZES[GGMLQuantizationType.Q8_0] == (32, 34)
+    for name in ("dequant", "quant"):
+        assert callable(getattr(kerns, "_" + name)) and getattr(te, "_" + name) is getattr(kerns, "_" + name)
+        assert list(inspect.signature(getattr(kerns, "_" + name)).parameters) == ["qtype", "qblock_size", "qtype_size", "x", "y"]
+        assert str(getattr(torch.ops.minfer, name).default._schema) == \
+            f"minfer::{name}(int qtype, int qblock_size, int qtype_size, Tensor x, Tensor(a!) y) -> ()"
     assert list(inspect.signature(te.gemm).parameters) == ["qtype_int", "qblock_size", "qtype_size", "alpha", "beta", "A", "B", "C", "D"]
     assert str(torch.ops.minfer.gemm.default._schema) == ("minfer::gemm(int qtype_int, int qblock_size, int qtype_size, float alpha, "
                                                           "float beta, Tensor A, Tensor B, Tensor C, Tensor(a!) out) -> ()")
@@ -193,6 +243,13 @@ def test_no_cpu_fallback(kerns):
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.qkv(1, 1, 1, 1, 1, 1, 2, 2, 2, h, *[torch.zeros(64, 64, dtype=torch.float16)] * 3, *[torch.empty_like(h) for _ in range(3)])
     with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns._quant(8, 32, 34, torch.zeros(2, 64), torch.zeros(2, 68, dtype=torch.uint8))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns._dequant(8, 32, 34, torch.zeros(2, 68, dtype=torch.uint8), torch.zeros(2, 64))
+    with pytest.raises((NotImplementedError, RuntimeError)):
+        kerns.flash_attn_decode(8, 32, 34, q[:, :, :1], torch.zeros(1, 2, 64, 136, dtype=torch.uint8), torch.zeros(1, 2, 64, 136, dtype=torch.uint8),
+                                torch.ones(1, dtype=torch.int32), torch.empty_like(q[:, :, :1]))
+    with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.il_rope(64, 0, 1e4, x)
     with pytest.raises((NotImplementedError, RuntimeError)):
         kerns.neox_rope(64, 0, 1e4, x)
@@ -225,3 +282,5 @@ def test_workload_generators_are_seeded():
     q, k, v, pos, kc, vc = workloads.kv_append(seed=0, L=16)
     assert q.shape == (1, 16, 32, 128) and k.shape == v.shape == (1, 16, 8, 128) and kc.shape == (1, 8, 16, 128)
     assert workloads.kv_append_bytes(1, 16, 32, 8, 128, 128) == (2 * 16 * 32 * 128 + 4 * 16 * 8 * 128) * 2
+    assert workloads.kv_append_bytes_q8_0(1, 16, 32, 8, 128, 128) == 16 * (2 * 32 * 128 * 2 + 2 * 8 * 128 * 2 + 2 * 8 * 136)
+    assert workloads.decode_bytes_q8_0([10, 20], 32, 8, 128) == 30 * 8 * 136 * 2 + 2 * 2 * 32 * 128 * 2
