@@ -4,9 +4,9 @@ A step is one call of the prefill operator on the Llama-3-8B-shaped workload (B=
 S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmic TFLOP/s
 (4*D*Hq*attended pairs), inputs resident in HBM, every kernel the op launches inside the timed
 region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
-under "decode" with its own HBM roofline, the rotary-embedding step that feeds attention under "rope"
-"rope_kv_append", "rmsnorm" and "gemm", and the reference's CPU attention path (torch SDPA in fp32 on the host cores) under
-"cpu_baseline".  Prints ONE JSON line.
+under "decode" with its own HBM roofline (and again over Q8_0 caches under "decode_q8_0"), the steps that feed
+attention under "rope", "rope_kv_append" (into Q8_0 caches: "rope_kv_append_q8_0"), "rmsnorm" and "gemm", and the
+reference's CPU attention path (torch SDPA in fp32 on the host cores) under "cpu_baseline".  Prints ONE JSON line.
 """
 import argparse
 import ctypes
@@ -31,8 +31,8 @@ ROPE_TRAFFIC_BYTES = 393306 * 1024          # il_rope on [8,4096,48,128], rotary
 APPEND_TRAFFIC_BYTES = 786577 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
 NORM_TRAFFIC_BYTES = 786708 * 1024          # rmsnorm on [8,4096,6144]
 GEMM_TRAFFIC_BYTES = 328543 * 1024          # gemm 4096^3 (B is re-read by each of the 8 XCDs)
-DECODE_Q8_TRAFFIC_BYTES = None              # decode over Q8_0 caches
-APPEND_Q8_TRAFFIC_BYTES = None              # rope_kv_append into Q8_0 caches
+DECODE_Q8_TRAFFIC_BYTES = 584044 * 1024     # decode over Q8_0 caches (split + combine)
+APPEND_Q8_TRAFFIC_BYTES = 737482 * 1024     # rope_kv_append into Q8_0 caches
 
 
 class HipEvents:

@@ -299,12 +299,16 @@ template <int D> struct DecodeGeomQ8 {
     static constexpr int PARK = kGroupRowsQ8 * RB;
     static constexpr int PS = D + 4;                          // floats per head in a wave's partial result
     static constexpr int PART = 16 * PS * 4;
-    static constexpr int WAVE_LDS = (2 * RAW_LDS + PARK > PART ? 2 * RAW_LDS + PARK : PART);
+    // K's pieces are consumed into registers before V's arrive, so one raw area serves both
+    static constexpr int WAVE_LDS = (RAW_LDS + PARK > PART ? RAW_LDS + PARK : PART);
 };
 
 // kv0/kv1 of DecodeParams are byte strides here; q and out are fp16.
+#ifndef MINFER_DECODE_Q8_MIN_WAVES_PER_SIMD
+#define MINFER_DECODE_Q8_MIN_WAVES_PER_SIMD 2
+#endif
 template <int D>
-__global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD) void decode_split_q8_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_SIMD) void decode_split_q8_kernel(const DecodeParams p) {
     using T = F16;
     using GEO = DecodeGeom<D>;
     using Q = DecodeGeomQ8<D>;
@@ -336,8 +340,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     const int heads_here = min(16, p.n_rep - hg * 16);
     const int head0 = g * p.n_rep + hg * 16;
     char* raw_k = lds[w];
-    char* raw_v = lds[w] + Q::RAW_LDS;
-    char* park_v = lds[w] + 2 * Q::RAW_LDS;
+    char* raw_v = lds[w];                    // after K's blocks have been read (a wave's LDS operations execute in order)
+    char* park_v = lds[w] + Q::RAW_LDS;
 
     // The (sequence, KV head)'s rows start at kb; pieces are counted from the 16-byte boundary at or below it.
     // (plain pointer arithmetic, so that the loads below stay global-memory loads)
@@ -425,11 +429,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
             const int off = piece_offset(t, j, last_k, goff);
             *reinterpret_cast<u32x4*>(raw_k + off) = st.k[j];
         }
-#pragma unroll
-        for (int j = 0; j < NL; ++j) {
-            const int off = piece_offset(t, j, last_v, goff);
-            *reinterpret_cast<u32x4*>(raw_v + off) = st.v[j];
-        }
         // ---- S^T = K Q^T for the two 16-key halves: lane gets head l16, keys 16h + 4*quad + r ---------------
         f32x4 s[2];
 #pragma unroll
@@ -452,7 +451,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[h][r] = (key0 + r < row_hi) ? s[h][r] : -INFINITY;
         }
-        // ---- V: every lane dequantises GR * BPR / 64 blocks and parks them as fp16 rows (swizzled) ----------
+        // ---- V: its pieces over K's, then every lane dequantises GR * BPR / 64 blocks and parks them as fp16 rows (swizzled)
+#pragma unroll
+        for (int j = 0; j < NL; ++j) {
+            const int off = piece_offset(t, j, last_v, goff);
+            *reinterpret_cast<u32x4*>(raw_v + off) = st.v[j];
+        }
 #pragma unroll
         for (int i = 0; i < GR * BPR / 64; ++i) {
             const int idx = 64 * i + lane, row = idx / BPR, c = idx % BPR;
