@@ -1,30 +1,32 @@
 // Single-token decode attention for gfx950: split-KV partial kernel + log-sum-exp combine.
 //
-// The op is HBM-bound (each K/V byte is used once per query head of its GQA group), so the
-// design goal is bytes in flight, not FLOPs.  A workgroup (4 waves) owns one (sequence, KV
-// head, chunk of `chunk` cache rows); only chunks that exist are enumerated (a wave-level prefix
-// sum over ctx_lens maps the linear chunk id to its sequence), so no workgroup is launched just
-// to find out that it has nothing to do while others wait for its slot.  Every wave runs a
-// private NS-deep register ring over 16-row groups of the chunk: K rows are loaded straight into
-// the MFMA A-operand layout, V rows as full 256-byte rows; the wave waits only on its own loads
-// -- no workgroup barrier in the loop -- and with 8 waves per CU and NS-1 groups of 8 KB in
+// The op is HBM-bound (each K/V byte is used once per query head of its GQA group), so the design goal is
+// bytes in flight, not FLOPs.  All the cache rows that have to be read -- every sequence, every KV head, rows
+// 0..ctx-1 -- are laid out on one line in 16-row groups, and the line is cut into as many equal shares as the
+// chip holds waves of this kernel (two workgroups of four waves per compute unit): a wave streams its share
+// from start to end on its own, with no barrier and no exchange with its neighbours, and all waves finish
+// together whatever the mix of context lengths.  Where a share crosses from one (sequence, KV head) to the next
+// the wave writes the partial result of the piece it has finished (a segment) and goes on.
+//
+// Every wave runs a private NS-deep register ring over its 16-row groups: K and V rows are loaded as full
+// 256-byte rows; the wave waits only on its own loads, and with 8 waves per CU and NS-1 groups of 8 KB in
 // flight per wave well over 100 KB per CU are outstanding.
 //
 // Compute per group: S^T[16 keys x 16 heads] = K Q^T (16x16x32 MFMA; the GQA group's query heads
 // are the 16 columns, unused columns are zero), online softmax per head (a lane holds 4 keys of
 // one head), then O^T[D x heads] += V^T P^T with 16x16x16 MFMAs whose B operand is the score
 // registers as they are and whose A operand comes from LDS transpose reads of the V rows the
-// wave has just parked in its private 4 KB of LDS.
+// wave has just parked in its private 4 KB of LDS (K goes through the wave's other 4 KB the same way).
 //
-// Every (sequence, head, chunk) writes an un-normalised fp32 partial (O, max, sum) to the
-// workspace; the combine kernel merges the chunks of a row with the usual log-sum-exp weights.
+// Every segment writes an un-normalised fp32 partial (O, max, sum) to the workspace; the combine kernel
+// merges the partials of a (sequence, head) with the usual log-sum-exp weights.
 //
 // Q8_0 caches (decode_split_q8_kernel): a cache row is D/32 blocks of 34 bytes, an fp16 scale d followed by
 // 32 int8 (reference: src/minfer/kernels/torch_ext/csrc/common/types.hpp:141-146), so blocks start on 2-byte
 // boundaries.  Global memory is read in aligned 16-byte pieces all the same (2-byte-aligned wide loads run at a
 // fraction of the rate): a wave's ring holds 32-row groups as the flat run of aligned pieces that covers them,
-// the pieces are dropped into the wave's LDS area, and every lane picks its own blocks out of it with 2-byte
-// aligned LDS reads.  A block becomes the 32 fp16 values (half)(q * d) the reference's dequantiser produces
+// the pieces are dropped into the wave's LDS area, and every lane picks its own blocks out of it as aligned
+// words.  A block becomes the 32 fp16 values (half)(q * d) the reference's dequantiser produces
 // (reference: cuda/quants/impls.cuh:121-143).  K needs no further LDS pass: lane (key, quad) holds values
 // D/4 * quad .. of its key, which is a valid MFMA contraction order as long as Q^T is loaded in the same
 // order.  V is parked as fp16 rows and read back transposed, as on the fp16 path.
@@ -51,47 +53,120 @@ constexpr int kDecodeStages = MINFER_DECODE_STAGES; // ring depth
 struct DecodeParams {
     const void* q; const void* k; const void* v;
     const int32_t* ctx;
-    float* part_o;   // [B][Hq][S][D]
-    float* part_ml;  // [B][Hq][S][2]: reference max (raw score units), sum
+    float* part_o;     // [B][Hq][S][D]
+    float* part_ml;    // [B][Hq][S][2]: reference max (raw score units), sum
+    int32_t* seq_off;  // [B + 1]: linear start of every sequence's work, written by workgroup 0 for the combine kernel
     int64_t q0, q1, kv0, kv1, kv2;
     int B, Hq, Hkv, n_rep, Lmax;
-    int chunk;       // cache rows per workgroup (multiple of 64)
-    int S;           // chunks per sequence = ceil(Lmax / chunk), at most 64
-    int n_hg;        // head groups of <= 16 heads per KV head
+    int n_wg;          // workgroups of the split launch (kDecodeWaves waves each)
+    int min_quota;     // smallest share of the work a wave takes, in groups
+    int group_rows;    // cache rows per group: the unit the work is counted in
+    int S;             // partial results a (sequence, head) can have: slots per row of the workspace, at most 64
+    int n_hg;          // head groups of <= 16 heads per KV head
     float scale_log2;
 };
 
-MA_DEV int chunks_of(int ctx, int Lmax, int chunk) { return (min(max(ctx, 0), Lmax) + chunk - 1) / chunk; }
+// The work, laid out on a line: for every sequence, for every (head group, KV head) pair, the pair's cache rows in
+// groups of `group_rows`.  Wave i of the launch takes groups [i * quota, (i + 1) * quota) of that line, whatever
+// sequences and pairs they belong to, so every wave streams the same number of cache rows, on its own, and all of them
+// end together; a piece of one pair inside one wave's share is a segment, and yields one partial result.
+MA_DEV int groups_of(const DecodeParams& p, int ctx) { return (min(max(ctx, 0), p.Lmax) + p.group_rows - 1) / p.group_rows; }
 
-// Maps a linear chunk id to (sequence, chunk inside the sequence) by a wave-wide inclusive scan of
-// the per-sequence chunk counts; returns false when the id is past the last chunk.
-MA_DEV bool locate_chunk(const DecodeParams& p, int id, int lane, int& b_out, int& split_out, int& ctx_out) {
+MA_DEV int wave_inclusive_scan(int x, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(x, d);
+        if (lane >= d) x += up;
+    }
+    return x;
+}
+
+// Length of the line (every lane gets it).  With `publish`, also stores every sequence's start on the line and,
+// at index B, the length.
+MA_DEV int work_total(const DecodeParams& p, int lane, bool publish) {
+    const int pairs = p.Hkv * p.n_hg;
     int offset = 0;
     for (int base = 0; base < p.B; base += 64) {
         const int b = base + lane;
+        const int n = b < p.B ? groups_of(p, p.ctx[b]) * pairs : 0;
+        const int incl = wave_inclusive_scan(n, lane);
+        if (publish && b < p.B) p.seq_off[b] = offset + incl - n;
+        offset += __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+    }
+    if (publish && lane == 0) p.seq_off[p.B] = offset;
+    return offset;
+}
+MA_DEV int work_quota(const DecodeParams& p, int total) {
+    const int n_waves = p.n_wg * kDecodeWaves;
+    return max((total + n_waves - 1) / n_waves, p.min_quota);
+}
+
+// The sequence that holds position x (< total) of the line, its start on the line and its context length.
+MA_DEV void locate_sequence(const DecodeParams& p, int x, int lane, int& b_out, int& off_out, int& ctx_out) {
+    const int pairs = p.Hkv * p.n_hg;
+    int offset = 0;
+    b_out = 0; off_out = 0; ctx_out = 0;
+    for (int base = 0; base < p.B; base += 64) {
+        const int b = base + lane;
         const int c = b < p.B ? p.ctx[b] : 0;
-        const int n = chunks_of(c, p.Lmax, p.chunk);
-        int incl = n;
-#pragma unroll
-        for (int d = 1; d < 64; d <<= 1) {
-            const int up = __shfl_up(incl, d);
-            if (lane >= d) incl += up;
-        }
-        const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63));   // wave-uniform, and known to be
-        if (id < offset + total) {
-            const uint64_t hit = __ballot(id < offset + incl);
+        const int n = b < p.B ? groups_of(p, c) * pairs : 0;
+        const int incl = wave_inclusive_scan(n, lane);
+        const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+        if (x < offset + total) {
+            const uint64_t hit = __ballot(x < offset + incl);
             const int src = __ffsll((unsigned long long)hit) - 1;
             // every lane holds the same values; saying so keeps the kernel's control flow (and with it
             // the compiler's wait-count bookkeeping in the main loop) scalar
             b_out = __builtin_amdgcn_readfirstlane(base + src);
-            split_out = __builtin_amdgcn_readfirstlane(id - offset - __shfl(incl - n, src));
+            off_out = __builtin_amdgcn_readfirstlane(offset + __shfl(incl - n, src));
             ctx_out = __builtin_amdgcn_readfirstlane(__shfl(c, src));
-            return true;
+            return;
         }
         offset += total;
     }
-    return false;
 }
+
+// Walks a wave's share of the line segment by segment.
+struct SegmentWalk {
+    int x, x_end, quota;     // position on the line, end of the share
+    int b, off_b, ctx, n_b;  // current sequence: index, start on the line, context length, groups per pair
+    // set by next():
+    int pair, g0, g1, slot;  // (head group, KV head) pair, its groups [g0, g1), index of the partial result among the pair's
+
+    int wave;                // index of the wave in the launch
+    MA_DEV bool start(const DecodeParams& p, int lane, int w) {
+        wave = (int)blockIdx.x * kDecodeWaves + w;
+        const int total = work_total(p, lane, wave == 0);
+        quota = work_quota(p, total);
+        x = wave * quota;
+        x_end = min(total, x + quota);
+        if (x >= x_end) return false;
+        int c;
+        locate_sequence(p, x, lane, b, off_b, c);
+        ctx = min(max(c, 0), p.Lmax);
+        n_b = groups_of(p, ctx);
+        return true;
+    }
+    MA_DEV bool next(const DecodeParams& p) {
+        if (x >= x_end) return false;
+        const int pairs = p.Hkv * p.n_hg;
+        if (x >= off_b + pairs * n_b) {        // the sequence is done: on to the next one that has rows
+            off_b += pairs * n_b;
+            do {
+                ++b;
+                ctx = min(max(p.ctx[b], 0), p.Lmax);
+                n_b = groups_of(p, ctx);
+            } while (n_b == 0);
+        }
+        const int y = x - off_b;
+        pair = y / n_b;
+        g0 = y - pair * n_b;
+        g1 = min(n_b, g0 + (x_end - x));
+        slot = wave - (off_b + pair * n_b) / quota;
+        x += g1 - g0;
+        return true;
+    }
+};
 
 template <int D> struct DecodeGeom {
     static constexpr int RB = D * 2;
@@ -111,27 +186,23 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     constexpr int KC = D / 32;   // 32-wide contraction chunks of K Q^T
     constexpr int DB = D / 16;   // 16-row blocks of O^T
     constexpr int NS = kDecodeStages;
-    constexpr int PS = D + 4;    // floats per head in a wave's partial result (O, max, sum, pad)
 
     __shared__ __attribute__((aligned(1024))) char v_lds[kDecodeWaves][kGroupRows * RB];
     __shared__ __attribute__((aligned(1024))) char k_lds[kDecodeWaves][kGroupRows * RB];
-    __shared__ __attribute__((aligned(16))) float part_lds[kDecodeWaves][16 * PS];
 
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    const int per_chunk = p.Hkv * p.n_hg;
-    const int y = blockIdx.x % per_chunk;
-    const int g = y % p.Hkv, hg = y / p.Hkv;
-    int b, split, ctx_raw;
-    if (!locate_chunk(p, blockIdx.x / per_chunk, lane, b, split, ctx_raw)) return;   // past the last chunk
-
-    const int ctx = min(max(ctx_raw, 0), p.Lmax);
-    const int row_lo = split * p.chunk;
-    const int row_hi = min(row_lo + p.chunk, ctx);
-    const int n_groups = (row_hi - row_lo + kGroupRows - 1) / kGroupRows;
-    const int my_groups = (n_groups - w + kDecodeWaves - 1) / kDecodeWaves;  // groups w, w+4, ...
-    auto group_of = [&](int t) { return w + t * kDecodeWaves; };
-    auto wave_has_work = [&](int ww) { return ww < n_groups; };
+    SegmentWalk walk;
+    if (!walk.start(p, lane, w)) return;   // no share of the work
+    while (walk.next(p)) {
+    const int b = walk.b, split = walk.slot;
+    const int g = walk.pair % p.Hkv, hg = walk.pair / p.Hkv;
+    const int ctx = walk.ctx;
+    const int row_lo = walk.g0 * kGroupRows;
+    const int row_hi = min(walk.g1 * kGroupRows, ctx);
+    const int n_groups = walk.g1 - walk.g0;
+    const int my_groups = n_groups;
+    auto group_of = [&](int t) { return t; };
 
     const int heads_here = min(16, p.n_rep - hg * 16);
     const int head0 = g * p.n_rep + hg * 16;
@@ -244,40 +315,21 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     for (int t0 = 0; t0 < my_groups; t0 += NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            consume(t0 + s, kr[s], vr[s]);
+            if (t0 + s < my_groups) consume(t0 + s, kr[s], vr[s]);
             load_group(t0 + s + NS, kr[s], vr[s]);
         }
     }
 
-    // ---- merge the four waves' partial results through LDS, write the chunk's partial ----------
+    // ---- the segment's partial result: un-normalised O, reference max and sum of every head -------------
     l_sum += __shfl_xor(l_sum, 16);
     l_sum += __shfl_xor(l_sum, 32);
-    float* mine = part_lds[w];   // [16 heads][PS]
     if (l16 < heads_here) {
+        const int64_t slot = ((int64_t)b * p.Hq + head0 + l16) * p.S + split;
+        float* dst = p.part_o + slot * D + 4 * quad;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(mine + l16 * PS + 16 * db + 4 * quad) = o_acc[db];
-        if (quad == 0) { mine[l16 * PS + D] = m_ref; mine[l16 * PS + D + 1] = l_sum; }
+        for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = o_acc[db];
+        if (quad == 0) { p.part_ml[slot * 2] = m_ref; p.part_ml[slot * 2 + 1] = l_sum; }
     }
-    __syncthreads();
-    for (int idx = tid; idx < heads_here * D; idx += kDecodeWaves * 64) {
-        const int hh = idx / D, d = idx % D;
-        float M = -INFINITY;
-#pragma unroll
-        for (int ww = 0; ww < kDecodeWaves; ++ww)
-            if (wave_has_work(ww)) M = fmaxf(M, part_lds[ww][hh * PS + D]);
-        float o = 0.f, l = 0.f;
-#pragma unroll
-        for (int ww = 0; ww < kDecodeWaves; ++ww) {
-            const float* src = part_lds[ww] + hh * PS;
-            if (wave_has_work(ww) && src[D] > -INFINITY) {
-                const float wgt = fast_exp2((src[D] - M) * c2);
-                o += src[d] * wgt;
-                l += src[D + 1] * wgt;
-            }
-        }
-        const int64_t slot = ((int64_t)b * p.Hq + head0 + hh) * p.S + split;
-        p.part_o[slot * D + d] = o;
-        if (d == 0) { p.part_ml[slot * 2] = M; p.part_ml[slot * 2 + 1] = l; }
     }
 }
 
@@ -297,10 +349,8 @@ template <int D> struct DecodeGeomQ8 {
     static constexpr int RAW_LDS = NG * 16;
     static constexpr int RB = D * 2;                          // bytes of a parked fp16 row
     static constexpr int PARK = kGroupRowsQ8 * RB;
-    static constexpr int PS = D + 4;                          // floats per head in a wave's partial result
-    static constexpr int PART = 16 * PS * 4;
     // K's pieces are consumed into registers before V's arrive, so one raw area serves both
-    static constexpr int WAVE_LDS = (RAW_LDS + PARK > PART ? RAW_LDS + PARK : PART);
+    static constexpr int WAVE_LDS = RAW_LDS + PARK;
 };
 
 // kv0/kv1 of DecodeParams are byte strides here; q and out are fp16.
@@ -316,26 +366,23 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
     constexpr int KC = D / 32;   // 32-wide contraction steps of K Q^T
     constexpr int DB = D / 16;   // 16-row blocks of O^T
     constexpr int NS = kDecodeStagesQ8;
-    constexpr int PS = Q::PS;
     constexpr int GR = kGroupRowsQ8;
 
     __shared__ __attribute__((aligned(1024))) char lds[kDecodeWaves][(Q::WAVE_LDS + 1023) / 1024 * 1024];
 
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    const int per_chunk = p.Hkv * p.n_hg;
-    const int y = blockIdx.x % per_chunk;
-    const int g = y % p.Hkv, hg = y / p.Hkv;
-    int b, split, ctx_raw;
-    if (!locate_chunk(p, blockIdx.x / per_chunk, lane, b, split, ctx_raw)) return;   // past the last chunk
-
-    const int ctx = min(max(ctx_raw, 0), p.Lmax);
-    const int row_lo = split * p.chunk;                      // a multiple of 64
-    const int row_hi = min(row_lo + p.chunk, ctx);
-    const int n_groups = (row_hi - row_lo + GR - 1) / GR;
-    const int my_groups = (n_groups - w + kDecodeWaves - 1) / kDecodeWaves;  // groups w, w+4, ...
-    auto group_of = [&](int t) { return w + t * kDecodeWaves; };
-    auto wave_has_work = [&](int ww) { return ww < n_groups; };
+    SegmentWalk walk;
+    if (!walk.start(p, lane, w)) return;   // no share of the work
+    while (walk.next(p)) {
+    const int b = walk.b, split = walk.slot;
+    const int g = walk.pair % p.Hkv, hg = walk.pair / p.Hkv;
+    const int ctx = walk.ctx;
+    const int row_lo = walk.g0 * GR;                         // a multiple of 32
+    const int row_hi = min(walk.g1 * GR, ctx);
+    const int n_groups = walk.g1 - walk.g0;
+    const int my_groups = n_groups;
+    auto group_of = [&](int t) { return t; };
 
     const int heads_here = min(16, p.n_rep - hg * 16);
     const int head0 = g * p.n_rep + hg * 16;
@@ -519,40 +566,21 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
     for (int t0 = 0; t0 < my_groups; t0 += NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            consume(t0 + s, ring[s]);
+            if (t0 + s < my_groups) consume(t0 + s, ring[s]);
             load_group(t0 + s + NS, ring[s]);
         }
     }
 
-    // ---- merge the four waves' partial results through LDS (over the wave's own areas), write the chunk's partial
+    // ---- the segment's partial result: un-normalised O, reference max and sum of every head -------------
     l_sum += __shfl_xor(l_sum, 16);
     l_sum += __shfl_xor(l_sum, 32);
-    float* mine = reinterpret_cast<float*>(lds[w]);   // [16 heads][PS]
     if (l16 < heads_here) {
+        const int64_t slot = ((int64_t)b * p.Hq + head0 + l16) * p.S + split;
+        float* dst = p.part_o + slot * D + 4 * quad;
 #pragma unroll
-        for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(mine + l16 * PS + 16 * db + 4 * quad) = o_acc[db];
-        if (quad == 0) { mine[l16 * PS + D] = m_ref; mine[l16 * PS + D + 1] = l_sum; }
+        for (int db = 0; db < DB; ++db) *reinterpret_cast<f32x4*>(dst + 16 * db) = o_acc[db];
+        if (quad == 0) { p.part_ml[slot * 2] = m_ref; p.part_ml[slot * 2 + 1] = l_sum; }
     }
-    __syncthreads();
-    for (int idx = tid; idx < heads_here * D; idx += kDecodeWaves * 64) {
-        const int hh = idx / D, d = idx % D;
-        float M = -INFINITY;
-#pragma unroll
-        for (int ww = 0; ww < kDecodeWaves; ++ww)
-            if (wave_has_work(ww)) M = fmaxf(M, reinterpret_cast<const float*>(lds[ww])[hh * PS + D]);
-        float o = 0.f, l = 0.f;
-#pragma unroll
-        for (int ww = 0; ww < kDecodeWaves; ++ww) {
-            const float* src = reinterpret_cast<const float*>(lds[ww]) + hh * PS;
-            if (wave_has_work(ww) && src[D] > -INFINITY) {
-                const float wgt = fast_exp2((src[D] - M) * c2);
-                o += src[d] * wgt;
-                l += src[D + 1] * wgt;
-            }
-        }
-        const int64_t slot = ((int64_t)b * p.Hq + head0 + hh) * p.S + split;
-        p.part_o[slot * D + d] = o;
-        if (d == 0) { p.part_ml[slot * 2] = M; p.part_ml[slot * 2 + 1] = l; }
     }
 }
 
@@ -566,7 +594,12 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     const int row = blockIdx.x * 4 + wave_id();
     if (row >= p.B * p.Hq) return;
     const int b = row / p.Hq, hq = row % p.Hq;
-    const int ns = chunks_of(p.ctx[b], p.Lmax, p.chunk);
+    // the partial results of this row: one per workgroup whose share of the line overlaps the row's pair
+    const int n_b = groups_of(p, p.ctx[b]);
+    const int quota = work_quota(p, p.seq_off[p.B]);
+    const int g = hq / p.n_rep, hg = (hq % p.n_rep) / 16;
+    const int start = p.seq_off[b] + (hg * p.Hkv + g) * n_b;
+    const int ns = n_b > 0 ? (start + n_b - 1) / quota - start / quota + 1 : 0;
     const int64_t slot0 = (int64_t)row * p.S;
     float m = -INFINITY, l = 0.f;
     if (lane < ns) { m = p.part_ml[(slot0 + lane) * 2]; l = p.part_ml[(slot0 + lane) * 2 + 1]; }
@@ -609,37 +642,41 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     }
 }
 
-// Cache rows per workgroup.  Smallest: 256 (or more for very long caches, so that a row never has more
-// than 64 chunks, which is what one wave of the combine kernel merges).  Larger chunks mean fewer
-// partials and fewer workgroup start-ups, so the launcher doubles the chunk while the grid would still
-// hold well over a thousand workgroups.  The workspace is sized for the smallest chunk.
-static int decode_min_chunk_rows(int64_t Lmax) {
-    int64_t c = (Lmax + 63) / 64;
+// Smallest share of the work a workgroup takes, in cache rows: 256, or more for very long caches, so that a
+// (sequence, head) never has more than 64 partial results, which is what one wave of the combine kernel merges.
+static int decode_min_share_rows(int64_t Lmax) {
+    int64_t c = (Lmax + 59) / 60;
     c = (c + 63) / 64 * 64;
     return (int)(c > 256 ? c : 256);
 }
-static int decode_chunk_rows(int64_t B, int64_t Hkv, int64_t n_hg, int64_t Lmax) {
-#ifdef MINFER_DECODE_CHUNK
-    const int forced = MINFER_DECODE_CHUNK;
-    return forced > decode_min_chunk_rows(Lmax) ? forced : decode_min_chunk_rows(Lmax);
-#else
-    int chunk = decode_min_chunk_rows(Lmax);
-    while (chunk < 1024 && B * Hkv * n_hg * ((Lmax + 2 * chunk - 1) / (2 * chunk)) >= 2048) chunk *= 2;
-    return chunk;
-#endif
-}
+// Partial results a (sequence, head) can have: a pair's rows overlap at most this many shares.
+static int decode_slots(int64_t Lmax) { return (int)(Lmax / decode_min_share_rows(Lmax)) + 3; }
 
 static size_t decode_ws_bytes(int64_t B, int64_t Hq, int64_t Lmax, int64_t D) {
-    const int64_t chunk = decode_min_chunk_rows(Lmax);
-    const int64_t S = (Lmax + chunk - 1) / chunk;
-    return (size_t)(B * Hq * S * (D + 2) * 4 + 255) / 256 * 256 + 256;
+    const int64_t S = decode_slots(Lmax);
+    return (size_t)(B * Hq * S * (D + 2) * 4 + 255) / 256 * 256 + (size_t)((B + 1) * 4 + 255) / 256 * 256 + 256;
+}
+
+// Workgroups of the split launch: as many as the chip holds at once (two per compute unit: LDS and registers
+// allow no more), so that each gets one equal share of the work and all run from start to end.
+#ifndef MINFER_DECODE_WG_PER_CU
+#define MINFER_DECODE_WG_PER_CU 2
+#endif
+static int decode_workgroups() {
+    static int cached[64] = {0};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    if (cached[dev] == 0) {
+        int cus = 0;
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cached[dev] = cus * MINFER_DECODE_WG_PER_CU;
+    }
+    return cached[dev];
 }
 
 template <class T, int D>
 static int launch_decode(const DecodeParams& p, void* out, int64_t o0, int64_t o1, hipStream_t stream) {
-    // chunk id is the slow index, so every chunk that exists is dispatched before the ids past the end
-    const int64_t grid = (int64_t)p.B * p.S * p.Hkv * p.n_hg;
-    hipLaunchKernelGGL((decode_split_kernel<T, D>), dim3((unsigned)grid), dim3(kDecodeWaves * 64), 0, stream, p);
+    hipLaunchKernelGGL((decode_split_kernel<T, D>), dim3((unsigned)p.n_wg), dim3(kDecodeWaves * 64), 0, stream, p);
     if (int rc = check_launch("decode_split_kernel")) return rc;
     hipLaunchKernelGGL((decode_combine_kernel<T, D>), dim3((p.B * p.Hq + 3) / 4), dim3(256), 0, stream, p, out, o0, o1);
     return check_launch("decode_combine_kernel");
@@ -647,8 +684,7 @@ static int launch_decode(const DecodeParams& p, void* out, int64_t o0, int64_t o
 
 template <int D>
 static int launch_decode_q8(const DecodeParams& p, void* out, int64_t o0, int64_t o1, hipStream_t stream) {
-    const int64_t grid = (int64_t)p.B * p.S * p.Hkv * p.n_hg;
-    hipLaunchKernelGGL((decode_split_q8_kernel<D>), dim3((unsigned)grid), dim3(kDecodeWaves * 64), 0, stream, p);
+    hipLaunchKernelGGL((decode_split_q8_kernel<D>), dim3((unsigned)p.n_wg), dim3(kDecodeWaves * 64), 0, stream, p);
     if (int rc = check_launch("decode_split_q8_kernel")) return rc;
     hipLaunchKernelGGL((decode_combine_kernel<F16, D>), dim3((p.B * p.Hq + 3) / 4), dim3(256), 0, stream, p, out, o0, o1);
     return check_launch("decode_combine_kernel");
@@ -666,7 +702,7 @@ MINFER_ATTN_EXPORT size_t minfer_flash_attn_decode_workspace_bytes(int64_t B, in
 // Fills the launch parameters both decode entry points share; returns an error code or MINFER_ATTN_OK.
 static int fill_decode(DecodeParams& p, const void* q, const void* k_cache, const void* v_cache, const int32_t* ctx_lens,
                        int64_t B, int64_t Hq, int64_t Hkv, int64_t Lmax, int64_t D, const minfer_attn_strides* st,
-                       void* workspace, size_t workspace_bytes) {
+                       void* workspace, size_t workspace_bytes, int group_rows) {
     if (!ctx_lens) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: ctx_lens is null");
     if (B < 0 || Lmax < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: negative B or Lmax");
     if (B > 65535 || Hq > 65535) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: B or n_heads > 65535 unsupported");
@@ -678,15 +714,19 @@ static int fill_decode(DecodeParams& p, const void* q, const void* k_cache, cons
     p.q0 = st->q0; p.q1 = st->q1; p.kv0 = st->kv0; p.kv1 = st->kv1; p.kv2 = st->kv2;
     p.B = (int)B; p.Hq = (int)Hq; p.Hkv = (int)Hkv; p.n_rep = (int)(Hq / Hkv); p.Lmax = (int)Lmax;
     p.n_hg = (p.n_rep + 15) / 16;
-    p.chunk = decode_chunk_rows(B, Hkv, p.n_hg, Lmax);
-    p.S = (int)((Lmax + p.chunk - 1) / p.chunk);
-    if (p.S < 1) p.S = 1;
-    if ((int64_t)B * p.S * Hkv * ((Hq / Hkv + 15) / 16) > 0x7fffffffLL)
+    p.group_rows = group_rows;
+    p.min_quota = decode_min_share_rows(Lmax) / group_rows;
+    p.S = decode_slots(Lmax);
+    p.n_wg = decode_workgroups();
+    // the line of work is indexed with 32-bit integers
+    if ((int64_t)B * Hkv * p.n_hg * ((Lmax + group_rows - 1) / group_rows) > 0x7fffffffLL - 65536)
         return fail(MINFER_ATTN_EINVAL, "flash_attn_decode: problem too large for one launch");
     p.scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
-    const size_t o_bytes = (size_t)B * Hq * p.S * D * 4;
+    const size_t o_bytes = ((size_t)B * Hq * p.S * D * 4 + 255) / 256 * 256;
+    const size_t ml_bytes = ((size_t)B * Hq * p.S * 2 * 4 + 255) / 256 * 256;
     p.part_o = (float*)workspace;
-    p.part_ml = (float*)((char*)workspace + (o_bytes + 255) / 256 * 256);
+    p.part_ml = (float*)((char*)workspace + o_bytes);
+    p.seq_off = (int32_t*)((char*)workspace + o_bytes + ml_bytes);
     return MINFER_ATTN_OK;
 }
 
@@ -697,7 +737,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode(int dtype, const void* q, const 
     clear_error();
     if (int rc = check_common(dtype, q, k_cache, v_cache, out, Hq, Hkv, D, st)) return rc;
     DecodeParams p{};
-    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes)) return rc;
+    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes, kGroupRows)) return rc;
     if (B == 0) return MINFER_ATTN_OK;
     hipStream_t stream = (hipStream_t)stream_v;
 
@@ -726,7 +766,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode_q8_0(const void* q, const void* 
     if (st->kv0 < 0 || st->kv1 < 0 || st->kv0 % 2 || st->kv1 % 2)
         return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_q8_0: cache strides must be non-negative even byte counts");
     DecodeParams p{};
-    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes)) return rc;
+    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes, kGroupRowsQ8)) return rc;
     if (B == 0) return MINFER_ATTN_OK;
     hipStream_t stream = (hipStream_t)stream_v;
     return D == 128 ? launch_decode_q8<128>(p, out, st->o0, st->o1, stream) : launch_decode_q8<64>(p, out, st->o0, st->o1, stream);

@@ -275,6 +275,40 @@ def test_decode_matches_oracle(dtype, B, Hq, Hkv, Lmax, D, lo, hi):
     assert torch.all(out[ctx.to(DEV) == 0] == 0)
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,Lmax,D,ctx", [
+    (200, 8, 2, 64, 64, "tiny"),          # shares of the work span many short sequences, some empty; B > 64
+    (1, 4, 1, 40000, 128, "full"),        # one (sequence, KV head) cut into ~57 shares: as many partials per row
+    (70, 40, 2, 1000, 128, "gaps"),       # empty sequences at both ends and in between, two head groups
+    (3, 16, 16, 5000, 64, "full"),
+])
+def test_decode_work_is_shared_out_evenly_whatever_the_lengths(B, Hq, Hkv, Lmax, D, ctx):
+    g = torch.Generator().manual_seed(B + Lmax)
+    q = torch.randn(B, Hq, 1, D, generator=g).half()
+    kc = torch.randn(B, Hkv, Lmax, D, generator=g).half()
+    vc = torch.randn(B, Hkv, Lmax, D, generator=g).half()
+    if ctx == "tiny":
+        lens = torch.randint(0, 41, (B,), generator=g, dtype=torch.int32)
+    elif ctx == "full":
+        lens = torch.full((B,), Lmax, dtype=torch.int32)
+    else:
+        lens = torch.randint(1, Lmax + 1, (B,), generator=g, dtype=torch.int32)
+        lens[:3] = 0
+        lens[-2:] = 0
+        lens[10:40:7] = 0
+    out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)
+    assert capi.flash_attn_decode(q.to(DEV), kc.to(DEV), vc.to(DEV), lens.to(DEV), out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert max_err(out, oracle.flash_attn_decode(q, kc, vc, lens)) <= TOL[torch.float16]
+    assert torch.all(out[lens.to(DEV) == 0] == 0)
+    # the same caches as Q8_0 blocks
+    kq, vq = torch.from_numpy(oracle.quant_q8_0(kc.float())), torch.from_numpy(oracle.quant_q8_0(vc.float()))
+    out8 = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)
+    assert capi.flash_attn_decode_q8_0(q.to(DEV), kq.to(DEV), vq.to(DEV), lens.to(DEV), out8) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert max_err(out8, oracle.flash_attn_decode_q8_0(q, kq, vq, lens)) <= TOL[torch.float16]
+    assert torch.all(out8[lens.to(DEV) == 0] == 0)
+
+
 def test_decode_equals_last_prefill_row():
     """Splitting the KV range and merging by log-sum-exp must not change the result: the decode of
     position ctx-1 equals the last row of a causal prefill over the same ctx rows."""

@@ -34,8 +34,12 @@ def test_workspace_sizes():
     assert L.minfer_flash_attn_workspace_bytes(1, 4096) >= 64 * 64
     assert L.minfer_flash_attn_workspace_bytes(2, 100) >= 2 * 2 * 2
     assert L.minfer_flash_attn_workspace_bytes(1, 32768) >= 512 * 512
-    # fp32 partial (D values + max + sum) per (sequence, head, 512-row chunk)
-    assert L.minfer_flash_attn_decode_workspace_bytes(64, 32, 8192, 128) >= 64 * 32 * 16 * 130 * 4
+    # fp32 partials (D values + max + sum), one per share of at least 256 rows that can overlap a (sequence, head)'s rows
+    # (8192/256 + 2 of them), plus one line offset per sequence
+    need = L.minfer_flash_attn_decode_workspace_bytes(64, 32, 8192, 128)
+    assert 64 * 32 * 34 * 130 * 4 + 65 * 4 <= need <= 2 * 64 * 32 * 34 * 130 * 4
+    # never more than 64 partials per row, however long the cache
+    assert L.minfer_flash_attn_decode_workspace_bytes(1, 8, 1 << 20, 128) <= 8 * 64 * 130 * 4 + 4096
 
 
 def _call_prefill(dtype=capi.F16, q=0x1000, k=0x2000, v=0x3000, mask=0x4000, out=0x5000, B=1, Hq=8, Hkv=2,
