@@ -136,13 +136,32 @@ struct SegmentWalk {
     int wave;                // index of the wave in the launch
     MA_DEV bool start(const DecodeParams& p, int lane, int w) {
         wave = (int)blockIdx.x * kDecodeWaves + w;
-        const int total = work_total(p, lane, wave == 0);
-        quota = work_quota(p, total);
-        x = wave * quota;
-        x_end = min(total, x + quota);
-        if (x >= x_end) return false;
         int c;
-        locate_sequence(p, x, lane, b, off_b, c);
+        if (p.B <= 64) {   // one scan gives the line's length and the share's first sequence
+            c = lane < p.B ? p.ctx[lane] : 0;
+            const int n = lane < p.B ? groups_of(p, c) * p.Hkv * p.n_hg : 0;
+            const int incl = wave_inclusive_scan(n, lane);
+            const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+            if (wave == 0) {
+                if (lane < p.B) p.seq_off[lane] = incl - n;
+                if (lane == 0) p.seq_off[p.B] = total;
+            }
+            quota = work_quota(p, total);
+            x = wave * quota;
+            x_end = min(total, x + quota);
+            if (x >= x_end) return false;
+            const int src = __ffsll((unsigned long long)__ballot(x < incl)) - 1;
+            b = __builtin_amdgcn_readfirstlane(src);
+            off_b = __builtin_amdgcn_readfirstlane(__shfl(incl - n, src));
+            c = __builtin_amdgcn_readfirstlane(__shfl(c, src));
+        } else {
+            const int total = work_total(p, lane, wave == 0);
+            quota = work_quota(p, total);
+            x = wave * quota;
+            x_end = min(total, x + quota);
+            if (x >= x_end) return false;
+            locate_sequence(p, x, lane, b, off_b, c);
+        }
         ctx = min(max(c, 0), p.Lmax);
         n_b = groups_of(p, ctx);
         return true;
@@ -594,15 +613,31 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     const int row = blockIdx.x * 4 + wave_id();
     if (row >= p.B * p.Hq) return;
     const int b = row / p.Hq, hq = row % p.Hq;
-    // the partial results of this row: one per workgroup whose share of the line overlaps the row's pair
+    const int64_t slot0 = (int64_t)row * p.S;
+    const float* src = p.part_o + slot0 * D + EPL * lane;
+    auto load_o = [&](int slot, float (&x)[EPL]) {
+        const float* ptr = src + (int64_t)slot * D;
+        if (EPL == 2) {
+            const f32x2 v2 = *reinterpret_cast<const f32x2*>(ptr);
+            x[0] = v2[0]; x[EPL - 1] = v2[1];
+        } else {
+            x[0] = ptr[0];
+        }
+    };
+    // Everything is requested at once: how many partial results the row has, and, before that is known, every
+    // slot's (max, sum) and the first eight slots' O (slots past the count hold stale bytes and are discarded).
+    const int sl = min(lane, p.S - 1);
+    const float m_raw = p.part_ml[(slot0 + sl) * 2], l_raw = p.part_ml[(slot0 + sl) * 2 + 1];
+    float x[8][EPL];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) load_o(min(u, p.S - 1), x[u]);
+    // the partial results of this row: one per share of the line that overlaps the rows of its (sequence, KV head)
     const int n_b = groups_of(p, p.ctx[b]);
     const int quota = work_quota(p, p.seq_off[p.B]);
     const int g = hq / p.n_rep, hg = (hq % p.n_rep) / 16;
     const int start = p.seq_off[b] + (hg * p.Hkv + g) * n_b;
     const int ns = n_b > 0 ? (start + n_b - 1) / quota - start / quota + 1 : 0;
-    const int64_t slot0 = (int64_t)row * p.S;
-    float m = -INFINITY, l = 0.f;
-    if (lane < ns) { m = p.part_ml[(slot0 + lane) * 2]; l = p.part_ml[(slot0 + lane) * 2 + 1]; }
+    const float m = lane < ns ? m_raw : -INFINITY, l = lane < ns ? l_raw : 0.f;
     float M = m;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) M = fmaxf(M, __shfl_xor(M, d));
@@ -613,24 +648,17 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
     float acc[EPL];
 #pragma unroll
     for (int e = 0; e < EPL; ++e) acc[e] = 0.f;
-    const float* src = p.part_o + slot0 * D + EPL * lane;
-    for (int s0 = 0; s0 < ns; s0 += 8) {   // 8 chunk partials at a time, all loads in flight together
-        float x[8][EPL];
+    for (int s0 = 0; s0 < ns; s0 += 8) {   // 8 partial results at a time, all loads in flight together
+        if (s0 > 0) {
 #pragma unroll
-        for (int u = 0; u < 8; ++u) {
-            const float* ptr = src + (int64_t)min(s0 + u, ns - 1) * D;
-            if (EPL == 2) {
-                const f32x2 v2 = *reinterpret_cast<const f32x2*>(ptr);
-                x[u][0] = v2[0]; x[u][EPL - 1] = v2[1];
-            } else {
-                x[u][0] = ptr[0];
-            }
+            for (int u = 0; u < 8; ++u) load_o(min(s0 + u, ns - 1), x[u]);
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
-            const float ws = (s0 + u < ns) ? __shfl(wgt, s0 + u) : 0.f;
+            const bool on = s0 + u < ns;
+            const float ws = __shfl(wgt, min(s0 + u, 63));
 #pragma unroll
-            for (int e = 0; e < EPL; ++e) acc[e] += x[u][e] * ws;
+            for (int e = 0; e < EPL; ++e) acc[e] += on ? x[u][e] * ws : 0.f;
         }
     }
     const float inv = L > 0.f ? 1.f / L : 0.f;
