@@ -24,6 +24,10 @@
 
 namespace minfer_attn {
 
+#ifndef MINFER_GEMM_GROUP_M
+#define MINFER_GEMM_GROUP_M 4
+#endif
+
 constexpr int kBK = 64;
 // Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
 // 128 x 128 otherwise.  A wave owns 32*MB rows x 64 columns.
@@ -62,7 +66,12 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
     // ---- which tile ----------------------------------------------------------------------------------
     const int t = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
     if (t >= p.tiles_m * p.tiles_n) return;
-    const int m0 = (t / p.tiles_n) * kBM, n0 = (t % p.tiles_n) * kBN;
+    // Tiles are numbered down bands of kGroupM tile rows, so that the tiles an XCD runs at one time form a block that
+    // shares A row panels as well as B column panels in its L2 (row-major numbering made every XCD read all of B).
+    constexpr int kGroupM = MINFER_GEMM_GROUP_M;
+    const int band = t / (kGroupM * p.tiles_n), in_band = t % (kGroupM * p.tiles_n);
+    const int first_m = band * kGroupM, gm = min(kGroupM, p.tiles_m - first_m);
+    const int m0 = (first_m + in_band % gm) * kBM, n0 = (in_band / gm) * kBN;
     const bool full_m = m0 + kBM <= p.M, full_n = n0 + kBN <= p.N;
 
     const short* Ag = (const short*)p.A;
