@@ -7,7 +7,7 @@
 // per vector and reads the vector twice from memory.
 //
 // HBM-bound: every element is read once and written once, in 16-byte lane accesses, and stays in registers
-// between the sum of squares and the scaling.  Vectors up to 8192 elements (per-head norm, and per-token norm
+// between the sum of squares and the scaling, as does the lane's share of the weight.  Vectors up to 8192 elements (per-head norm, and per-token norm
 // of the usual hidden sizes) are handled by a group of 8..64 lanes of one wave, several short vectors per
 // wave, reduced with lane exchanges only and with no barrier; longer vectors by one 256-thread workgroup
 // with one LDS exchange.
@@ -51,15 +51,13 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const NormPa
     const int64_t wave = (int64_t)blockIdx.x * (kNormThreads / 64) + (threadIdx.x >> 6);
     const int64_t n_waves = (int64_t)gridDim.x * (kNormThreads / 64);
     const int chunks = p.dim >> 3;
-    // the lane's share of the weight: kept in registers when it is small, re-read (from cache) per vector otherwise
-    constexpr bool KEEP_W = NCH <= 4;
-    s16x8 wv[KEEP_W ? NCH : 1];
-    if (KEEP_W) {
+    // the lane's share of the weight stays in registers for all the vectors the wave handles (re-reading it from
+    // cache per vector cost 5 % at 4096-6144 elements)
+    s16x8 wv[NCH];
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            const int c = j * LANES + gl;
-            wv[j] = c < chunks ? *reinterpret_cast<const s16x8*>((const short*)p.w + 8 * c) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
-        }
+    for (int j = 0; j < NCH; ++j) {
+        const int c = j * LANES + gl;
+        wv[j] = c < chunks ? *reinterpret_cast<const s16x8*>((const short*)p.w + 8 * c) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
     }
     for (int64_t v0 = wave * VPW; v0 < p.n_vec; v0 += n_waves * VPW) {
         const int64_t vec = v0 + lane / LANES;
@@ -81,10 +79,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const NormPa
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
             const int c = j * LANES + gl;
-            if (on && c < chunks) {
-                const s16x8 wj = KEEP_W ? wv[KEEP_W ? j : 0] : *reinterpret_cast<const s16x8*>((const short*)p.w + 8 * c);
-                *reinterpret_cast<s16x8*>(dst + 8 * c) = scale8w<T>(x[j], wj, sc);
-            }
+            if (on && c < chunks) *reinterpret_cast<s16x8*>(dst + 8 * c) = scale8w<T>(x[j], wv[j], sc);
         }
     }
 }
@@ -160,7 +155,9 @@ static void launch_norm(const NormParams& p, bool vec_ok, hipStream_t stream) {
         else if (chunks <= 64) MINFER_ROWS(64, 1)
         else if (chunks <= 128) MINFER_ROWS(64, 2)
         else if (chunks <= 256) MINFER_ROWS(64, 4)
+        else if (chunks <= 384) MINFER_ROWS(64, 6)
         else if (chunks <= 512) MINFER_ROWS(64, 8)
+        else if (chunks <= 768) MINFER_ROWS(64, 12)
         else MINFER_ROWS(64, 16)
 #undef MINFER_ROWS
     } else {
