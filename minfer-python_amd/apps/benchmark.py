@@ -1,7 +1,7 @@
-"""Times the attention ops against the PyTorch reference statements, one table per op.
+"""Times the ops of the attention path against the PyTorch reference statements, one table per op.
 
-Same command-line shape and timing method as the reference's benchmark script
-(reference: apps/benchmark.py:210-290): torch.utils.benchmark.Timer.blocked_autorange per shape,
+Same command-line shape, test cases and timing method as the reference's benchmark script
+(reference: apps/benchmark.py:18-290): torch.utils.benchmark.Timer.blocked_autorange per shape,
 Compare(...).print(); for `--which ref` the GQA expansion of K/V is outside the timed closure.
 """
 import argparse
@@ -80,8 +80,111 @@ def flash_attn_varlen(backend: str, which: str):
     Compare([_measure(fn, f"16 seqs, T={q.shape[2]}, n_heads=64, n_kv_heads=8, head_dim=128", which, "flash_attn_varlen")]).print()
 
 
+def _table(label, cases, make, which):
+    """One Timer row per case; make(case) returns (sub_label, minfer closure, ref closure)."""
+    results = []
+    for case in cases:
+        sub_label, mine, ref = make(case)
+        with torch.no_grad():
+            results.append(_measure(mine if which == "minfer" else ref, sub_label, which, label))
+        del mine, ref
+        gc.collect()
+        torch.cuda.empty_cache()
+    Compare(results).print()
+
+
+def flash_attn_decode_q8_0(backend: str, which: str):
+    """Decode over Q8_0 caches; `ref` is the fp16 decode op over the dequantised caches."""
+    kerns = KernelBackend(backend)
+    q8 = GGMLQuantizationType.Q8_0
+
+    def make(B):
+        q, kc, vc, ctx = workloads.decode_cache(device="cuda", B=B)
+        out = torch.zeros_like(q)
+        kq, vq = workloads.q8_0_rows(kc), workloads.q8_0_rows(vc)
+        return (f"B={B}, ctx~U[512,8192], n_heads=32, n_kv_heads=8, head_dim=128",
+                lambda: kerns.flash_attn_decode(q8, *GGML_QUANT_SIZES[q8], q, kq, vq, ctx, out),
+                lambda: kerns.flash_attn_decode(QT, QB, QS, q, kc, vc, ctx, out))
+    _table("flash_attn_decode_q8_0", [16, 64], make, which)
+
+
+def rmsnorm(backend: str, which: str):
+    """The reference's cases (reference: apps/benchmark.py:23-32): per token and per head, L = 1024..16384."""
+    kerns = KernelBackend(backend)
+
+    def make(case):
+        B, L, shape, eps = case
+        x = torch.randn((B, L, *shape), dtype=torch.float16, device="cuda")
+        w = shape[-1] ** -0.5 * torch.randn(shape[-1], dtype=torch.float16, device="cuda")
+        out = torch.zeros_like(x)
+        what = f"hidden_dim={shape[-1]}" if len(shape) == 1 else f"n_heads={shape[0]}, head_dim={shape[1]}"
+        return f"B={B}, L={L}, {what}", lambda: kerns.rmsnorm(eps, x, w, out), lambda: refs.rmsnorm(x, w, eps)
+    _table("rmsnorm", [(8, L, shape, 1e-6) for shape in ((6144,), (48, 128)) for L in (1024, 4096, 8192, 16384)], make, which)
+
+
+def _rope(name, backend, which):
+    """The reference's cases (reference: apps/benchmark.py:74-79, :118-123): x [8, L, 48, 128], rotary 64, base 1e6."""
+    kerns = KernelBackend(backend)
+
+    def make(L):
+        x = torch.randn((8, L, 48, 128), dtype=torch.float16, device="cuda")
+        return (f"B=8, L={L}, n_heads=48, head_dim=128, rotary_dim=64",
+                lambda: getattr(kerns, name)(64, 0, 1e6, x), lambda: getattr(refs, name)(x, 64, 0, 1e6))
+    _table(name, [1024, 4096, 8192, 16384], make, which)
+
+
+def il_rope(backend: str, which: str):
+    _rope("il_rope", backend, which)
+
+
+def neox_rope(backend: str, which: str):
+    _rope("neox_rope", backend, which)
+
+
+def rope_kv_append(backend: str, which: str):
+    """The fused producer at the Llama-3-8B head shape, into fp16 and into Q8_0 caches; `ref` is the statements it
+    replaces (rope q, rope k, two transposed copies)."""
+    kerns = KernelBackend(backend)
+
+    def make(case):
+        L, q8 = case
+        q, k, v, pos, kc, vc = workloads.kv_append(device="cuda", B=8, L=L)
+        if q8:
+            kc = torch.zeros(kc.shape[:-1] + (kc.shape[-1] // 32 * 34,), dtype=torch.uint8, device="cuda")
+            vc = torch.zeros_like(kc)
+
+        def ref():
+            refs.neox_rope(q, 128, 0, 5e5)
+            rk = refs.neox_rope(k, 128, 0, 5e5).transpose(1, 2)
+            if q8:
+                rk, rv = workloads.q8_0_rows(rk.contiguous()), workloads.q8_0_rows(v.transpose(1, 2).contiguous())
+                kc[:, :, :L], vc[:, :, :L] = rk, rv
+            else:
+                kc[:, :, :L], vc[:, :, :L] = rk, v.transpose(1, 2)
+        return (f"B=8, L={L}, n_heads=32, n_kv_heads=8, head_dim=128, {'Q8_0' if q8 else 'fp16'} caches",
+                lambda: kerns.rope_kv_append(1, 128, 5e5, q, k, v, pos, kc, vc), ref)
+    _table("rope_kv_append", [(L, q8) for q8 in (False, True) for L in (1024, 4096)], make, which)
+
+
+def gemm(backend: str, which: str):
+    """The reference's cases (reference: apps/benchmark.py:164-166): M = K = N = 512..8192, four (alpha, beta)."""
+    kerns = KernelBackend(backend)
+
+    def make(case):
+        s, alpha, beta = case
+        a, w, bias = workloads.gemm_input(s, s, s, device="cuda")
+        out = torch.zeros_like(bias)
+        return (f"alpha={alpha}, beta={beta}, M={s}, K={s}, N={s}",
+                lambda: kerns.gemm(QT, QB, QS, alpha, beta, a, w, bias, out),
+                lambda: refs.gemm(a[0], w, bias[0], out[0], alpha, beta))
+    _table("gemm", [(s, al, be) for s in (512, 1024, 2048, 4096, 8192) for al, be in ((1.0, 0.0), (1.0, 1.0), (2.0, 3.0), (0.5, 2.0))],
+           make, which)
+
+
 if __name__ == "__main__":
-    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen}
+    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
+               "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "rmsnorm": rmsnorm, "il_rope": il_rope, "neox_rope": neox_rope,
+               "rope_kv_append": rope_kv_append, "gemm": gemm}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)
