@@ -194,6 +194,14 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     short* Oh = (short*)p.out + (MODE == MODE_DENSE ? (int64_t)b * p.o0 : 0) + (int64_t)head * p.o1 + (int64_t)seq_lo * p.o2;
     const uint8_t* mrow = MODE == MODE_DENSE ? p.mask + ((size_t)b * p.L + min(qrow, last_row)) * p.L : nullptr;
 
+    // the wave's Q rows are requested now and used after the tile list is built, so that the two latencies overlap
+    s16x8 q_raw[KC];
+    {
+        const short* src = Qh + (int64_t)min(qrow, last_row) * p.q2 + 8 * h;
+#pragma unroll
+        for (int c = 0; c < KC; ++c) q_raw[c] = *reinterpret_cast<const s16x8*>(src + 16 * c);
+    }
+
     // ---- list of key tiles this workgroup visits ---------------------------------------------
     // entry = key tile | (2-bit class for each 64-row query tile the workgroup overlaps) << 16
     const int qt64_first = (qtile * QBW * 32) >> 6;
@@ -229,13 +237,11 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
     // Q is multiplied by scale*log2(e) once, here, so that the MFMA accumulator of Q K^T is directly
     // the base-2 exponent of the softmax weight (minus the running reference it is initialised with).
+    // (The loads were requested before the tile list was built.)
     const float c2 = p.scale_log2;
     s16x8 qf[KC];
-    {
-        const short* src = Qh + (int64_t)min(qrow, last_row) * p.q2 + 8 * h;
 #pragma unroll
-        for (int c = 0; c < KC; ++c) qf[c] = T::scale8(*reinterpret_cast<const s16x8*>(src + 16 * c), c2);
-    }
+    for (int c = 0; c < KC; ++c) qf[c] = T::scale8(q_raw[c], c2);
 
     // ---- global -> LDS tile copy ----------------------------------------------------------
     // Instruction j of this wave fills rows (j*kWaves + w)*RPI .. +RPI-1 of the tile; the lane's byte
