@@ -625,12 +625,13 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
         }
     };
     // Everything is requested at once: how many partial results the row has, and, before that is known, every
-    // slot's (max, sum) and the first eight slots' O (slots past the count hold stale bytes and are discarded).
+    // slot's (max, sum) and the first four slots' O (slots past the count hold stale bytes and are discarded).
     const int sl = min(lane, p.S - 1);
     const float m_raw = p.part_ml[(slot0 + sl) * 2], l_raw = p.part_ml[(slot0 + sl) * 2 + 1];
+    constexpr int kEarly = 4;
     float x[8][EPL];
 #pragma unroll
-    for (int u = 0; u < 8; ++u) load_o(min(u, p.S - 1), x[u]);
+    for (int u = 0; u < kEarly; ++u) load_o(min(u, p.S - 1), x[u]);
     // the partial results of this row: one per share of the line that overlaps the rows of its (sequence, KV head)
     const int n_b = groups_of(p, p.ctx[b]);
     const int quota = work_quota(p, p.seq_off[p.B]);
@@ -652,6 +653,9 @@ __global__ __launch_bounds__(256) void decode_combine_kernel(const DecodeParams 
         if (s0 > 0) {
 #pragma unroll
             for (int u = 0; u < 8; ++u) load_o(min(s0 + u, ns - 1), x[u]);
+        } else {
+#pragma unroll
+            for (int u = kEarly; u < 8; ++u) load_o(min(u, ns - 1), x[u]);
         }
 #pragma unroll
         for (int u = 0; u < 8; ++u) {
