@@ -62,17 +62,18 @@ MA_DEV f32x2 table_entry(double inv_freq, int pos) {
 }
 
 // Per token: every thread requests the 16-byte chunks it owns (a few in flight), the first rd/2 threads
-// meanwhile fill the token's cos/sin table, one barrier, then rotate and store.  The fused producer requests
-// the first chunks of its next token before it works on the current one.
+// meanwhile fill the token's cos/sin table, one barrier, then rotate and store.  The producer into Q8_0 caches
+// requests the first chunks of its next token before it works on the current one.
 //
 // Chunk numbering inside a token.  Rotary chunks of a tensor with NH heads: interleaved style, chunk c of
 // head hd covers elements 8c..8c+7 (pairs 4c..4c+3), rd/8 chunks per head; NeoX style, chunk c covers
 // elements 8c..8c+7 and their partners rd/2 + 8c.., rd/16 chunks per head.  Sections, in order: q rotary,
 // then (fused only) k rotary, k tail (elements rd..D-1, copied), v (copied).
 template <class T, int STYLE, bool FUSED, bool Q8 = false>
-__global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) {
+__global__ __launch_bounds__(kRopeThreads, FUSED ? 1 : 8) void rope_kernel(const RopeParams p) {
     static_assert(FUSED || !Q8, "only the fused producer writes a cache");
     __shared__ f32x2 tab[2][kMaxPairs];
+    __shared__ double freq[kMaxPairs];   // the kernel argument array, where a thread can index it cheaply
     const int tid = threadIdx.x;
     const int half_rd = p.rd >> 1;
     const int cph = STYLE == ROPE_IL ? p.rd >> 3 : p.rd >> 4;   // rotary chunks per head
@@ -81,8 +82,14 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
     const int n_kr = FUSED ? p.Hkv * cph : 0;
     const int n_kt = FUSED ? p.Hkv * tail : 0;
     const int n_v = FUSED ? p.Hkv * (p.D >> 3) : 0;
-    const int n_all = n_q + n_kr + n_kt + n_v;
+    // Chunk numbers of a token: sections in the order above, each starting at a multiple of the wave size, so that the
+    // 64 chunks a wave takes at a time are of one kind and its base pointers and branches are scalar.
+    const int k_begin = FUSED ? (n_q + 63) & ~63 : n_q;
+    const int kt_begin = FUSED ? (k_begin + n_kr + 63) & ~63 : n_q;
+    const int v_begin = FUSED ? (kt_begin + n_kt + 63) & ~63 : n_q;
+    const int n_all = FUSED ? v_begin + n_v : n_q;
     const int tokens = p.B * p.L;
+    if (tid < half_rd) freq[tid] = p.inv_freq[tid];   // read back by the same thread only
 
     // what a token's chunks are addressed from
     struct Token {
@@ -105,53 +112,49 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
         k.qv = Q8 ? (char*)p.v_cache + (int64_t)b * p.c0 + (int64_t)k.pos * p.c2 : nullptr;
         return k;
     };
-    // Where chunk t of the token lives: kind 0 rotate, 1 copy, 2 nothing.  Evaluated once to request the
-    // chunk and again to store it (the index is made opaque in between), so that only the loaded data
-    // stays in registers across the barrier.
-    // For a Q8_0 cache, crow is the (row, head) the chunk belongs to and elem its first element there.
-    auto locate = [&](const Token& k, int t, const short*& src, short*& dst, int& kind, int& chunk, char*& crow, int& elem) __attribute__((always_inline)) {
-        src = k.xq; dst = k.xq; kind = 2; chunk = 0; crow = nullptr; elem = 0;
-        if (t < n_q) {
-            const int hd = t / cph; chunk = t - hd * cph;
-            src = dst = k.xq + hd * p.D + 8 * chunk;
-            kind = 0;
-        } else if (FUSED && t < n_all && k.row_ok) {
-            t -= n_q;
-            if (t < n_kr) {
-                const int hd = t / cph; chunk = t - hd * cph;
-                src = k.xk + hd * p.D + 8 * chunk;
-                if (Q8) { crow = k.qk + hd * p.c1; elem = 8 * chunk; }
-                else dst = k.ck + hd * p.c1 + 8 * chunk;
-                kind = 0;
-            } else if (t < n_kr + n_kt) {
-                t -= n_kr;
-                const int hd = t / tail, c = t - hd * tail;
-                src = k.xk + hd * p.D + p.rd + 8 * c;
-                if (Q8) { crow = k.qk + hd * p.c1; elem = p.rd + 8 * c; }
-                else dst = k.ck + hd * p.c1 + p.rd + 8 * c;
-                kind = 1;
-            } else {
-                t -= n_kr + n_kt;
-                const int per = p.D >> 3, hd = t / per, c = t - hd * per;
-                src = k.xv + hd * p.D + 8 * c;
-                if (Q8) { crow = k.qv + hd * p.c1; elem = 8 * c; }
-                else dst = k.cv + hd * p.c1 + 8 * c;
-                kind = 1;
-            }
+    // Which chunk of a token a thread works on, and where that chunk sits inside the token's q, k, v and cache rows,
+    // does not depend on the token: a slot is worked out once (integer divisions) and then only added to the token's
+    // base pointers.  sect is the same for all lanes of a wave; elem is the chunk's first element inside its head.
+    enum { Q_ROT = 0, K_ROT = 1, K_COPY = 2, V_COPY = 3 };
+    struct Slot {
+        int sect; uint32_t where;     // where: head << 16 | elem, all ones = no chunk for this lane
+        MA_DEV bool valid() const { return where != ~0u; }
+        MA_DEV int hd() const { return (int)(where >> 16); }
+        MA_DEV int elem() const { return (int)(where & 0xffffu); }
+    };
+    auto place = [&](int t) __attribute__((always_inline)) {
+        const int w0 = __builtin_amdgcn_readfirstlane(t) & ~63;   // a wave's lanes hold 64 consecutive numbers
+        int sect = Q_ROT, begin = 0, n = n_q, per = cph, elem0 = 0;
+        if (FUSED && w0 >= k_begin) {
+            if (w0 < kt_begin) { sect = K_ROT; begin = k_begin; n = n_kr; }
+            else if (w0 < v_begin) { sect = K_COPY; begin = kt_begin; n = n_kt; per = tail; elem0 = p.rd; }
+            else { sect = V_COPY; begin = v_begin; n = n_v; per = p.D >> 3; }
         }
+        const int i = t - begin, hd = i / per;
+        return Slot{sect, i < n ? (uint32_t)hd << 16 | (uint32_t)(elem0 + 8 * (i - hd * per)) : ~0u};
+    };
+    auto live = [&](const Token& k, const Slot& s) __attribute__((always_inline)) {
+        return s.valid() && (s.sect == Q_ROT || k.row_ok);
     };
     // chunks in flight per thread and buffer: a NeoX rotary chunk is two 16-byte pieces, so half as many
     constexpr int UN = STYLE == ROPE_IL ? 4 : 2;
     struct Buffer { s16x8 lo[UN], hi[UN]; };
-    auto request = [&](const Token& k, int t0, Buffer& buf) __attribute__((always_inline)) {
+    struct Slots { Slot s[UN]; };
+    auto place_batch = [&](int t0) __attribute__((always_inline)) {
+        Slots b;
+#pragma unroll
+        for (int u = 0; u < UN; ++u) b.s[u] = place(t0 + u * kRopeThreads);
+        return b;
+    };
+    auto request = [&](const Token& k, const Slots slots, Buffer& buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const short* src; short* dst; int kind, chunk, elem; char* crow;
-            locate(k, t0 + u * kRopeThreads, src, dst, kind, chunk, crow, elem);
+            const Slot s = slots.s[u];
+            const short* src = (s.sect == Q_ROT ? k.xq : s.sect == V_COPY ? k.xv : k.xk) + (s.hd() * p.D + s.elem());
             buf.lo[u] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (kind != 2) buf.lo[u] = *reinterpret_cast<const s16x8*>(src);
+            if (live(k, s)) buf.lo[u] = *reinterpret_cast<const s16x8*>(src);
             buf.hi[u] = buf.lo[u];
-            if (STYLE == ROPE_NEOX && kind == 0) buf.hi[u] = *reinterpret_cast<const s16x8*>(src + half_rd);
+            if (STYLE == ROPE_NEOX && live(k, s) && s.sect <= K_ROT) buf.hi[u] = *reinterpret_cast<const s16x8*>(src + half_rd);
         }
     };
     // 8 values to their place: as they are, or (Q8_0 cache) quantised with the block's three other lanes
@@ -167,15 +170,18 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
             *reinterpret_cast<s16x8*>(dst) = val;
         }
     };
-    auto finish = [&](const Token& k, int t0, const Buffer& buf, int parity) __attribute__((always_inline)) {
-        asm volatile("" : "+v"(t0));
+    auto finish = [&](const Token& k, const Slots slots, const Buffer& buf, int parity) __attribute__((always_inline)) {
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
-            const short* src; short* dst; int kind, chunk, elem; char* crow;
-            locate(k, t0 + u * kRopeThreads, src, dst, kind, chunk, crow, elem);
-            if (kind == 2) continue;
+            const Slot s = slots.s[u];
+            if (!live(k, s)) continue;
+            short* dst = nullptr; char* crow = nullptr;
+            const int elem = s.elem(), chunk = elem >> 3;
+            if (s.sect == Q_ROT) dst = k.xq + (s.hd() * p.D + elem);
+            else if (Q8) crow = (s.sect == V_COPY ? k.qv : k.qk) + s.hd() * p.c1;
+            else dst = (s.sect == V_COPY ? k.cv : k.ck) + (s.hd() * p.c1 + elem);
             s16x8 a = buf.lo[u];
-            if (kind == 0) {
+            if (s.sect <= K_ROT) {
                 if (STYLE == ROPE_IL) {
 #pragma unroll
                     for (int j = 0; j < 4; ++j) {
@@ -199,48 +205,53 @@ __global__ __launch_bounds__(kRopeThreads) void rope_kernel(const RopeParams p) 
             put(dst, crow, elem, a);
         }
     };
+    // the slots of a thread's first batch of chunks, and the frequency of the table entry it computes
+    const Slots first = place_batch(tid);
     // One token: its table (the token's first chunks are already on their way in `buf`), the one barrier of the
     // token (the next token writes the other table), rotate and store, then any further batches of chunks.
     auto one_token = [&](const Token& k, Buffer& buf, int parity) __attribute__((always_inline)) {
-        if (tid < half_rd) tab[parity][tid] = table_entry(p.inv_freq[tid], k.pos);
+        if (tid < half_rd) tab[parity][tid] = table_entry(freq[tid], k.pos);
         __syncthreads();
-        finish(k, tid, buf, parity);
+        finish(k, first, buf, parity);
         for (int t0 = tid + UN * kRopeThreads; t0 < n_all; t0 += UN * kRopeThreads) {
-            request(k, t0, buf);
-            finish(k, t0, buf, parity);
+            const Slots more = place_batch(t0);
+            request(k, more, buf);
+            finish(k, more, buf, parity);
         }
     };
 
     const int stride = gridDim.x;
     int tok = blockIdx.x;
     if (tok >= tokens) return;
-    if (!FUSED) {
-        // in place: one token at a time (fetching ahead costs registers and gains nothing here: -2..-5 %)
+    if (!(FUSED && Q8)) {
+        // One token at a time.  With every compute unit holding 7-8 workgroups the memory system is saturated as it
+        // is: fetching a token ahead costs registers, hence resident workgroups, and is 2-6 % slower, in place as
+        // into fp16 caches.
         Buffer buf;
         int parity = 0;
         for (; tok < tokens; tok += stride, parity ^= 1) {
             const Token k = token_at(tok);
-            request(k, tid, buf);
+            request(k, first, buf);
             one_token(k, buf, parity);
         }
         return;
     }
-    // The fused producer (+2.5 %, +6 % into Q8_0 caches): two tokens per trip, so that the two buffers are fixed
-    // registers; while a token is rotated and stored, the first chunks of the workgroup's next token are already in
-    // flight in the other buffer.
+    // Into Q8_0 caches the quantiser's dependent chain makes a token long, and fetching ahead pays (+7 %): two
+    // tokens per trip, so that the two buffers are fixed registers; while a token is rotated, quantised and stored,
+    // the first chunks of the workgroup's next token are already in flight in the other buffer.
     Buffer buf_a, buf_b;
     Token cur = token_at(tok);
-    request(cur, tid, buf_a);
+    request(cur, first, buf_a);
     for (;;) {
         const bool more_b = tok + stride < tokens;
         const Token nxt = token_at(more_b ? tok + stride : tok);
-        if (more_b) request(nxt, tid, buf_b);
+        if (more_b) request(nxt, first, buf_b);
         one_token(cur, buf_a, 0);
         if (!more_b) break;
         tok += stride;
         const bool more_a = tok + stride < tokens;
         cur = token_at(more_a ? tok + stride : tok);
-        if (more_a) request(cur, tid, buf_a);
+        if (more_a) request(cur, first, buf_a);
         one_token(nxt, buf_b, 1);
         if (!more_a) break;
         tok += stride;
@@ -279,7 +290,7 @@ static int fill_rope(RopeParams& p, int dtype, int style, int64_t B, int64_t L, 
     if (rotary_dim % 2 != 0) return bad("rotary_dim must be even");
     if (rotary_dim > 2 * kMaxPairs) return bad("rotary_dim > 256 unsupported");
     if (!(freq_base > 0.0)) return bad("freq_base must be positive");
-    if (B * L > 0x7fffffffLL || H > 65535 || D > 65535) return bad("problem too large");
+    if (B * L > 0x7fffffffLL || H > 65535 || D > 65535 || H * D > 0x7fffffffLL) return bad("problem too large");
     p.B = (int)B; p.L = (int)L; p.H = (int)H; p.D = (int)D; p.rd = (int)rotary_dim;
     for (int i = 0; i < rotary_dim / 2; ++i) p.inv_freq[i] = pow(freq_base, -2.0 * i / (double)rotary_dim);
     return MINFER_ATTN_OK;

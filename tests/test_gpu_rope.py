@@ -117,6 +117,7 @@ def run_append(style, q, k, v, pos, kc, vc, rd, base):
     (2, 40, 8, 2, 128, 64, 128, [24, 0]),
     (4, 1, 32, 8, 128, 96, 64, [95, 0, 50, 96]),  # decode step; sequence 3 is full (row 96 does not exist)
     (1, 3, 2, 1, 16, 8, 0, [2]),                  # rotary_dim 0: pure append
+    (1, 6, 80, 10, 128, 16, 96, [3]),             # more chunks per token than one pass of the workgroup takes
 ])
 def test_kv_append_matches_oracle(style, dtype, B, L, Hq, Hkv, D, Lmax, rd, pos):
     g = torch.Generator().manual_seed(B * 100 + L)
