@@ -251,12 +251,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
             const int row = j * RPI + lane / G;
-            kk[j] = *reinterpret_cast<const s16x8*>(Kb + (int64_t)min(r0 + row, row_hi - 1) * p.kv2 + 8 * (lane % G));
+            kk[j] = stream_load(reinterpret_cast<const s16x8*>(Kb + (int64_t)min(r0 + row, row_hi - 1) * p.kv2 + 8 * (lane % G)));
         }
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
             const int row = j * RPI + lane / G;
-            vv[j] = *reinterpret_cast<const s16x8*>(Vb + (int64_t)min(r0 + row, row_hi - 1) * p.kv2 + 8 * (lane % G));
+            vv[j] = stream_load(reinterpret_cast<const s16x8*>(Vb + (int64_t)min(r0 + row, row_hi - 1) * p.kv2 + 8 * (lane % G)));
         }
     };
     // Loads and the consume step below are issued unconditionally (rows are clamped into the chunk and
@@ -453,13 +453,13 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
         for (int j = 0; j < NL; ++j) {
             int64_t goff;
             const int off = piece_offset(t, j, last_k, goff);
-            st.k[j] = *reinterpret_cast<const u32x4*>(kb16 + goff + off);
+            st.k[j] = stream_load(reinterpret_cast<const u32x4*>(kb16 + goff + off));
         }
 #pragma unroll
         for (int j = 0; j < NL; ++j) {
             int64_t goff;
             const int off = piece_offset(t, j, last_v, goff);
-            st.v[j] = *reinterpret_cast<const u32x4*>(vb16 + goff + off);
+            st.v[j] = stream_load(reinterpret_cast<const u32x4*>(vb16 + goff + off));
         }
     };
 #pragma unroll
