@@ -169,13 +169,11 @@ MA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 // Loads and stores of bytes that a kernel touches once (cache rows being streamed, rows of a normalisation):
 // marked non-temporal, so that the caches between the compute units and HBM do not keep the lines.  On this chip
 // that alone raises the HBM throughput of a streaming kernel by 10-15 %.
-#ifdef MINFER_NO_STREAM_HINT
-template <class V> MA_DEV V stream_load(const V* p) { return *p; }
-template <class V> MA_DEV void stream_store(V* p, V v) { *p = v; }
-#else
 template <class V> MA_DEV V stream_load(const V* p) { return __builtin_nontemporal_load(p); }
 template <class V> MA_DEV void stream_store(V* p, V v) { __builtin_nontemporal_store(v, p); }
-#endif
+// The same with the choice made per launch (template argument): see kStreamBytes on the host side.
+template <bool STREAM, class V> MA_DEV V load_once(const V* p) { return STREAM ? __builtin_nontemporal_load(p) : *p; }
+template <bool STREAM, class V> MA_DEV void store_once(V* p, V v) { if (STREAM) __builtin_nontemporal_store(v, p); else *p = v; }
 
 MA_DEV int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 

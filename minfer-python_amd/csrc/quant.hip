@@ -49,7 +49,7 @@ __global__ __launch_bounds__(kQuantThreads) void quant_q8_0_kernel(const void* x
 }
 
 // x: n_blocks * 34 bytes; y: n_blocks * 32 values.  DST: 0 fp32, 1 fp16.
-template <int DST>
+template <int DST, bool STREAM>
 __global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kernel(const char* x, void* y, int64_t n_blocks) {
     if (DST == 0) {
         // fp32 output is 4 bytes out per byte in: a lane takes 4 quants and stores one 16-byte piece, so that every
@@ -66,7 +66,7 @@ __global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kernel(const char*
             f32x4 a;
 #pragma unroll
             for (int j = 0; j < 4; ++j) a[j] = (float)(int8_t)(q >> (8 * j)) * d;
-            ((f32x4*)y)[i] = a;
+            store_once<STREAM>((f32x4*)y + i, a);
         }
         return;
     }
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kernel(const char*
         if (DST == 1) {
             const _Float16 dh = __builtin_bit_cast(_Float16, d_bits);
             const h16x2 d2 = {dh, dh};
-            ((s16x8*)y)[i] = dequant8(q.x, q.y, d2);
+            store_once<STREAM>((s16x8*)y + i, dequant8(q.x, q.y, d2));
         } else {
             const float d = (float)__builtin_bit_cast(_Float16, d_bits);
             f32x4 a, b;
@@ -145,7 +145,13 @@ MINFER_ATTN_EXPORT int minfer_dequant_q8_0(int dst_dtype, const void* x, void* y
     if (n_blocks == 0) return MINFER_ATTN_OK;
     hipStream_t stream = (hipStream_t)stream_v;
     const dim3 grid(grid_for(n_blocks * 4)), block(kQuantThreads);
-    if (dst_dtype == MINFER_ATTN_F32) hipLaunchKernelGGL((dequant_q8_0_kernel<0>), grid, block, 0, stream, (const char*)x, y, n_blocks);
-    else hipLaunchKernelGGL((dequant_q8_0_kernel<1>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+    const bool streamed = n_blocks * (34 + 32 * (dst_dtype == MINFER_ATTN_F32 ? 4 : 2)) > kStreamBytes;
+    if (dst_dtype == MINFER_ATTN_F32) {
+        if (streamed) hipLaunchKernelGGL((dequant_q8_0_kernel<0, true>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+        else hipLaunchKernelGGL((dequant_q8_0_kernel<0, false>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+    } else {
+        if (streamed) hipLaunchKernelGGL((dequant_q8_0_kernel<1, true>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+        else hipLaunchKernelGGL((dequant_q8_0_kernel<1, false>), grid, block, 0, stream, (const char*)x, y, n_blocks);
+    }
     return check_launch("dequant_q8_0_kernel");
 }

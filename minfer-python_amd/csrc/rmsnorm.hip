@@ -44,7 +44,7 @@ template <class T> MA_DEV s16x8 scale8w(s16x8 v, s16x8 w, float sc) {
 
 // LANES lanes per vector, NCH 16-byte chunks per lane (dim <= LANES * 8 * NCH, dim % 8 == 0): chunk j of a
 // lane covers elements 8 * (j * LANES + lane_in_group) .., so a group reads contiguous 16 * LANES bytes.
-template <class T, int LANES, int NCH>
+template <class T, int LANES, int NCH, bool STREAM>
 __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const NormParams p) {
     const int lane = threadIdx.x & 63, gl = lane & (LANES - 1);
     constexpr int VPW = 64 / LANES;                               // vectors per wave
@@ -68,7 +68,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const NormPa
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
             const int c = j * LANES + gl;
-            x[j] = (on && c < chunks) ? *reinterpret_cast<const s16x8*>(src + 8 * c) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            x[j] = (on && c < chunks) ? load_once<STREAM>(reinterpret_cast<const s16x8*>(src + 8 * c)) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
         for (int j = 0; j < NCH; ++j) ss += sum_sq8<T>(x[j]);
@@ -79,7 +79,7 @@ __global__ __launch_bounds__(kNormThreads) void rmsnorm_rows_kernel(const NormPa
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
             const int c = j * LANES + gl;
-            if (on && c < chunks) *reinterpret_cast<s16x8*>(dst + 8 * c) = scale8w<T>(x[j], wv[j], sc);
+            if (on && c < chunks) store_once<STREAM>(reinterpret_cast<s16x8*>(dst + 8 * c), scale8w<T>(x[j], wv[j], sc));
         }
     }
 }
@@ -143,11 +143,13 @@ static void launch_norm(const NormParams& p, bool vec_ok, hipStream_t stream) {
     const int waves_cap = 256 * 8 * 4;   // resident waves of the chip, times a few
     if (vec_ok && p.dim <= 8192) {
         const int chunks = p.dim >> 3;
+        const bool streamed = 2 * p.n_vec * p.dim * 2 > kStreamBytes;   // input and output
 #define MINFER_ROWS(LANES, NCH)                                                                                   \
     {                                                                                                             \
         const int64_t waves = (p.n_vec + (64 / LANES) - 1) / (64 / LANES);                                        \
         const int grid = (int)std::min<int64_t>((waves + 3) / 4, waves_cap / 4);                                  \
-        hipLaunchKernelGGL((rmsnorm_rows_kernel<T, LANES, NCH>), dim3(grid), dim3(kNormThreads), 0, stream, p);   \
+        if (streamed) hipLaunchKernelGGL((rmsnorm_rows_kernel<T, LANES, NCH, true>), dim3(grid), dim3(kNormThreads), 0, stream, p);  \
+        else hipLaunchKernelGGL((rmsnorm_rows_kernel<T, LANES, NCH, false>), dim3(grid), dim3(kNormThreads), 0, stream, p);          \
     }
         if (chunks <= 8) MINFER_ROWS(8, 1)
         else if (chunks <= 16) MINFER_ROWS(16, 1)

@@ -69,7 +69,7 @@ MA_DEV f32x2 table_entry(double inv_freq, int pos) {
 // head hd covers elements 8c..8c+7 (pairs 4c..4c+3), rd/8 chunks per head; NeoX style, chunk c covers
 // elements 8c..8c+7 and their partners rd/2 + 8c.., rd/16 chunks per head.  Sections, in order: q rotary,
 // then (fused only) k rotary, k tail (elements rd..D-1, copied), v (copied).
-template <class T, int STYLE, bool FUSED, bool Q8 = false>
+template <class T, int STYLE, bool FUSED, bool Q8, bool STREAM>
 __global__ __launch_bounds__(kRopeThreads, FUSED ? 1 : 8) void rope_kernel(const RopeParams p) {
     static_assert(FUSED || !Q8, "only the fused producer writes a cache");
     __shared__ f32x2 tab[2][kMaxPairs];
@@ -152,9 +152,9 @@ __global__ __launch_bounds__(kRopeThreads, FUSED ? 1 : 8) void rope_kernel(const
             const Slot s = slots.s[u];
             const short* src = (s.sect == Q_ROT ? k.xq : s.sect == V_COPY ? k.xv : k.xk) + (s.hd() * p.D + s.elem());
             buf.lo[u] = s16x8{0, 0, 0, 0, 0, 0, 0, 0};
-            if (live(k, s)) buf.lo[u] = *reinterpret_cast<const s16x8*>(src);
+            if (live(k, s)) buf.lo[u] = load_once<STREAM>(reinterpret_cast<const s16x8*>(src));
             buf.hi[u] = buf.lo[u];
-            if (STYLE == ROPE_NEOX && live(k, s) && s.sect <= K_ROT) buf.hi[u] = *reinterpret_cast<const s16x8*>(src + half_rd);
+            if (STYLE == ROPE_NEOX && live(k, s) && s.sect <= K_ROT) buf.hi[u] = load_once<STREAM>(reinterpret_cast<const s16x8*>(src + half_rd));
         }
     };
     // 8 values to their place: as they are, or (Q8_0 cache) quantised with the block's three other lanes
@@ -167,7 +167,7 @@ __global__ __launch_bounds__(kRopeThreads, FUSED ? 1 : 8) void rope_kernel(const
             const uint2 q = quant8_q8_0(f, d_bits);
             store_q8_piece(crow + (elem >> 5) * 34, elem & 31, q, d_bits);
         } else {
-            *reinterpret_cast<s16x8*>(dst) = val;
+            store_once<STREAM>(reinterpret_cast<s16x8*>(dst), val);
         }
     };
     auto finish = [&](const Token& k, const Slots slots, const Buffer& buf, int parity) __attribute__((always_inline)) {
@@ -300,17 +300,26 @@ static bool vector_ok(int style, int64_t D, int64_t rd) {
     return D % 8 == 0 && rd % (style == ROPE_IL ? 8 : 16) == 0;
 }
 
+template <bool FUSED, bool Q8, bool STREAM>
+static void launch_rope_as(int dtype, int style, const RopeParams& p, int grid, hipStream_t stream) {
+    if (dtype == MINFER_ATTN_F16) {
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<F16, ROPE_IL, FUSED, Q8, STREAM>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_kernel<F16, ROPE_NEOX, FUSED, Q8, STREAM>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+    } else {
+        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<BF16, ROPE_IL, FUSED, Q8, STREAM>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+        else hipLaunchKernelGGL((rope_kernel<BF16, ROPE_NEOX, FUSED, Q8, STREAM>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
+    }
+}
+
 template <bool FUSED, bool Q8 = false>
 static int launch_rope(int dtype, int style, const RopeParams& p, hipStream_t stream) {
     const int tokens = p.B * p.L;
     const int grid = std::min(tokens, 256 * 16);
-    if (dtype == MINFER_ATTN_F16) {
-        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<F16, ROPE_IL, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
-        else hipLaunchKernelGGL((rope_kernel<F16, ROPE_NEOX, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
-    } else {
-        if (style == ROPE_IL) hipLaunchKernelGGL((rope_kernel<BF16, ROPE_IL, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
-        else hipLaunchKernelGGL((rope_kernel<BF16, ROPE_NEOX, FUSED, Q8>), dim3(grid), dim3(kRopeThreads), 0, stream, p);
-    }
+    // distinct bytes the launch touches: q's rotary part (in place), and for the producer k, v and their cache rows
+    int64_t touched = (int64_t)tokens * p.H * p.rd * 2;
+    if (FUSED) touched += (int64_t)tokens * p.Hkv * p.D * 2 * (Q8 ? 3 : 4);
+    if (touched > kStreamBytes) launch_rope_as<FUSED, Q8, true>(dtype, style, p, grid, stream);
+    else launch_rope_as<FUSED, Q8, false>(dtype, style, p, grid, stream);
     return check_launch("rope_kernel");
 }
 
