@@ -26,13 +26,13 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
 PREFILL_TRAFFIC_BYTES = 107374 * 1024
-DECODE_TRAFFIC_BYTES = 1094936 * 1024
-ROPE_TRAFFIC_BYTES = 393306 * 1024          # il_rope on [8,4096,48,128], rotary 64
-APPEND_TRAFFIC_BYTES = 786710 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
-NORM_TRAFFIC_BYTES = 786929 * 1024          # rmsnorm on [8,4096,6144]
+DECODE_TRAFFIC_BYTES = 1092838 * 1024
+ROPE_TRAFFIC_BYTES = 393312 * 1024          # il_rope on [8,4096,48,128], rotary 64
+APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
+NORM_TRAFFIC_BYTES = 786659 * 1024          # rmsnorm on [8,4096,6144]
 GEMM_TRAFFIC_BYTES = 230579 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
-DECODE_Q8_TRAFFIC_BYTES = 589554 * 1024     # decode over Q8_0 caches (split + combine)
-APPEND_Q8_TRAFFIC_BYTES = 737660 * 1024     # rope_kv_append into Q8_0 caches
+DECODE_Q8_TRAFFIC_BYTES = 598453 * 1024     # decode over Q8_0 caches (split + combine)
+APPEND_Q8_TRAFFIC_BYTES = 737585 * 1024     # rope_kv_append into Q8_0 caches
 
 
 class HipEvents:
@@ -286,7 +286,7 @@ def main():
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,
-                                   "traffic": NORM_TRAFFIC_BYTES, "kernel": "rmsnorm_rows_kernel<F16,64,12>", "algorithmic_bytes": nbytes}}
+                                   "traffic": NORM_TRAFFIC_BYTES, "kernel": "rmsnorm_rows_kernel<F16,64,12,streamed>", "algorithmic_bytes": nbytes}}
     rec["gemm"] = {"value": g_tf, "unit": "TFLOP/s", "ms": g_avg_ms, "median_ms": g_med_ms,
                    "workload": "gemm alpha=1 beta=0, A [1,4096,4096] x W [4096,4096] fp16 (reference README HGEMM table, M=K=N=4096)",
                    "published_reference_us": 605.3,
