@@ -477,8 +477,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
     // the lane, fixed for the whole kernel (rows and 64-block strides are multiples of 4 bytes).
     const bool k_odd = ((pre_k + (D == 128 ? quad : quad >> 1) * 34) & 2) != 0;
     const bool v_odd = ((pre_v + lane * 34) & 2) != 0;
-    const uint32_t k_sel_a = k_odd ? kQ8SelOddA : kQ8SelEvenA, k_sel_b = k_odd ? kQ8SelOddB : kQ8SelEvenB;
-    const uint32_t v_sel_a = v_odd ? kQ8SelOddA : kQ8SelEvenA, v_sel_b = v_odd ? kQ8SelOddB : kQ8SelEvenB;
+    const uint32_t k_sel = k_odd ? kQ8SelOdd : kQ8SelEven, v_sel = v_odd ? kQ8SelOdd : kQ8SelEven;
     // the block's scale from its first memory word (zero for rows past the chunk's end, whose bytes were never loaded)
     auto scale_of = [&](uint32_t w0, bool odd, bool row_ok) {
         const uint16_t bits = (uint16_t)(odd ? w0 >> 16 : w0);
@@ -512,7 +511,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
             s[h] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
             for (int c = 0; c < KC; ++c)
-                s[h] = T::mfma16(dequant8_shifted(wq[2 * c], wq[2 * c + 1], wq[2 * c + 2], k_sel_a, k_sel_b, d2), qf[c], s[h]);
+                s[h] = T::mfma16(dequant8_shifted(wq[2 * c], wq[2 * c + 1], wq[2 * c + 2], k_sel, d2), qf[c], s[h]);
             const int key0 = r0 + 16 * h + 4 * quad;
 #pragma unroll
             for (int r = 0; r < 4; ++r) s[h][r] = (key0 + r < row_hi) ? s[h][r] : -INFINITY;
@@ -537,7 +536,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
 #pragma unroll
             for (int j = 0; j < 4; ++j)
                 *reinterpret_cast<s16x8*>(rowp + 16 * ((4 * c + j) ^ sw)) =
-                    dequant8_shifted(wv[2 * j], wv[2 * j + 1], wv[2 * j + 2], v_sel_a, v_sel_b, d2);
+                    dequant8_shifted(wv[2 * j], wv[2 * j + 1], wv[2 * j + 2], v_sel, d2);
         }
         // ---- online softmax over this group's 32 keys ----------------------------------------------------
         float mx = fmaxf(fmaxf(fmaxf(s[0][0], s[0][1]), fmaxf(s[0][2], s[0][3])), fmaxf(fmaxf(s[1][0], s[1][1]), fmaxf(s[1][2], s[1][3])));

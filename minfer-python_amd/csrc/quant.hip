@@ -80,7 +80,7 @@ __global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kernel(const char*
         if (DST == 1) {
             const _Float16 dh = __builtin_bit_cast(_Float16, d_bits);
             const h16x2 d2 = {dh, dh};
-            store_once<STREAM>((s16x8*)y + i, dequant8(q.x, q.y, d2));
+            store_once<STREAM>((s16x8*)y + i, dequant8_words(q.x, q.y, d2));
         } else {
             const float d = (float)__builtin_bit_cast(_Float16, d_bits);
             f32x4 a, b;

@@ -9,44 +9,34 @@ namespace minfer_attn {
 // One Q8_0 block as a lane holds it: the 32 int8 in eight words, the scale's fp16 bits.
 struct Q8Block { uint4 lo, hi; uint32_t d; };
 
-// (half)(q * d) for the four int8 of a word (reference: cuda/quants/impls.cuh:121-143): q + 1152 is built
-// exactly by placing (q ^ 0x80) under the exponent of 1024, the subtraction is exact, and the packed
-// multiply rounds the exact product once, as the conversion of the fp32 product does.
-MA_DEV void dequant4(uint32_t w, h16x2 d2, uint32_t& out_lo, uint32_t& out_hi) {
-    const uint32_t x = w ^ 0x80808080u;
-    const h16x2 bias = {(_Float16)1152.f, (_Float16)1152.f};
-    const h16x2 a = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, x, 0x04010400u));
-    const h16x2 b = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(0x64646464u, x, 0x04030402u));
-    out_lo = __builtin_bit_cast(uint32_t, (a - bias) * d2);
-    out_hi = __builtin_bit_cast(uint32_t, (b - bias) * d2);
+// The four int8 of a word as fp16, exactly: sub-dword addressing lets the int16 -> fp16 conversion take one byte,
+// sign-extended, as its source and one half of the destination as its target, so a value costs one instruction
+// (building q + 1152 under the exponent byte of 1024 with a byte permute and an exclusive or, then subtracting, costs 1.5).
+MA_DEV void int8x4_to_f16(uint32_t w, uint32_t& out_lo, uint32_t& out_hi) {
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(out_lo) : "v"(w));
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1" : "+v"(out_lo) : "v"(w));
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_2" : "=v"(out_hi) : "v"(w));
+    asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3" : "+v"(out_hi) : "v"(w));
 }
-// the 8 fp16 values of words w0, w1 of a block
-MA_DEV s16x8 dequant8(uint32_t w0, uint32_t w1, h16x2 d2) {
+// (half)(q * d) for the 8 int8 of two quant words (reference: cuda/quants/impls.cuh:121-143): conversion, then one
+// packed multiply per pair, which rounds the exact product once, as the conversion of the fp32 product does.
+MA_DEV s16x8 dequant8_words(uint32_t a0, uint32_t a1, h16x2 d2) {
     uint4 u;
-    dequant4(w0, d2, u.x, u.y);
-    dequant4(w1, d2, u.z, u.w);
+    int8x4_to_f16(a0, u.x, u.y);
+    int8x4_to_f16(a1, u.z, u.w);
+    u.x = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2, u.x) * d2);
+    u.y = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2, u.y) * d2);
+    u.z = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2, u.z) * d2);
+    u.w = __builtin_bit_cast(uint32_t, __builtin_bit_cast(h16x2, u.w) * d2);
     return __builtin_bit_cast(s16x8, u);
 }
 
-// The same from a block that is only 2-byte aligned, read as aligned words: `lo`, `hi` are consecutive words of
-// memory and the four int8 wanted start at byte 2 of `lo` (block on a 4-byte boundary: sel_a, sel_b =
-// kQ8SelEvenA, kQ8SelEvenB) or are `hi` itself (block 2 bytes past one: kQ8SelOddA, kQ8SelOddB).  The byte
-// permute that spreads the quants under the exponent bytes does the shift on the way.
-constexpr uint32_t kQ8SelEvenA = 0x0c030c02u, kQ8SelEvenB = 0x0c050c04u, kQ8SelOddA = 0x0c050c04u, kQ8SelOddB = 0x0c070c06u;
-MA_DEV void dequant4_shifted(uint32_t lo, uint32_t hi, uint32_t sel_a, uint32_t sel_b, h16x2 d2, uint32_t& out_lo, uint32_t& out_hi) {
-    const h16x2 bias = {(_Float16)1152.f, (_Float16)1152.f};
-    // selector 0x0c yields a zero byte; (q ^ 0x80) | 0x6400 in each half is one exclusive or
-    const h16x2 a = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(hi, lo, sel_a) ^ 0x64806480u);
-    const h16x2 b = __builtin_bit_cast(h16x2, __builtin_amdgcn_perm(hi, lo, sel_b) ^ 0x64806480u);
-    out_lo = __builtin_bit_cast(uint32_t, (a - bias) * d2);
-    out_hi = __builtin_bit_cast(uint32_t, (b - bias) * d2);
-}
-// the 8 fp16 values of quant words j, j+1 of such a block, given memory words w[j], w[j+1], w[j+2]
-MA_DEV s16x8 dequant8_shifted(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t sel_a, uint32_t sel_b, h16x2 d2) {
-    uint4 u;
-    dequant4_shifted(w0, w1, sel_a, sel_b, d2, u.x, u.y);
-    dequant4_shifted(w1, w2, sel_a, sel_b, d2, u.z, u.w);
-    return __builtin_bit_cast(s16x8, u);
+// The same from a block that is only 2-byte aligned, read as aligned words w0, w1, w2 of memory: quant word j of the
+// block is bytes 2..5 of {w[j+1], w[j]} when the block starts on a 4-byte boundary (kQ8SelEven) and w[j+1] itself when
+// it starts 2 bytes past one (kQ8SelOdd); one byte permute per word, its selector a per-lane constant, does the shift.
+constexpr uint32_t kQ8SelEven = 0x05040302u, kQ8SelOdd = 0x07060504u;
+MA_DEV s16x8 dequant8_shifted(uint32_t w0, uint32_t w1, uint32_t w2, uint32_t sel, h16x2 d2) {
+    return dequant8_words(__builtin_amdgcn_perm(w1, w0, sel), __builtin_amdgcn_perm(w2, w1, sel), d2);
 }
 
 // Quantises the lane's 8 values of a block whose 32 values are spread over the 4 lanes 4i..4i+3 (all four
