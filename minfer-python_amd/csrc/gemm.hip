@@ -30,14 +30,17 @@ namespace minfer_attn {
 
 constexpr int kBK = 64;
 // Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
-// 128 x 128 otherwise.  A wave owns 32*MB rows x 64 columns.
-template <int MB_, int WAVES_N_> struct GemmShape {
-    static constexpr int MB = MB_, WAVES_M = 2, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N;
-    static constexpr int BM = 32 * MB * WAVES_M, BN = 64 * WAVES_N;
+// 128 x 128 otherwise.  A wave owns 32*MB rows x 32*NB columns; OCC waves per SIMD.
+template <int MB_, int NB_, int WAVES_N_, int OCC_> struct GemmShape {
+    static constexpr int MB = MB_, NB = NB_, WAVES_M = 2, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N, OCC = OCC_;
+    static constexpr int BM = 32 * MB * WAVES_M, BN = 32 * NB * WAVES_N;
     static constexpr int A_PANEL = BM * 128, B_PANEL = BN * 128;   // bytes of one K step
+    static constexpr int A_COPIES = A_PANEL / 1024 / WAVES, B_COPIES = B_PANEL / 1024 / WAVES;   // wave-wide copies per wave
 };
-using GemmBig = GemmShape<4, 4>;
-using GemmSmall = GemmShape<2, 2>;
+// (4 waves with 128 x 128 each, GemmShape<4, 4, 2, 1>, read a third fewer LDS bytes per flop and run 3.2x slower: with
+// one wave per SIMD nothing covers a wave's waits for its fragments.)
+using GemmBig = GemmShape<4, 2, 4, 2>;
+using GemmSmall = GemmShape<2, 2, 2, 2>;
 constexpr int kRowTile = 8192;              // sub-tile [64 rows][64 k], 128-byte rows (A, and B as [N, K])
 constexpr int kColTile = 16384;             // sub-tile [64 k][128 n], 256-byte rows (B as [K, N])
 
@@ -54,8 +57,8 @@ MA_DEV int swz_row_tile(int row) { return (row >> 1) & 7; }        // 128-byte r
 MA_DEV int swz_col_tile(int row) { return (row & 3) << 2; }        // 256-byte rows, read 4 rows x 64 bytes (transposing)
 
 template <class T, bool NT, class SH>
-__global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParams p) {
-    constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB;
+__global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const GemmParams p) {
+    constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB, NB = SH::NB, CA = SH::A_COPIES, CB = SH::B_COPIES;
     __shared__ __attribute__((aligned(1024))) char a_lds[2][SH::A_PANEL];
     __shared__ __attribute__((aligned(1024))) char b_lds[2][SH::B_PANEL];
 
@@ -81,17 +84,19 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
     // Every wave issues 4 wave-wide copies (1 KB each) per panel and K step; copy q = j*NW + w of a panel covers
     //   A (and B as [N, K]): rows 8*(q%8) .. +7 of sub-tile q/8 (64 rows of 128 bytes each);
     //   B as [K, N]:         k rows 4*(q%16) .. +3 of sub-tile q/16 (64 k rows of 256 bytes, 128 columns).
-    uint32_t a_off[4], b_off[4];
-    int a_dst[4], b_dst[4];
+    uint32_t a_off[CA], b_off[CB];
+    int a_dst[CA], b_dst[CB];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
+    for (int j = 0; j < CA; ++j) {
         const int q = j * NW + w;
-        {
-            const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
-            const int m = min(m0 + 64 * sub + row, p.M - 1) - m0;
-            a_off[j] = (uint32_t)((int64_t)m * p.lda + 8 * (pg ^ swz_row_tile(row))) * 2u;
-            a_dst[j] = sub * kRowTile + 8 * (q & 7) * 128;
-        }
+        const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
+        const int m = min(m0 + 64 * sub + row, p.M - 1) - m0;
+        a_off[j] = (uint32_t)((int64_t)m * p.lda + 8 * (pg ^ swz_row_tile(row))) * 2u;
+        a_dst[j] = sub * kRowTile + 8 * (q & 7) * 128;
+    }
+#pragma unroll
+    for (int j = 0; j < CB; ++j) {
+        const int q = j * NW + w;
         if (NT) {
             const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
             const int n = min(n0 + 64 * sub + row, p.N - 1) - n0;
@@ -109,10 +114,9 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
         const short* abase = Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK;
         const short* bbase = NT ? Bg + (int64_t)n0 * p.ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * p.ldb + n0;
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            copy16_global_to_lds(abase, a_off[j], &a_lds[stage][a_dst[j]]);
-            copy16_global_to_lds(bbase, b_off[j], &b_lds[stage][b_dst[j]]);
-        }
+        for (int j = 0; j < CA; ++j) copy16_global_to_lds(abase, a_off[j], &a_lds[stage][a_dst[j]]);
+#pragma unroll
+        for (int j = 0; j < CB; ++j) copy16_global_to_lds(bbase, b_off[j], &b_lds[stage][b_dst[j]]);
     };
 
     // ---- per-lane LDS read addresses (stage 0; stage, sub-tile and block offsets are immediates) ---------
@@ -125,7 +129,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
         for (int kk = 0; kk < 4; ++kk) {
             const uint32_t o = l32 * 128 + 16 * ((2 * kk + h) ^ sw);
             m_rd[kk] = lds_addr(&a_lds[0][0]) + (MB / 2) * wm * kRowTile + o;
-            if (NT) n_rd[kk] = lds_addr(&b_lds[0][0]) + wn * kRowTile + o;    // n fragments: row 32*nb + l32 of sub-tile wn
+            if (NT) n_rd[kk] = lds_addr(&b_lds[0][0]) + (NB / 2) * wn * kRowTile + o;    // n fragments: as the m fragments
         }
         if (!NT) {
             // n fragments through transpose reads of the [k][n] sub-tile wn>>1: per 16-lane group 4 k rows x 16 columns
@@ -133,28 +137,27 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
             const int krow = 8 * h + (li >> 2);   // lane half h contracts k = 16kk + 8h + 0..7, like the 16-byte reads of A
             const int swv = swz_col_tile(krow);
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) {
-                const int col = 32 * (2 * (wn & 1) + nb) + 16 * (blk & 1) + 4 * (li & 3);
-                n_rd[nb] = lds_addr(&b_lds[0][0]) + (wn >> 1) * kColTile + krow * 256 + 16 * ((col >> 3) ^ swv) + 2 * (col & 7);
+            for (int nb = 0; nb < 4; ++nb) {
+                const int n = 32 * (NB * wn + (nb < NB ? nb : 0)), col = (n & 127) + 16 * (blk & 1) + 4 * (li & 3);
+                n_rd[nb] = lds_addr(&b_lds[0][0]) + (n >> 7) * kColTile + krow * 256 + 16 * ((col >> 3) ^ swv) + 2 * (col & 7);
             }
-            n_rd[2] = n_rd[3] = 0;
         }
     }
 
-    f32x16 acc[2][MB];
+    f32x16 acc[NB][MB];
 #pragma unroll
-    for (int nb = 0; nb < 2; ++nb)
+    for (int nb = 0; nb < NB; ++nb)
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.f;
 
-    auto load_frags = [&](auto stage_tag, int kk, s16x8 (&nf)[2], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
+    auto load_frags = [&](auto stage_tag, int kk, s16x8 (&nf)[NB], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
         constexpr int AOFF = decltype(stage_tag)::value * SH::A_PANEL, BOFF = decltype(stage_tag)::value * SH::B_PANEL;
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NB; ++nb) {
             if (NT) {
-                nf[nb] = lds_read_b128(n_rd[kk], BOFF + 32 * nb * 128);
+                nf[nb] = lds_read_b128(n_rd[kk], BOFF + (nb >> 1) * kRowTile + 32 * (nb & 1) * 128);
             } else {
                 const s16x4 t0 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk) * 256);
                 const s16x4 t1 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk + 4) * 256);
@@ -172,12 +175,12 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
     // stage just vacated and reads the next step's first fragments, all of which overlaps with the last slice's
     // MFMAs, so the matrix pipe does not drain at step boundaries.
     const int KT = p.K / kBK;
-    s16x8 nf[2][2], mf[2][MB];
+    s16x8 nf[2][NB], mf[2][MB];
     auto mfmas = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int nb = 0; nb < 2; ++nb) acc[nb][mb] = T::mfma32(nf[buf][nb], mf[buf][mb], acc[nb][mb]);
+            for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = T::mfma32(nf[buf][nb], mf[buf][mb], acc[nb][mb]);
     };
     auto step = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
         constexpr int STAGE = decltype(stage_tag)::value;
@@ -196,7 +199,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
     };
     issue(0, 0);
     if (KT > 1) issue(1, 1);
-    if (KT > 1) wait_vmcnt<8>(); else wait_vmcnt<0>();   // the 8 copies of step 0 retire first
+    if (KT > 1) wait_vmcnt<CA + CB>(); else wait_vmcnt<0>();   // the copies of step 0 retire first
     __syncthreads();
     load_frags(std::integral_constant<int, 0>{}, 0, nf[0], mf[0]);
     for (int kt = 0; kt < KT; kt += 2) {
@@ -212,10 +215,10 @@ __global__ __launch_bounds__(SH::WAVES * 64, 2) void gemm_kernel(const GemmParam
         const int m = m0 + 32 * MB * wm + 32 * mb + l32;
         if (m >= p.M) continue;
 #pragma unroll
-        for (int nb = 0; nb < 2; ++nb) {
+        for (int nb = 0; nb < NB; ++nb) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int n = n0 + 64 * wn + 32 * nb + 8 * j + 4 * h;
+                const int n = n0 + 32 * NB * wn + 32 * nb + 8 * j + 4 * h;
                 if (n >= p.N) continue;
                 float v[4];
 #pragma unroll
