@@ -182,6 +182,34 @@ def test_kv_append_llama_shape_then_decode_reads_it():
     assert float((out.float().cpu() - torch.from_numpy(want)).abs().max()) <= 2e-3
 
 
+def test_large_launches_equal_the_same_work_in_small_ones():
+    """A launch that touches more than the memory-side cache holds marks its loads and stores non-temporal; one
+    batch entry at a time stays below that.  Both must give the same bits: in place over whole heads, the producer
+    into fp16 caches and into Q8_0 caches."""
+    B, L = 8, 4096
+    x = workloads.rope_input(seed=5, device=DEV)                       # [8, 4096, 48, 128]
+    big = run_rope(NEOX, x, 128, 7, 5e5)
+    for b in range(B):
+        assert torch.equal(big[b:b + 1], run_rope(NEOX, x[b:b + 1].contiguous(), 128, 7, 5e5)), b
+    del big, x
+    q, k, v, pos, kc, vc = workloads.kv_append(seed=2, device=DEV, B=B, L=L, pos_hi=9)
+    q2, kc2, vc2 = run_append(NEOX, q, k, v, pos, kc, vc, 128, 5e5)
+    kq = torch.zeros(B, 8, kc.shape[2], 136, dtype=torch.uint8, device=DEV)
+    vq = torch.zeros_like(kq)
+    q3 = q.clone()
+    assert capi.rope_kv_append_q8_0(NEOX, q3, k, v, pos, kq, vq, 128, 5e5) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(q3, q2)
+    for b in range(B):
+        one = slice(b, b + 1)
+        qs, ks, vs = run_append(NEOX, q[one].contiguous(), k[one].contiguous(), v[one].contiguous(), pos[one], kc[one].contiguous(), vc[one].contiguous(), 128, 5e5)
+        assert torch.equal(q2[one], qs) and torch.equal(kc2[one], ks) and torch.equal(vc2[one], vs), b
+        kqs, vqs, qq = torch.zeros_like(kq[one]), torch.zeros_like(vq[one]), q[one].contiguous()
+        assert capi.rope_kv_append_q8_0(NEOX, qq, k[one].contiguous(), v[one].contiguous(), pos[one], kqs, vqs, 128, 5e5) == capi.OK
+        torch.cuda.synchronize()
+        assert torch.equal(kq[one], kqs) and torch.equal(vq[one], vqs), b
+
+
 def test_torch_ops_equal_c_abi_and_keep_the_reference_checks(kerns):
     g = torch.Generator().manual_seed(4)
     x = torch.randn(2, 50, 6, 128, generator=g).half().to(DEV)
