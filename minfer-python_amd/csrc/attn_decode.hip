@@ -133,32 +133,39 @@ struct SegmentWalk {
     // set by next():
     int pair, g0, g1, slot;  // (head group, KV head) pair, its groups [g0, g1), index of the partial result among the pair's
 
-    int wave;                // index of the wave in the launch
+    int wave;                // index of the wave's share of the line
+    // Shares are dealt to the waves of a workgroup in turn; when there are no more shares than workgroups (few or
+    // short sequences), every share goes to a workgroup of its own instead, so that as many compute units as
+    // possible pull on the memory system (B = 1 over 131072 rows: 107 -> 94 us, over 8192 rows: 19.4 -> 17.7 us).
+    MA_DEV void take_share(int total, int w) {
+        const int n_shares = (total + quota - 1) / quota;
+        wave = n_shares <= (int)gridDim.x ? w * (int)gridDim.x + (int)blockIdx.x : (int)blockIdx.x * kDecodeWaves + w;
+        x = wave * quota;
+        x_end = min(total, x + quota);
+    }
     MA_DEV bool start(const DecodeParams& p, int lane, int w) {
-        wave = (int)blockIdx.x * kDecodeWaves + w;
+        const bool first = blockIdx.x == 0 && w == 0;   // the wave that also stores the sequences' offsets
         int c;
         if (p.B <= 64) {   // one scan gives the line's length and the share's first sequence
             c = lane < p.B ? p.ctx[lane] : 0;
             const int n = lane < p.B ? groups_of(p, c) * p.Hkv * p.n_hg : 0;
             const int incl = wave_inclusive_scan(n, lane);
             const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
-            if (wave == 0) {
+            if (first) {
                 if (lane < p.B) p.seq_off[lane] = incl - n;
                 if (lane == 0) p.seq_off[p.B] = total;
             }
             quota = work_quota(p, total);
-            x = wave * quota;
-            x_end = min(total, x + quota);
+            take_share(total, w);
             if (x >= x_end) return false;
             const int src = __ffsll((unsigned long long)__ballot(x < incl)) - 1;
             b = __builtin_amdgcn_readfirstlane(src);
             off_b = __builtin_amdgcn_readfirstlane(__shfl(incl - n, src));
             c = __builtin_amdgcn_readfirstlane(__shfl(c, src));
         } else {
-            const int total = work_total(p, lane, wave == 0);
+            const int total = work_total(p, lane, first);
             quota = work_quota(p, total);
-            x = wave * quota;
-            x_end = min(total, x + quota);
+            take_share(total, w);
             if (x >= x_end) return false;
             locate_sequence(p, x, lane, b, off_b, c);
         }
