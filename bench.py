@@ -194,6 +194,31 @@ def main():
     d8_gbs = d8bytes / (d8_avg_ms * 1e-3) / 1e9
     del kq8, vq8
 
+    # ---- the two other prefill configurations: long context (bf16) and ragged packed sequences ----
+    lq, lk, lv, lmask = workloads.long_context_prefill(seed=0, device=dev)
+    lout = torch.empty_like(lq)
+    bt = GGMLQuantizationType.BF16
+    btb, bts = GGML_QUANT_SIZES[bt]
+    lstep = lambda: kerns.flash_attn(bt, btb, bts, lq, lk, lv, lmask, lout)
+    for _ in range(5):
+        lstep()
+    torch.cuda.synchronize()
+    l_avg_ms, l_med_ms = ev.time_each(lstep, stream, 10)
+    lflops = workloads.prefill_flops(32, 128, [lq.shape[2]])
+    l_tf = lflops / (l_avg_ms * 1e-3) / 1e12
+    del lq, lk, lv, lmask, lout
+    vq, vk, vv, vcu = workloads.ragged_prefill(seed=0, device=dev)
+    vlens = (vcu[1:] - vcu[:-1]).tolist()
+    vout = torch.empty_like(vq)
+    vstep = lambda: kerns.flash_attn_varlen(qt, qb, qs, vq, vk, vv, vcu, max(vlens), vout)
+    for _ in range(50):
+        vstep()
+    torch.cuda.synchronize()
+    v_avg_ms, v_med_ms = ev.time_each(vstep, stream, 50)
+    vflops = workloads.prefill_flops(64, 128, vlens)
+    v_tf = vflops / (v_avg_ms * 1e-3) / 1e12
+    del vq, vk, vv, vout
+
     # ---- the step before attention: rotary embedding, alone and fused with the cache append ----
     x = workloads.rope_input(seed=0, device=dev)                      # the reference test's shape
     rstep = lambda: kerns.il_rope(64, 2048, 1e6, x)
@@ -271,6 +296,14 @@ def main():
                                        "frac": d8_gbs / PEAK_HBM_GBS, "traffic": DECODE_Q8_TRAFFIC_BYTES,
                                        "kernel": "decode_split_q8_kernel<128> + decode_combine_kernel",
                                        "algorithmic_bytes": d8bytes}}
+    rec["long_context"] = {"value": l_tf, "unit": "TFLOP/s", "ms": l_avg_ms, "median_ms": l_med_ms,
+                           "workload": "prefill B=1 Hq=32 Hkv=8 S=32768 D=128 bf16 causal dense-mask, mask 1 GiB (BASELINE configs[3])",
+                           "roofline": {"bound": "mfma", "achieved": l_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": l_tf / PEAK_MFMA_TFLOPS,
+                                        "traffic": None, "kernel": "classify_mask_kernel + prefill_kernel<BF16,128,dense>", "algorithmic_flops": lflops}}
+    rec["ragged"] = {"value": v_tf, "unit": "TFLOP/s", "ms": v_avg_ms, "median_ms": v_med_ms,
+                     "workload": f"packed prefill of 16 sequences, lengths U[128,2048] (T={sum(vlens)}), Hq=64 Hkv=8 D=128 fp16, causal within a sequence (BASELINE configs[4])",
+                     "roofline": {"bound": "mfma", "achieved": v_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": v_tf / PEAK_MFMA_TFLOPS,
+                                  "traffic": None, "kernel": "prefill_kernel<F16,128,varlen>", "algorithmic_flops": vflops}}
     rec["rope_kv_append_q8_0"] = {"value": a8_gbs, "unit": "GB/s", "ms": a8_avg_ms, "median_ms": a8_med_ms,
                                   "workload": "the rope_kv_append workload into Q8_0 caches, uint8 [8,8,4096,136]",
                                   "roofline": {"bound": "hbm", "achieved": a8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a8_gbs / PEAK_HBM_GBS,
