@@ -166,6 +166,16 @@ MA_DEV float sum_across_halves(float x) {
 
 MA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
 
+// Inclusive prefix sum of x over the lanes of a wave.
+MA_DEV int wave_inclusive_scan(int x, int lane) {
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const int up = __shfl_up(x, d);
+        if (lane >= d) x += up;
+    }
+    return x;
+}
+
 // Loads and stores of bytes that a kernel touches once (cache rows being streamed, rows of a normalisation):
 // marked non-temporal, so that the caches between the compute units and HBM do not keep the lines.  On this chip
 // that alone raises the HBM throughput of a streaming kernel by 10-15 %.

@@ -72,15 +72,6 @@ struct DecodeParams {
 // end together; a piece of one pair inside one wave's share is a segment, and yields one partial result.
 MA_DEV int groups_of(const DecodeParams& p, int ctx) { return (min(max(ctx, 0), p.Lmax) + p.group_rows - 1) / p.group_rows; }
 
-MA_DEV int wave_inclusive_scan(int x, int lane) {
-#pragma unroll
-    for (int d = 1; d < 64; d <<= 1) {
-        const int up = __shfl_up(x, d);
-        if (lane >= d) x += up;
-    }
-    return x;
-}
-
 // Length of the line (every lane gets it).  With `publish`, also stores every sequence's start on the line and,
 // at index B, the length.
 MA_DEV int work_total(const DecodeParams& p, int lane, bool publish) {

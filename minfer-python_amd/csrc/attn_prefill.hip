@@ -169,15 +169,29 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     if (MODE == MODE_DENSE) {
         qtile = p.NQ - 1 - rank;    // longest rows of a causal mask first
     } else {
-        int x = rank, s = 0, nt = 0;
-        for (; s < p.n_seqs; ++s) {
-            seq_lo = p.cu[s];
-            seq_len = p.cu[s + 1] - seq_lo;
-            nt = (seq_len + 32 * QBW - 1) / (32 * QBW);
-            if (x < nt) break;
-            x -= nt;
+        // the sequence that holds query tile `rank` of the packed batch: 64 sequences per step, a prefix sum of their
+        // tile counts over the lanes (one sequence per step cost a workgroup ~40 ns per sequence before its tile)
+        int x = rank, nt = 0;
+        bool found = false;
+        for (int base = 0; base < p.n_seqs && !found; base += 64) {
+            const int sq = base + lane;
+            const int lo = sq < p.n_seqs ? p.cu[sq] : 0;
+            const int len = sq < p.n_seqs ? p.cu[sq + 1] - lo : 0;
+            const int n = (len + 32 * QBW - 1) / (32 * QBW);
+            const int incl = wave_inclusive_scan(n, lane);
+            const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
+            if (x < total) {
+                const int src = __ffsll((unsigned long long)__ballot(x < incl)) - 1;
+                seq_lo = __builtin_amdgcn_readfirstlane(__shfl(lo, src));
+                seq_len = __builtin_amdgcn_readfirstlane(__shfl(len, src));
+                nt = __builtin_amdgcn_readfirstlane(__shfl(n, src));
+                x -= __builtin_amdgcn_readfirstlane(__shfl(incl - n, src));
+                found = true;
+            } else {
+                x -= total;
+            }
         }
-        if (s >= p.n_seqs) return;
+        if (!found) return;
         qtile = nt - 1 - x;
     }
 

@@ -328,6 +328,7 @@ def test_decode_equals_last_prefill_row():
     (8, 1, 64, [130, 31, 0, 77]),
     (6, 2, 128, [1, 1, 1]),
     (4, 4, 64, [300]),
+    (8, 2, 128, [(7 * i) % 41 for i in range(150)]),      # more sequences than a wave has lanes, some empty
 ])
 def test_varlen_matches_oracle_and_dense(dtype, Hq, Hkv, D, lens):
     g = torch.Generator().manual_seed(sum(lens))
@@ -345,7 +346,9 @@ def test_varlen_matches_oracle_and_dense(dtype, Hq, Hkv, D, lens):
     for lo, hi in zip(cu[:-1].tolist(), cu[1:].tolist()):
         blk[lo:hi, lo:hi] = torch.ones(hi - lo, hi - lo, dtype=torch.bool).tril()
     dense = run_prefill(q.to(DEV), k.to(DEV), v.to(DEV), blk[None, None].contiguous().to(DEV))
-    assert max_err(out, dense) <= TOL[dtype] / 2
+    # (two bf16 results may round an element above 1 to neighbouring values, 2^-7 apart)
+    one_ulp = float(dense.float().abs().max()) * 2.0 ** -8 if dtype == torch.bfloat16 else 0.0
+    assert max_err(out, dense) <= TOL[dtype] / 2 + one_ulp
 
 
 # ------------------------------------------------------------------------------------------------
