@@ -237,6 +237,76 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     }
 }
 
+// Few rows of A (the tokens of a decode step) against a weight stored [N, K]: the work is reading the weight once.
+// A workgroup owns 16 columns n of D and all K; its 8 waves split K, each streaming its slice of the 16 weight rows
+// (non-temporal 32-byte pieces per lane, four lanes covering one 128-byte line of a row) into the A operand of
+// v_mfma_f32_16x16x32, the rows of A (from L2) being the B operand, 16 at a time; the waves' partial sums meet in LDS.
+// Within a 64-wide K step lane (row, quad) takes k = 16*quad + 0..15 for both operands, which is just another order
+// of the contraction.  MB = ceil(M / 16) <= 4.
+constexpr int kSkinnyWaves = 8;
+template <class T, int MB>
+__global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const GemmParams p) {
+    __shared__ f32x4 part[kSkinnyWaves][MB][64];
+    const int lane = threadIdx.x & 63, w = wave_id();
+    const int l16 = lane & 15, quad = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16;
+    const int steps = p.K / 64, per = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
+    const int s0 = w * per, s1 = min(steps, s0 + per);
+    const short* wrow = (const short*)p.B + (int64_t)min(n0 + l16, p.N - 1) * p.ldb + 16 * quad;
+    const short* xrow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xrow[mb] = (const short*)p.A + (int64_t)min(16 * mb + l16, p.M - 1) * p.lda + 16 * quad;
+    f32x4 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
+    for (int s = s0; s < s1; ++s) {
+        const int k0 = 64 * s;
+        const s16x8 w0 = stream_load(reinterpret_cast<const s16x8*>(wrow + k0));
+        const s16x8 w1 = stream_load(reinterpret_cast<const s16x8*>(wrow + k0 + 8));
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) {
+            const s16x8 x0 = *reinterpret_cast<const s16x8*>(xrow[mb] + k0);
+            const s16x8 x1 = *reinterpret_cast<const s16x8*>(xrow[mb] + k0 + 8);
+            acc[mb] = T::mfma16(w0, x0, acc[mb]);
+            acc[mb] = T::mfma16(w1, x1, acc[mb]);
+        }
+    }
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) part[w][mb][lane] = acc[mb];
+    __syncthreads();
+    if (w >= MB) return;
+    // wave mb adds up block mb: register r of a lane is n = n0 + 4*quad + r, m = 16*mb + l16
+    f32x4 sum = part[0][w][lane];
+#pragma unroll
+    for (int ww = 1; ww < kSkinnyWaves; ++ww) sum += part[ww][w][lane];
+    const int m = 16 * w + l16, n = n0 + 4 * quad;
+    if (m >= p.M || n >= p.N) return;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
+    if (p.beta != 0.f) {
+        const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+    }
+    uint2 pk;
+    pk.x = T::pack2(v[0], v[1]);
+    pk.y = T::pack2(v[2], v[3]);
+    *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+}
+
+template <class T>
+static int launch_skinny(const GemmParams& p, hipStream_t stream) {
+    const dim3 grid((p.N + 15) / 16), block(kSkinnyWaves * 64);
+    const int mb = (p.M + 15) / 16;
+    if (mb == 1) hipLaunchKernelGGL((gemm_skinny_kernel<T, 1>), grid, block, 0, stream, p);
+    else if (mb == 2) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2>), grid, block, 0, stream, p);
+    else if (mb == 3) hipLaunchKernelGGL((gemm_skinny_kernel<T, 3>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_skinny_kernel<T, 4>), grid, block, 0, stream, p);
+    return check_launch("gemm_skinny_kernel");
+}
+
 // Any shape and alignment: one thread per element of D, fp32 accumulation.  Small or odd problems only.
 template <class T, bool NT>
 __global__ __launch_bounds__(256) void gemm_plain_kernel(const GemmParams p) {
@@ -301,6 +371,11 @@ MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const
                       aligned16(A) && aligned16(B) && ((uintptr_t)D & 7u) == 0 && ((uintptr_t)C & 7u) == 0 &&
                       (int64_t)GemmBig::BM * lda < (1LL << 30) && (int64_t)std::max<int64_t>(GemmBig::BN, kBK) * ldb < (1LL << 30);
     hipStream_t stream = (hipStream_t)stream_v;
+    // a decode step's few tokens against an [N, K] weight: stream the weight once
+    // (up to 32 rows it beats the tiled kernel at every weight size measured, 7-34 us against 40-133 us; with 33-64 rows,
+    // whose fragments are re-read from L2 for every 16 columns, only while the weight is small)
+    if (fast && nt && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))
+        return dtype == MINFER_ATTN_F16 ? launch_skinny<F16>(p, stream) : launch_skinny<BF16>(p, stream);
     if (dtype == MINFER_ATTN_F16) return nt ? launch_gemm<F16, true>(p, fast, stream) : launch_gemm<F16, false>(p, fast, stream);
     return nt ? launch_gemm<BF16, true>(p, fast, stream) : launch_gemm<BF16, false>(p, fast, stream);
 }

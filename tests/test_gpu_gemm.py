@@ -53,10 +53,15 @@ def make(M, N, K, layout, dtype, seed):
     (3000, 4104, 64, 2.0, 0.0),      # the same with ragged edges
     (33, 17, 50, 1.0, 1.0),          # nothing tileable: plain kernel
     (64, 64, 72, 1.0, 0.0),          # K not a multiple of 64: plain kernel
+    (8, 4096, 4096, 1.0, 0.0),       # a decode step's tokens: with an [N, K] weight, the kernel that streams it once
+    (64, 1024, 1792, 2.0, 3.0),      # its largest row count; K steps not a multiple of the eight waves
+    (48, 8192, 8192, 1.0, 0.0),      # more than 32 rows against a large weight: the tiled kernel again
+    (37, 24, 192, 0.5, 1.0),         # ragged rows, a last group of 16 columns that is half empty
+    (17, 4104, 64, 1.0, 1.0),        # one K step: seven of the eight waves have nothing to add
 ])
 def test_gemm_matches_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, M + N + K)
-    if M * N * K <= 1 << 26:
+    if M * N * K <= 1 << 26 or M <= 64:
         exact = oracle.gemm(a, b, c, alpha, beta, layout)
         rows = slice(None)
     else:       # the oracle is a scalar CPU program: a sample of rows at this size
