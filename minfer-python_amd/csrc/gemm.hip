@@ -244,43 +244,58 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 // Within a 64-wide K step lane (row, quad) takes k = 16*quad + 0..15 for both operands, which is just another order
 // of the contraction.  MB = ceil(M / 16) <= 4.
 constexpr int kSkinnyWaves = 8;
-template <class T, int MB>
+// NR groups of 16 columns per workgroup (2 for wide weights: half as many workgroups, each A fragment used twice)
+template <class T, int MB, int NR>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const GemmParams p) {
-    __shared__ f32x4 part[kSkinnyWaves][MB][64];
+    __shared__ f32x4 part[kSkinnyWaves][NR][MB][64];
     const int lane = threadIdx.x & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    const int n0 = (int)blockIdx.x * 16;
+    const int n0 = (int)blockIdx.x * 16 * NR;
     const int steps = p.K / 64, per = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
     const int s0 = w * per, s1 = min(steps, s0 + per);
-    const short* wrow = (const short*)p.B + (int64_t)min(n0 + l16, p.N - 1) * p.ldb + 16 * quad;
+    const short* wrow[NR];
+#pragma unroll
+    for (int nr = 0; nr < NR; ++nr) wrow[nr] = (const short*)p.B + (int64_t)min(n0 + 16 * nr + l16, p.N - 1) * p.ldb + 16 * quad;
     const short* xrow[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) xrow[mb] = (const short*)p.A + (int64_t)min(16 * mb + l16, p.M - 1) * p.lda + 16 * quad;
-    f32x4 acc[MB];
+    f32x4 acc[NR][MB];
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    for (int nr = 0; nr < NR; ++nr)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nr][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll 4
     for (int s = s0; s < s1; ++s) {
         const int k0 = 64 * s;
-        const s16x8 w0 = stream_load(reinterpret_cast<const s16x8*>(wrow + k0));
-        const s16x8 w1 = stream_load(reinterpret_cast<const s16x8*>(wrow + k0 + 8));
+        s16x8 w0[NR], w1[NR];
+#pragma unroll
+        for (int nr = 0; nr < NR; ++nr) {
+            w0[nr] = stream_load(reinterpret_cast<const s16x8*>(wrow[nr] + k0));
+            w1[nr] = stream_load(reinterpret_cast<const s16x8*>(wrow[nr] + k0 + 8));
+        }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb) {
             const s16x8 x0 = *reinterpret_cast<const s16x8*>(xrow[mb] + k0);
             const s16x8 x1 = *reinterpret_cast<const s16x8*>(xrow[mb] + k0 + 8);
-            acc[mb] = T::mfma16(w0, x0, acc[mb]);
-            acc[mb] = T::mfma16(w1, x1, acc[mb]);
+#pragma unroll
+            for (int nr = 0; nr < NR; ++nr) {
+                acc[nr][mb] = T::mfma16(w0[nr], x0, acc[nr][mb]);
+                acc[nr][mb] = T::mfma16(w1[nr], x1, acc[nr][mb]);
+            }
         }
     }
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) part[w][mb][lane] = acc[mb];
-    __syncthreads();
-    if (w >= MB) return;
-    // wave mb adds up block mb: register r of a lane is n = n0 + 4*quad + r, m = 16*mb + l16
-    f32x4 sum = part[0][w][lane];
+    for (int nr = 0; nr < NR; ++nr)
 #pragma unroll
-    for (int ww = 1; ww < kSkinnyWaves; ++ww) sum += part[ww][w][lane];
-    const int m = 16 * w + l16, n = n0 + 4 * quad;
+        for (int mb = 0; mb < MB; ++mb) part[w][nr][mb][lane] = acc[nr][mb];
+    __syncthreads();
+    // wave j adds up block (nr, mb) = (j / MB, j % MB): register r of a lane is n = n0 + 16*nr + 4*quad + r, m = 16*mb + l16
+    if (w >= NR * MB) return;
+    const int nr = w / MB, mb = w - nr * MB;
+    f32x4 sum = part[0][nr][mb][lane];
+#pragma unroll
+    for (int ww = 1; ww < kSkinnyWaves; ++ww) sum += part[ww][nr][mb][lane];
+    const int m = 16 * mb + l16, n = n0 + 16 * nr + 4 * quad;
     if (m >= p.M || n >= p.N) return;
     float v[4];
 #pragma unroll
@@ -296,14 +311,21 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const Ge
     *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
 }
 
+template <class T, int NR>
+static void launch_skinny_nr(const GemmParams& p, hipStream_t stream) {
+    const dim3 grid((p.N + 16 * NR - 1) / (16 * NR)), block(kSkinnyWaves * 64);
+    const int mb = (p.M + 15) / 16;
+    if (mb == 1) hipLaunchKernelGGL((gemm_skinny_kernel<T, 1, NR>), grid, block, 0, stream, p);
+    else if (mb == 2) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2, NR>), grid, block, 0, stream, p);
+    else if (mb == 3) hipLaunchKernelGGL((gemm_skinny_kernel<T, 3, NR>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_skinny_kernel<T, 4, NR>), grid, block, 0, stream, p);
+}
 template <class T>
 static int launch_skinny(const GemmParams& p, hipStream_t stream) {
-    const dim3 grid((p.N + 15) / 16), block(kSkinnyWaves * 64);
-    const int mb = (p.M + 15) / 16;
-    if (mb == 1) hipLaunchKernelGGL((gemm_skinny_kernel<T, 1>), grid, block, 0, stream, p);
-    else if (mb == 2) hipLaunchKernelGGL((gemm_skinny_kernel<T, 2>), grid, block, 0, stream, p);
-    else if (mb == 3) hipLaunchKernelGGL((gemm_skinny_kernel<T, 3>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((gemm_skinny_kernel<T, 4>), grid, block, 0, stream, p);
+    // two column groups per workgroup once that still leaves 160 workgroups and there is more than one block of rows
+    // to share between them (32 rows x 14336 columns: 52 -> 40 us; 64 x 6144: 38 -> 27; a single block of rows loses 5-10 %)
+    if (p.M > 16 && p.N >= 160 * 32) launch_skinny_nr<T, 2>(p, stream);
+    else launch_skinny_nr<T, 1>(p, stream);
     return check_launch("gemm_skinny_kernel");
 }
 

@@ -56,6 +56,7 @@ def make(M, N, K, layout, dtype, seed):
     (8, 4096, 4096, 1.0, 0.0),       # a decode step's tokens: with an [N, K] weight, the kernel that streams it once
     (64, 1024, 1792, 2.0, 3.0),      # its largest row count; K steps not a multiple of the eight waves
     (48, 8192, 8192, 1.0, 0.0),      # more than 32 rows against a large weight: the tiled kernel again
+    (30, 5200, 128, 2.0, 1.0),       # wide enough for two column groups per workgroup, the last one ragged
     (37, 24, 192, 0.5, 1.0),         # ragged rows, a last group of 16 columns that is half empty
     (17, 4104, 64, 1.0, 1.0),        # one K step: seven of the eight waves have nothing to add
 ])
