@@ -17,14 +17,17 @@ import time
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 PKG = os.path.join(ROOT, "minfer-python_amd")
-for p in (ROOT, PKG, os.path.join(PKG, "apps")):
+for p in (ROOT, PKG):
     if p not in sys.path:
         sys.path.insert(0, p)
+sys.path.append(os.path.join(PKG, "apps"))   # last: its profile.py must not shadow the standard library's
 
 PEAK_MFMA_TFLOPS = 2500.0   # MI355X dense fp16/bf16
 PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # HBM bytes per launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (each scaled by what the
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
+# These are figures from those earlier counter runs, not measured in the run that prints them.
+TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels_pmc.md (rocprofv3 --pmc runs of the same workloads; not re-measured by this run)"
 PREFILL_TRAFFIC_BYTES = 107374 * 1024
 DECODE_TRAFFIC_BYTES = 1092838 * 1024
 ROPE_TRAFFIC_BYTES = 393312 * 1024          # il_rope on [8,4096,48,128], rotary 64
@@ -51,6 +54,19 @@ class HipEvents:
         e = ctypes.c_void_p()
         assert self.hip.hipEventCreate(ctypes.byref(e)) == 0
         return e
+
+    def time_region(self, fn, stream, n):
+        """Average duration (ms) of n back-to-back calls of fn bracketed by ONE pair of events on `stream`: what the
+        GPU needs per call when calls follow each other, launch gaps included, no host clock involved."""
+        a, b = self.event(), self.event()
+        assert self.hip.hipEventRecord(a, stream) == 0
+        for _ in range(n):
+            fn()
+        assert self.hip.hipEventRecord(b, stream) == 0
+        assert self.hip.hipEventSynchronize(b) == 0
+        t = ctypes.c_float()
+        assert self.hip.hipEventElapsedTime(ctypes.byref(t), a, b) == 0
+        return t.value / n
 
     def time_each(self, fn, stream, n):
         """Average and median duration (ms) of n calls of fn, each bracketed by events on `stream`."""
@@ -107,7 +123,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=500)
     ap.add_argument("--warmup", type=int, default=300,
-                    help="untimed steps; the GPU needs some 15 ms of continuous work after an idle period to reach its clocks")
+                    help="untimed steps right before the timed ones (a time-based pre-warm of the clocks runs before them in any case)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--graph", action="store_true", help="replay one captured HIP graph per step instead of launching from Python")
     args = ap.parse_args()
@@ -157,15 +173,35 @@ def main():
         step()
         torch.cuda.synchronize()
         assert torch.equal(out, ref_out), "graph replay differs from the eager result"
+    # The chip needs some 15 ms of continuous work after an idle period to reach its clocks (a loop started cold
+    # averages 174 us per call instead of 146): whatever --warmup says, the step first runs back to back until
+    # PREWARM_MS of GPU time have passed, so that a short run (--warmup 5 --steps 20) measures the same steady
+    # state as a long one.
+    PREWARM_MS = 100.0
+    prewarm_ms, prewarm_calls = 0.0, 0
+    while prewarm_ms < PREWARM_MS:
+        prewarm_ms += ev.time_region(step, stream, 50) * 50
+        prewarm_calls += 50
     for _ in range(args.warmup):
         step()
+    # the timed region: exactly --steps steps, by the host clock between two synchronisations and, over the same
+    # steps, by one pair of events on the launch stream
+    t_a, t_b = ev.event(), ev.event()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
+    assert ev.hip.hipEventRecord(t_a, stream) == 0
     for _ in range(args.steps):
         step()
+    assert ev.hip.hipEventRecord(t_b, stream) == 0
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    avg_ms, med_ms = ev.time_each(step, stream, min(max(args.steps, 20), 200))
+    t_el = ctypes.c_float()
+    assert ev.hip.hipEventElapsedTime(ctypes.byref(t_el), t_a, t_b) == 0
+    region_ms = t_el.value / args.steps
+    # a region of at least 200 steps for the roofline figure when --steps is smaller (the same region otherwise)
+    event_steps = max(args.steps, 200)
+    avg_ms = region_ms if event_steps == args.steps else ev.time_region(step, stream, event_steps)
+    _, med_ms = ev.time_each(step, stream, min(event_steps, 200))
     flops = workloads.prefill_flops(32, 128, [L])
     tflops = flops / (wall_ms * 1e-3) / 1e12
     achieved = flops / (avg_ms * 1e-3) / 1e12
@@ -274,18 +310,19 @@ def main():
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": wall_ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "ms_per_step": wall_ms, "event_ms_per_step": region_ms, "event_steps": event_steps,
+        "prewarm_ms": prewarm_ms, "prewarm_calls": prewarm_calls, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic", "launch": "hipgraph replay of one op call" if args.graph else "eager",
         "config": {"workload": "prefill B=1 Hq=32 Hkv=8 S=4096 D=128 fp16 causal dense-mask (BASELINE configs[1])",
                    "global_batch": 1, "seq_len": L, "parallelism": "single-gpu"},
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_MFMA_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES,
+                     "frac": achieved / PEAK_MFMA_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                      "kernel": "classify_mask_kernel + prefill_kernel<F16,128,dense>",
                      "algorithmic_flops": flops, "avg_ms": avg_ms, "median_ms": med_ms},
         "decode": {"value": d_gbs, "unit": "GB/s", "ms": d_avg_ms, "median_ms": d_med_ms,
                    "workload": "decode B=64 Hq=32 Hkv=8 D=128 fp16 ctx~U[512,8192] cache [64,8,8192,128] (BASELINE configs[2])",
                    "roofline": {"bound": "hbm", "achieved": d_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                "frac": d_gbs / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES,
+                                "frac": d_gbs / PEAK_HBM_GBS, "traffic": DECODE_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                                 "kernel": "decode_split_kernel<F16,128> + decode_combine_kernel",
                                 "algorithmic_bytes": dbytes}},
     }
@@ -293,7 +330,7 @@ def main():
                           "speedup_over_fp16_cache": d_avg_ms / d8_avg_ms,
                           "workload": "the decode workload over Q8_0 caches, uint8 [64,8,8192,136] (34-byte blocks of 32 values), q/out fp16",
                           "roofline": {"bound": "hbm", "achieved": d8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
-                                       "frac": d8_gbs / PEAK_HBM_GBS, "traffic": DECODE_Q8_TRAFFIC_BYTES,
+                                       "frac": d8_gbs / PEAK_HBM_GBS, "traffic": DECODE_Q8_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
                                        "kernel": "decode_split_q8_kernel<128> + decode_combine_kernel",
                                        "algorithmic_bytes": d8bytes}}
     rec["long_context"] = {"value": l_tf, "unit": "TFLOP/s", "ms": l_avg_ms, "median_ms": l_med_ms,
@@ -307,24 +344,24 @@ def main():
     rec["rope_kv_append_q8_0"] = {"value": a8_gbs, "unit": "GB/s", "ms": a8_avg_ms, "median_ms": a8_med_ms,
                                   "workload": "the rope_kv_append workload into Q8_0 caches, uint8 [8,8,4096,136]",
                                   "roofline": {"bound": "hbm", "achieved": a8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a8_gbs / PEAK_HBM_GBS,
-                                               "traffic": APPEND_Q8_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,neox,fused append,Q8_0>", "algorithmic_bytes": a8bytes}}
+                                               "traffic": APPEND_Q8_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rope_kernel<F16,neox,fused append,Q8_0>", "algorithmic_bytes": a8bytes}}
     rec["rope"] = {"value": r_gbs, "unit": "GB/s", "ms": r_avg_ms, "median_ms": r_med_ms,
                    "workload": "il_rope in place, x [8,4096,48,128] fp16, rotary_dim 64, base 1e6, start_pos 2048 (reference test/kernels.py:76-96)",
                    "roofline": {"bound": "hbm", "achieved": r_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": r_gbs / PEAK_HBM_GBS,
-                                "traffic": ROPE_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,interleaved,in place>", "algorithmic_bytes": rbytes}}
+                                "traffic": ROPE_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rope_kernel<F16,interleaved,in place>", "algorithmic_bytes": rbytes}}
     rec["rope_kv_append"] = {"value": a_gbs, "unit": "GB/s", "ms": a_avg_ms, "median_ms": a_med_ms,
                              "workload": "NeoX rope(q) in place + rope(k), v appended to the cache: B=8 L=4096 Hq=32 Hkv=8 D=128 fp16, rotary_dim 128, base 5e5",
                              "roofline": {"bound": "hbm", "achieved": a_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a_gbs / PEAK_HBM_GBS,
-                                          "traffic": APPEND_TRAFFIC_BYTES, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
+                                          "traffic": APPEND_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,
-                                   "traffic": NORM_TRAFFIC_BYTES, "kernel": "rmsnorm_rows_kernel<F16,64,12,streamed>", "algorithmic_bytes": nbytes}}
+                                   "traffic": NORM_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rmsnorm_rows_kernel<F16,64,12,streamed>", "algorithmic_bytes": nbytes}}
     rec["gemm"] = {"value": g_tf, "unit": "TFLOP/s", "ms": g_avg_ms, "median_ms": g_med_ms,
                    "workload": "gemm alpha=1 beta=0, A [1,4096,4096] x W [4096,4096] fp16 (reference README HGEMM table, M=K=N=4096)",
                    "published_reference_us": 605.3,
                    "roofline": {"bound": "mfma", "achieved": g_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": g_tf / PEAK_MFMA_TFLOPS,
-                                "traffic": GEMM_TRAFFIC_BYTES, "kernel": "gemm_kernel<F16,[K,N],256x256>", "algorithmic_flops": gflops}}
+                                "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_kernel<F16,[K,N],256x256>", "algorithmic_flops": gflops}}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
         rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)

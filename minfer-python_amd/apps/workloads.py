@@ -52,6 +52,30 @@ def llama8b_prefill(seed=0, device="cpu", views=False, L=4096):
     return q, k, v, causal_mask(1, L, device=device)
 
 
+def reference_test_prefill(seed=0, device="cpu", B=8, L=4096, Hq=48, Hkv=8, D=128, window=None):
+    """The reference test's recipe (reference: test/kernels.py:225-244, 263-280): q ~ N(0,1), k and v ~ N(0,1)/sqrt(D),
+    drawn as [B,L,H*D] fp16 and handed over as transposed [B,H,L,D] views; mask causal (case A) or, with
+    ``window`` (256 there, case B), |i - j| < window."""
+    gen = torch.Generator().manual_seed(seed)
+    q = _qkv(gen, B, Hq, L, D, 1.0, torch.float16, True)
+    k = _qkv(gen, B, Hkv, L, D, D ** -0.5, torch.float16, True)
+    v = _qkv(gen, B, Hkv, L, D, D ** -0.5, torch.float16, True)
+    if device != "cpu":
+        q, k, v = (t.transpose(1, 2).to(device).transpose(1, 2) for t in (q, k, v))
+    mask = causal_mask(B, L, device=device) if window is None else window_mask(B, L, window, device=device)
+    return q, k, v, mask
+
+
+def reference_benchmark_prefill(seed=0, device="cpu", B=4, L=16384, Hq=48, Hkv=8, D=128):
+    """The reference benchmark's recipe (reference: apps/benchmark.py:215-237; L in 4096, 8192, 16384): q, k, v all
+    ~ N(0,1)/sqrt(D) as transposed views, causal mask."""
+    gen = torch.Generator().manual_seed(seed)
+    q, k, v = (_qkv(gen, B, H, L, D, D ** -0.5, torch.float16, True) for H in (Hq, Hkv, Hkv))
+    if device != "cpu":
+        q, k, v = (t.transpose(1, 2).to(device).transpose(1, 2) for t in (q, k, v))
+    return q, k, v, causal_mask(B, L, device=device)
+
+
 def long_context_prefill(seed=0, device="cpu", L=32768):
     """B=1, Hq=32, Hkv=8, S=32768, D=128, bf16, 0.5*N(0,1), causal."""
     q, k, v = dense_prefill(1, 32, 8, L, 128, torch.bfloat16, seed=seed, scale=0.5, device=device)

@@ -107,7 +107,7 @@ MA_DEV void copy16_global_to_lds(const void* src, void* lds_base) {
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                  :
                  : "s"(dst), "v"(src)
-                 : "memory");
+                 : "memory", "m0");
 }
 // Same, with the source given as a wave-uniform base plus a 32-bit unsigned per-lane byte offset, which
 // costs no vector ALU work when the offset is loop-invariant.
@@ -121,7 +121,7 @@ MA_DEV void copy16_global_to_lds(const void* uniform_base, uint32_t lane_byte_of
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
                  :
                  : "s"(dst), "v"(lane_byte_offset), "s"(sb)
-                 : "memory");
+                 : "memory", "m0");
 }
 
 // 32-bit LDS address of a __shared__ object, and reads at such an address plus a compile-time offset

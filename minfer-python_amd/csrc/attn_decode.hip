@@ -30,25 +30,19 @@
 // (reference: cuda/quants/impls.cuh:121-143).  K needs no further LDS pass: lane (key, quad) holds values
 // D/4 * quad .. of its key, which is a valid MFMA contraction order as long as Q^T is loaded in the same
 // order.  V is parked as fp16 rows and read back transposed, as on the fp16 path.
+#include <atomic>
+
 #include "attn_common.h"
 #include "attn_host.h"
 #include "quant_q8.h"
 
 namespace minfer_attn {
 
-// Tunables (overridable at compile time for sweeps).
-#ifndef MINFER_DECODE_WAVES
-#define MINFER_DECODE_WAVES 4
-#endif
-#ifndef MINFER_DECODE_STAGES
-#define MINFER_DECODE_STAGES 3
-#endif
-#ifndef MINFER_DECODE_MIN_WAVES_PER_SIMD
-#define MINFER_DECODE_MIN_WAVES_PER_SIMD 2
-#endif
-constexpr int kDecodeWaves = MINFER_DECODE_WAVES;
-constexpr int kGroupRows = 16;   // cache rows per ring slot of one wave
-constexpr int kDecodeStages = MINFER_DECODE_STAGES; // ring depth
+constexpr int kDecodeWaves = 4;         // waves per workgroup
+constexpr int kDecodeWavesPerSimd = 2;  // resident waves per SIMD the register budget is set for
+constexpr int kDecodeWgPerCu = 2;       // workgroups of the split launch per compute unit
+constexpr int kGroupRows = 16;          // cache rows per ring slot of one wave
+constexpr int kDecodeStages = 3;        // ring depth
 
 struct DecodeParams {
     const void* q; const void* k; const void* v;
@@ -197,7 +191,7 @@ template <int D> struct DecodeGeom {
 };
 
 template <class T, int D>
-__global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD) void decode_split_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode_split_kernel(const DecodeParams p) {
     using GEO = DecodeGeom<D>;
     constexpr int RB = GEO::RB, G = GEO::G, RPI = GEO::RPI, NI = GEO::NI;
     constexpr int KC = D / 32;   // 32-wide contraction chunks of K Q^T
@@ -218,8 +212,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     const int row_lo = walk.g0 * kGroupRows;
     const int row_hi = min(walk.g1 * kGroupRows, ctx);
     const int n_groups = walk.g1 - walk.g0;
-    const int my_groups = n_groups;
-    auto group_of = [&](int t) { return t; };
 
     const int heads_here = min(16, p.n_rep - hg * 16);
     const int head0 = g * p.n_rep + hg * 16;
@@ -245,7 +237,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
     s16x8 kr[NS][NI], vr[NS][NI];
     static_assert(NI == KC, "a 16-row group is NI row loads and KC contraction chunks");
     auto load_group = [&](int t, s16x8 (&kk)[NI], s16x8 (&vv)[NI]) {
-        const int r0 = row_lo + group_of(t) * kGroupRows;
+        const int r0 = row_lo + t * kGroupRows;
 #pragma unroll
         for (int j = 0; j < NI; ++j) {
             const int row = j * RPI + lane / G;
@@ -287,7 +279,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
                 s = T::mfma16(a, qf[c], s);
             }
         }
-        const int key0 = row_lo + group_of(t) * kGroupRows + 4 * quad;
+        const int key0 = row_lo + t * kGroupRows + 4 * quad;
 #pragma unroll
         for (int r = 0; r < 4; ++r) s[r] = (key0 + r < row_hi) ? s[r] : -INFINITY;
         // ---- park the V rows in LDS (swizzled) for the transpose reads -------------------------
@@ -329,10 +321,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
         }
     };
 
-    for (int t0 = 0; t0 < my_groups; t0 += NS) {
+    for (int t0 = 0; t0 < n_groups; t0 += NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            if (t0 + s < my_groups) consume(t0 + s, kr[s], vr[s]);
+            if (t0 + s < n_groups) consume(t0 + s, kr[s], vr[s]);
             load_group(t0 + s + NS, kr[s], vr[s]);
         }
     }
@@ -351,10 +343,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_MIN_WAVES_PER_SIMD
 }
 
 // ---- decode over Q8_0 caches -----------------------------------------------------------------------
-#ifndef MINFER_DECODE_STAGES_Q8
-#define MINFER_DECODE_STAGES_Q8 2
-#endif
-constexpr int kDecodeStagesQ8 = MINFER_DECODE_STAGES_Q8;   // ring depth, in 32-row groups
+constexpr int kDecodeStagesQ8 = 2;   // ring depth, in 32-row groups
 constexpr int kGroupRowsQ8 = 32;
 
 template <int D> struct DecodeGeomQ8 {
@@ -371,11 +360,8 @@ template <int D> struct DecodeGeomQ8 {
 };
 
 // kv0/kv1 of DecodeParams are byte strides here; q and out are fp16.
-#ifndef MINFER_DECODE_Q8_MIN_WAVES_PER_SIMD
-#define MINFER_DECODE_Q8_MIN_WAVES_PER_SIMD 2
-#endif
 template <int D>
-__global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_SIMD) void decode_split_q8_kernel(const DecodeParams p) {
+__global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode_split_q8_kernel(const DecodeParams p) {
     using T = F16;
     using GEO = DecodeGeom<D>;
     using Q = DecodeGeomQ8<D>;
@@ -398,8 +384,6 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
     const int row_lo = walk.g0 * GR;                         // a multiple of 32
     const int row_hi = min(walk.g1 * GR, ctx);
     const int n_groups = walk.g1 - walk.g0;
-    const int my_groups = n_groups;
-    auto group_of = [&](int t) { return t; };
 
     const int heads_here = min(16, p.n_rep - hg * 16);
     const int head0 = g * p.n_rep + hg * 16;
@@ -439,8 +423,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
     // wave's last group have every lane re-read one piece of the last group, which costs one cache line.  The
     // loop body stays straight-line code that way, which lets the compiler's wait counts keep NS-1 groups in flight.
     auto piece_offset = [&](int t, int j, int64_t last, int64_t& group_off) {
-        const bool real = group_of(t) < n_groups;
-        const int grp = min(group_of(t), n_groups - 1);
+        const bool real = t < n_groups;
+        const int grp = min(t, n_groups - 1);
         group_off = (int64_t)(row_lo + grp * GR) * ROWB;              // a multiple of 16, wave-uniform
         // the group's own pieces only (they are what its LDS area holds), and none past the chunk's last one
         const int rel_last = real ? (int)min(last - group_off, (int64_t)16 * (NG - 1)) : 0;   // >= 0
@@ -484,7 +468,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
     };
 
     auto consume = [&](int t, const Stage& st) {
-        const int r0 = row_lo + group_of(t) * GR;
+        const int r0 = row_lo + t * GR;
         int64_t goff;
         // ---- the group's pieces into the wave's raw areas ----------------------------------------------
 #pragma unroll
@@ -579,10 +563,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64, MINFER_DECODE_Q8_MIN_WAVES_PER_S
         }
     };
 
-    for (int t0 = 0; t0 < my_groups; t0 += NS) {
+    for (int t0 = 0; t0 < n_groups; t0 += NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            if (t0 + s < my_groups) consume(t0 + s, ring[s]);
+            if (t0 + s < n_groups) consume(t0 + s, ring[s]);
             load_group(t0 + s + NS, ring[s]);
         }
     }
@@ -686,21 +670,21 @@ static size_t decode_ws_bytes(int64_t B, int64_t Hq, int64_t Lmax, int64_t D) {
     return (size_t)(B * Hq * S * (D + 2) * 4 + 255) / 256 * 256 + (size_t)((B + 1) * 4 + 255) / 256 * 256 + 256;
 }
 
-// Workgroups of the split launch: as many as the chip holds at once (two per compute unit: LDS and registers
-// allow no more), so that each gets one equal share of the work and all run from start to end.
-#ifndef MINFER_DECODE_WG_PER_CU
-#define MINFER_DECODE_WG_PER_CU 2
-#endif
+// Workgroups of the split launch: as many as the chip holds at once (kDecodeWgPerCu per compute unit: LDS and
+// registers allow no more), so that each gets one equal share of the work and all run from start to end.
+// The per-device count is cached in atomics: concurrent first calls at worst both query the attribute.
 static int decode_workgroups() {
-    static int cached[64] = {0};
+    static std::atomic<int> cached[64];
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
-    if (cached[dev] == 0) {
+    int n = cached[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
         int cus = 0;
         if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
-        cached[dev] = cus * MINFER_DECODE_WG_PER_CU;
+        n = cus * kDecodeWgPerCu;
+        cached[dev].store(n, std::memory_order_relaxed);
     }
-    return cached[dev];
+    return n;
 }
 
 template <class T, int D>
@@ -724,8 +708,8 @@ static int launch_decode_q8(const DecodeParams& p, void* out, int64_t o0, int64_
 using namespace minfer_attn;
 
 MINFER_ATTN_EXPORT size_t minfer_flash_attn_decode_workspace_bytes(int64_t B, int64_t Hq, int64_t Lmax, int64_t D) {
-    if (B <= 0 || Hq <= 0 || Lmax <= 0 || D <= 0) return 256;
-    return decode_ws_bytes(B, Hq, Lmax, D);
+    if (B <= 0 || Hq <= 0 || Lmax < 0 || D <= 0) return 256;
+    return decode_ws_bytes(B, Hq, Lmax, D);   // Lmax == 0 (an empty cache) still has its rows' slots: the call writes zeros
 }
 
 // Fills the launch parameters both decode entry points share; returns an error code or MINFER_ATTN_OK.
@@ -764,6 +748,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode(int dtype, const void* q, const 
                                         int64_t Lmax, int64_t D, const minfer_attn_strides* st, void* workspace,
                                         size_t workspace_bytes, void* stream_v) {
     clear_error();
+    if (Lmax == 0) { k_cache = k_cache ? k_cache : q; v_cache = v_cache ? v_cache : q; }   // an empty cache has no rows to point at
     if (int rc = check_common(dtype, q, k_cache, v_cache, out, Hq, Hkv, D, st)) return rc;
     DecodeParams p{};
     if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, workspace, workspace_bytes, kGroupRows)) return rc;

@@ -110,10 +110,7 @@ struct PrefillParams {
 };
 
 enum { MODE_DENSE = 0, MODE_VARLEN = 1 };
-#ifndef MINFER_PREFILL_WAVES
-#define MINFER_PREFILL_WAVES 8
-#endif
-constexpr int kWaves = MINFER_PREFILL_WAVES;   // waves per workgroup
+constexpr int kWaves = 8;   // waves per workgroup
 constexpr int kThreads = kWaves * 64;
 
 template <int D> struct TileGeom {
@@ -546,6 +543,16 @@ static int dispatch_prefill(int dtype, int64_t D, const PrefillParams& p, int gr
     return D == 128 ? launch_prefill<BF16, 128, MODE>(p, grid, stream) : launch_prefill<BF16, 64, MODE>(p, grid, stream);
 }
 
+// The global->LDS tile copies address a tile's rows with a 32-bit unsigned per-lane byte offset from the tile's first
+// row (rows 0..63 of it, plus a granule inside the row): the K/V row stride must keep that below 2^32.
+static int check_row_stride(const minfer_attn_strides* st, const char* op) {
+    if (st->kv2 >= (INT64_C(1) << 25)) {
+        snprintf(error_buf(), 512, "%s: k/v row stride (dim 2) must be below 2^25 elements", op);
+        return MINFER_ATTN_EINVAL;
+    }
+    return MINFER_ATTN_OK;
+}
+
 static void fill_common(PrefillParams& p, const void* q, const void* k, const void* v, void* out,
                         int64_t Hq, int64_t Hkv, int64_t D, const minfer_attn_strides* st) {
     p.q = q; p.k = k; p.v = v; p.out = out;
@@ -573,6 +580,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k
                                  size_t workspace_bytes, void* stream_v) {
     clear_error();
     if (int rc = check_common(dtype, q, k, v, out, Hq, Hkv, D, st)) return rc;
+    if (int rc = check_row_stride(st, "flash_attn")) return rc;
     if (!mask) return fail(MINFER_ATTN_EINVAL, "flash_attn: mask is null");
     if (B < 0 || L < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn: negative B or L");
     if (B == 0 || L == 0) return MINFER_ATTN_OK;
@@ -606,6 +614,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const 
                                         const minfer_attn_strides* st, void* stream_v) {
     clear_error();
     if (int rc = check_common(dtype, q, k, v, out, Hq, Hkv, D, st)) return rc;
+    if (int rc = check_row_stride(st, "flash_attn_varlen")) return rc;
     if (!cu_seqlens) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: cu_seqlens is null");
     if (n_seqs < 0 || T < 0 || max_seqlen < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: negative size");
     if (n_seqs == 0 || T == 0) return MINFER_ATTN_OK;

@@ -24,9 +24,6 @@
 
 namespace minfer_attn {
 
-#ifndef MINFER_GEMM_GROUP_M
-#define MINFER_GEMM_GROUP_M 4
-#endif
 
 constexpr int kBK = 64;
 // Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
@@ -71,11 +68,10 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     if (t >= p.tiles_m * p.tiles_n) return;
     // Tiles are numbered down bands of kGroupM tile rows, so that the tiles an XCD runs at one time form a block that
     // shares A row panels as well as B column panels in its L2 (row-major numbering made every XCD read all of B).
-    constexpr int kGroupM = MINFER_GEMM_GROUP_M;
+    constexpr int kGroupM = 4;
     const int band = t / (kGroupM * p.tiles_n), in_band = t % (kGroupM * p.tiles_n);
     const int first_m = band * kGroupM, gm = min(kGroupM, p.tiles_m - first_m);
     const int m0 = (first_m + in_band % gm) * kBM, n0 = (in_band / gm) * kBN;
-    const bool full_m = m0 + kBM <= p.M, full_n = n0 + kBN <= p.N;
 
     const short* Ag = (const short*)p.A;
     const short* Bg = (const short*)p.B;
@@ -109,7 +105,6 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
             b_dst[j] = sub * kColTile + 4 * (q & 15) * 256;
         }
     }
-    (void)full_m; (void)full_n;
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
         const short* abase = Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK;
         const short* bbase = NT ? Bg + (int64_t)n0 * p.ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * p.ldb + n0;

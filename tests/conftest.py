@@ -5,9 +5,13 @@ import pytest
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 PKG = os.path.join(ROOT, "minfer-python_amd")
-for p in (ROOT, PKG, os.path.join(PKG, "apps"), os.path.dirname(os.path.abspath(__file__))):
+for p in (ROOT, PKG, os.path.dirname(os.path.abspath(__file__))):
     if p not in sys.path:
         sys.path.insert(0, p)
+# the apps directory goes last: it holds a profile.py (the reference's name for that script), which must not
+# shadow the standard library's `profile` module (cProfile, and through it torch.library.opcheck, imports it)
+if os.path.join(PKG, "apps") not in sys.path:
+    sys.path.append(os.path.join(PKG, "apps"))
 
 
 def pytest_configure(config):

@@ -59,6 +59,8 @@ def make(M, N, K, layout, dtype, seed):
     (30, 5200, 128, 2.0, 1.0),       # wide enough for two column groups per workgroup, the last one ragged
     (37, 24, 192, 0.5, 1.0),         # ragged rows, a last group of 16 columns that is half empty
     (17, 4104, 64, 1.0, 1.0),        # one K step: seven of the eight waves have nothing to add
+    (64, 6144, 4096, 2.0, 3.0),      # 64 rows, two column groups per workgroup: the few-row kernel's largest instantiation
+    (40, 5128, 1024, 1.0, 1.0),      # 40 rows (three row blocks), two column groups, the last one ragged
 ])
 def test_gemm_matches_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, M + N + K)

@@ -262,6 +262,7 @@ def test_ragged_prefill_full():
     (2, 40, 2, 700, 128, 500, 700),    # n_rep = 20: two head groups
     (3, 6, 6, 1537, 128, 1537, 1537),  # ctx = Lmax, n_rep = 1, 4 chunks with a 1-row tail
     (4, 4, 1, 17, 64, 1, 17),
+    (3, 8, 2, 0, 128, 0, 0),           # an empty cache: zeros, with the workspace size the library reports for it
 ])
 def test_decode_matches_oracle(dtype, B, Hq, Hkv, Lmax, D, lo, hi):
     scale = 1.0 if dtype == torch.float16 else 0.5

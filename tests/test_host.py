@@ -60,6 +60,9 @@ def test_validation_rejects_before_launch():
     assert _call_prefill(ws=0) == capi.EWORKSPACE
     assert _call_prefill(ws_bytes=0) == capi.EWORKSPACE and "workspace" in capi.last_error()
     assert _call_prefill(L=1 << 20) == capi.EINVAL
+    # a K/V row stride the tile copies' 32-bit lane offsets cannot span
+    assert _call_prefill(st=capi.Strides(8 * 64 * 128, 64 * 128, 128, 2 << 31, 1 << 31, 1 << 25, 8 * 64 * 128, 64 * 128, 128)) == capi.EINVAL \
+        and "row stride" in capi.last_error()
     # empty problems are accepted and launch nothing
     assert _call_prefill(B=0) == capi.OK and capi.last_error() == ""
     assert _call_prefill(L=0) == capi.OK
@@ -76,6 +79,14 @@ def test_validation_rejects_before_launch():
                                       ctypes.byref(st), None) == capi.EINVAL
     assert L.minfer_flash_attn_varlen(capi.BF16, 0x1000, 0x2000, 0x3000, 0x4000, 0, 64, 0x5000, 8, 2, 64, 128,
                                       ctypes.byref(st), None) == capi.OK
+    big = capi.Strides(1024, 128, 128, 1 << 32, 1 << 31, 1 << 25, 1024, 128, 128)
+    assert L.minfer_flash_attn_varlen(capi.BF16, 0x1000, 0x2000, 0x3000, 0x4000, 2, 64, 0x5000, 8, 2, 64, 128,
+                                      ctypes.byref(big), None) == capi.EINVAL and "row stride" in capi.last_error()
+    # an empty cache (Lmax = 0) is a valid call: the size the library asks for is the size it accepts
+    need0 = L.minfer_flash_attn_decode_workspace_bytes(2, 8, 0, 128)
+    assert need0 >= 2 * 8 * 130 * 4
+    assert L.minfer_flash_attn_decode(capi.F16, 0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 2, 8, 2, 0, 128,
+                                      ctypes.byref(st), 0x6000, need0 - 256, None) == capi.EWORKSPACE
 
 
 def test_rope_validation_rejects_before_launch():
