@@ -88,6 +88,24 @@ int minfer_flash_attn_decode(int dtype, const void* q, const void* k_cache, cons
                              void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * minfer_flash_attn_decode without a workspace argument, for callers that cannot allocate device memory: code
+ * under HIP graph capture, serving loops and harnesses that forbid hipMalloc.  It has no counterpart in the
+ * reference.  The split-KV partial results go to a device array that is part of the library's code object
+ * (MINFER_DECODE_NOALLOC_SCRATCH_BYTES bytes on every GPU the library is used on, held until the process ends);
+ * a problem whose minfer_flash_attn_decode_workspace_bytes(B, Hq, Lmax, D) exceeds that size is rejected with
+ * MINFER_ATTN_EWORKSPACE (nothing launched).  The call allocates and frees nothing.  Its first call on a device
+ * looks the array's address up (which may load the code object): make that call outside a graph capture.  All calls
+ * on one GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls that
+ * follow each other on one stream do not.  Arguments, results and errors are otherwise those of
+ * minfer_flash_attn_decode (16-bit caches only).
+ */
+#define MINFER_DECODE_NOALLOC_SCRATCH_BYTES (64u << 20)
+int minfer_flash_attn_decode_noalloc(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                                     const int32_t* ctx_lens, void* out,
+                                     int64_t B, int64_t Hq, int64_t Hkv, int64_t Lmax, int64_t D,
+                                     const minfer_attn_strides* strides, void* stream);
+
+/*
  * Packed ragged causal prefill: q,out [1,Hq,T,D]; k,v [1,Hkv,T,D]; cu_seqlens int32 [n_seqs+1]
  * on the device with cu_seqlens[0] == 0 and cu_seqlens[n_seqs] == T; token rows
  * cu_seqlens[s]..cu_seqlens[s+1]-1 form sequence s and attend causally inside it only.

@@ -31,6 +31,7 @@
 // D/4 * quad .. of its key, which is a valid MFMA contraction order as long as Q^T is loaded in the same
 // order.  V is parked as fp16 rows and read back transposed, as on the fp16 path.
 #include <atomic>
+#include <mutex>
 
 #include "attn_common.h"
 #include "attn_host.h"
@@ -784,4 +785,65 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode_q8_0(const void* q, const void* 
     if (B == 0) return MINFER_ATTN_OK;
     hipStream_t stream = (hipStream_t)stream_v;
     return D == 128 ? launch_decode_q8<128>(p, out, st->o0, st->o1, stream) : launch_decode_q8<64>(p, out, st->o0, st->o1, stream);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Decode for callers that cannot allocate (code under HIP graph capture, serving loops that must not touch the
+// allocator): the split-KV partial results live in a file-scope device array instead of a caller workspace.
+// Every GPU the library runs on holds its own copy of the array, at its own address, until the process ends; the
+// array's name is only a host-side handle, the device address comes from hipGetSymbolAddress, once per device.
+// The partial slots a call reads are all written by that call's split kernel first (slots past a row's count are
+// loaded and discarded), so nothing needs clearing between calls; calls that overlap in time on one GPU would
+// share the slots and race.
+// ------------------------------------------------------------------------------------------------
+namespace minfer_attn {
+static __device__ __align__(256) unsigned char scratch[MINFER_DECODE_NOALLOC_SCRATCH_BYTES];
+
+static int decode_scratch(void** ptr_out) {
+    static std::mutex mu;
+    static void* ptrs[64] = {nullptr};
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return fail(MINFER_ATTN_ELAUNCH, "flash_attn_decode_noalloc: hipGetDevice failed");
+    if (dev < 0 || dev >= 64) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: device index above 63 unsupported");
+    std::lock_guard<std::mutex> lock(mu);
+    if (!ptrs[dev]) {
+        void* ptr = nullptr;
+        const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr) {
+            snprintf(error_buf(), 512, "flash_attn_decode_noalloc: hipGetSymbolAddress failed: %s", hipGetErrorString(e));
+            return MINFER_ATTN_ELAUNCH;
+        }
+        ptrs[dev] = ptr;
+    }
+    *ptr_out = ptrs[dev];
+    return MINFER_ATTN_OK;
+}
+}  // namespace minfer_attn
+
+MINFER_ATTN_EXPORT int minfer_flash_attn_decode_noalloc(int dtype, const void* q, const void* k_cache, const void* v_cache,
+                                                const int32_t* ctx_lens, void* out, int64_t B, int64_t Hq, int64_t Hkv,
+                                                int64_t Lmax, int64_t D, const minfer_attn_strides* st, void* stream_v) {
+    clear_error();
+    if (Lmax == 0) { k_cache = k_cache ? k_cache : q; v_cache = v_cache ? v_cache : q; }   // an empty cache has no rows to point at
+    if (int rc = check_common(dtype, q, k_cache, v_cache, out, Hq, Hkv, D, st)) return rc;
+    if (!ctx_lens) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: ctx_lens is null");
+    if (B < 0 || Lmax < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: negative B or Lmax");
+    if (B > 65535 || Lmax > (1 << 30)) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: B > 65535 or Lmax > 2^30 unsupported");
+    if (B == 0) return MINFER_ATTN_OK;
+    if (decode_ws_bytes(B, Hq, Lmax, D) > (size_t)MINFER_DECODE_NOALLOC_SCRATCH_BYTES) {
+        snprintf(error_buf(), 512, "flash_attn_decode_noalloc: B=%lld Hq=%lld Lmax=%lld D=%lld needs %zu bytes of partial results, "
+                 "the built-in scratch holds %zu; use minfer_flash_attn_decode with a workspace",
+                 (long long)B, (long long)Hq, (long long)Lmax, (long long)D, decode_ws_bytes(B, Hq, Lmax, D),
+                 (size_t)MINFER_DECODE_NOALLOC_SCRATCH_BYTES);
+        return MINFER_ATTN_EWORKSPACE;
+    }
+    void* ws = nullptr;
+    if (int rc = decode_scratch(&ws)) return rc;
+    DecodeParams p{};
+    if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, ws,
+                             (size_t)MINFER_DECODE_NOALLOC_SCRATCH_BYTES, kGroupRows)) return rc;
+    hipStream_t stream = (hipStream_t)stream_v;
+    if (dtype == MINFER_ATTN_F16)
+        return D == 128 ? launch_decode<F16, 128>(p, out, st->o0, st->o1, stream) : launch_decode<F16, 64>(p, out, st->o0, st->o1, stream);
+    return D == 128 ? launch_decode<BF16, 128>(p, out, st->o0, st->o1, stream) : launch_decode<BF16, 64>(p, out, st->o0, st->o1, stream);
 }

@@ -40,6 +40,9 @@ def lib():
         L.minfer_flash_attn_decode.restype = ctypes.c_int
         L.minfer_flash_attn_decode.argtypes = [ctypes.c_int, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
                                                ctypes.POINTER(Strides), vp, sz, vp]
+        L.minfer_flash_attn_decode_noalloc.restype = ctypes.c_int
+        L.minfer_flash_attn_decode_noalloc.argtypes = [ctypes.c_int, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
+                                                       ctypes.POINTER(Strides), vp]
         L.minfer_flash_attn_varlen.restype = ctypes.c_int
         L.minfer_flash_attn_varlen.argtypes = [ctypes.c_int, vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, i64,
                                                ctypes.POINTER(Strides), vp]
@@ -110,6 +113,18 @@ def flash_attn_decode(q, k_cache, v_cache, ctx_lens, out, workspace=None):
     return lib().minfer_flash_attn_decode(_dtype_code(q), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                           ctx_lens.data_ptr(), out.data_ptr(), B, Hq, Hkv, Lmax, D,
                                           ctypes.byref(st), workspace.data_ptr(), workspace.numel(), _stream())
+
+
+DECODE_NOALLOC_SCRATCH_BYTES = 64 << 20
+
+
+def flash_attn_decode_noalloc(q, k_cache, v_cache, ctx_lens, out):
+    """The decode entry point that takes no workspace and allocates nothing."""
+    B, Hq, _, D = q.shape
+    st = _strides(q, k_cache, out)
+    return lib().minfer_flash_attn_decode_noalloc(_dtype_code(q), q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
+                                                  ctx_lens.data_ptr(), out.data_ptr(), B, Hq, k_cache.shape[1],
+                                                  k_cache.shape[2], D, ctypes.byref(st), _stream())
 
 
 def flash_attn_varlen(q, k, v, cu_seqlens, max_seqlen, out):

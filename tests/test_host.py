@@ -82,6 +82,12 @@ def test_validation_rejects_before_launch():
     big = capi.Strides(1024, 128, 128, 1 << 32, 1 << 31, 1 << 25, 1024, 128, 128)
     assert L.minfer_flash_attn_varlen(capi.BF16, 0x1000, 0x2000, 0x3000, 0x4000, 2, 64, 0x5000, 8, 2, 64, 128,
                                       ctypes.byref(big), None) == capi.EINVAL and "row stride" in capi.last_error()
+    # the allocation-free decode refuses, on the host, a problem its built-in scratch array cannot hold
+    assert L.minfer_flash_attn_decode_workspace_bytes(256, 64, 8192, 128) > capi.DECODE_NOALLOC_SCRATCH_BYTES
+    assert L.minfer_flash_attn_decode_noalloc(capi.F16, 0x1000, 0x2000, 0x3000, 0x4000, 0x5000, 256, 64, 8, 8192, 128,
+                                              ctypes.byref(st), None) == capi.EWORKSPACE and "scratch" in capi.last_error()
+    assert L.minfer_flash_attn_decode_noalloc(capi.F16, 0x1000, 0x2000, 0x3000, None, 0x5000, 1, 8, 2, 64, 128,
+                                              ctypes.byref(st), None) == capi.EINVAL
     # an empty cache (Lmax = 0) is a valid call: the size the library asks for is the size it accepts
     need0 = L.minfer_flash_attn_decode_workspace_bytes(2, 8, 0, 128)
     assert need0 >= 2 * 8 * 130 * 4
