@@ -150,6 +150,25 @@ int minfer_rope_kv_append(int dtype, int style, void* q, const void* k, const vo
                           int64_t rotary_dim, double freq_base, void* stream);
 
 /*
+ * The producer with the per-head RMS normalisation of q and k in front of the rotation (reference: the optional
+ * rmsnorm(q), rmsnorm(k) calls between the QKV projection and the rotary embedding, src/minfer/core.py:224-230, each
+ * being rmsnorm_cuda over [B,L,n_heads,head_dim], rmsnorm/op.cuh:20-70): every head of q is replaced by
+ * rope(round(rmsnorm(head, wq_norm, eps))), every head of k goes through the same with wk_norm on its way into the
+ * cache, v is copied; the result equals minfer_rmsnorm on q and on k followed by minfer_rope_kv_append (or
+ * minfer_rope_kv_append_q8_0) bit for bit, with one pass over q, k and v instead of two.  wq_norm / wk_norm are
+ * [D] in the activations' dtype; a null weight leaves that tensor un-normalised.  cache_type is the activations'
+ * dtype (caches [B,Hkv,Lmax,D], element strides) or MINFER_Q8_0 (caches of Q8_0 blocks, byte strides, rows dense:
+ * cache_stride_row = D/32 * 34).  D must be 64 or 128; the other requirements are those of minfer_rope_kv_append.
+ * No counterpart as one call in the reference.
+ */
+int minfer_rope_kv_append_norm(int dtype, int style, int cache_type, void* q, const void* k, const void* v,
+                               const void* wq_norm, const void* wk_norm, double eps,
+                               const int32_t* positions, void* k_cache, void* v_cache,
+                               int64_t B, int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
+                               int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_row,
+                               int64_t rotary_dim, double freq_base, void* stream);
+
+/*
  * RMS normalisation: in, out are n_vectors contiguous vectors of length dim; w has dim elements;
  *   out[v, i] = in[v, i] * w[i] / sqrt(mean_i(in[v, :]^2) + eps)      (fp32 arithmetic, one rounding)
  * The reference's [B,L,hidden] and [B,L,n_heads,head_dim] inputs are both this with dim = |w| and
@@ -175,6 +194,21 @@ int minfer_rmsnorm(int dtype, const void* in, const void* w, void* out, int64_t 
 int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
                 int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
                 double alpha, double beta, void* stream);
+
+/*
+ * The QKV projection in one launch: q_out[M,Nq] = x[M,K] wq^T, k_out[M,Nk] = x wk^T, v_out[M,Nv] = x wv^T, the three
+ * weights stored [N, K] (the reference's layout for them), 16-bit operands, fp32 accumulation, one rounding; ld* are
+ * row strides in elements.  What the reference's fused qkv operator is meant to be (reference:
+ * src/minfer/kernels/torch_ext/csrc/cuda/qkv/op.cuh:21-34, a stub there; the model's call src/minfer/core.py:222-223;
+ * expected values test/kernels.py:172-216).  One grid covers the column tiles of all three weights, so x is
+ * read by one kernel and the narrow k and v projections share the launch with the wide q projection; every element
+ * equals what minfer_gemm with MINFER_GEMM_B_NK, alpha 1, beta 0 gives for its weight.  Shapes the tiled kernels
+ * cannot take (see minfer_gemm) run as three plain launches.
+ */
+int minfer_qkv(int dtype, const void* x, const void* wq, const void* wk, const void* wv,
+               void* q_out, void* k_out, void* v_out, int64_t M, int64_t K, int64_t Nq, int64_t Nk, int64_t Nv,
+               int64_t ldx, int64_t ldwq, int64_t ldwk, int64_t ldwv, int64_t ldq, int64_t ldk, int64_t ldv,
+               void* stream);
 
 /*
  * Q8_0 blocks: 32 consecutive values of a row as an fp16 scale d followed by 32 int8, 34 bytes, no padding

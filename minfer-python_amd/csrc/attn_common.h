@@ -185,6 +185,24 @@ template <class V> MA_DEV void stream_store(V* p, V v) { __builtin_nontemporal_s
 template <bool STREAM, class V> MA_DEV V load_once(const V* p) { return STREAM ? __builtin_nontemporal_load(p) : *p; }
 template <bool STREAM, class V> MA_DEV void store_once(V* p, V v) { if (STREAM) __builtin_nontemporal_store(v, p); else *p = v; }
 
+// Pieces of the RMS normalisation that the normalisation kernels and the rope producer that normalises heads share
+// (the same code on both sides, so their results agree bit for bit): the sum of squares of 8 elements, and
+// x * w * scale rounded once to the element type.
+template <class T> MA_DEV float sum_sq8(s16x8 v) {
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { const float f = T::to_float(v[i]); s += f * f; }
+    return s;
+}
+template <class T> MA_DEV s16x8 scale8w(s16x8 v, s16x8 w, float sc) {
+    uint32_t r[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        r[i] = T::pack2(T::to_float(v[2 * i]) * T::to_float(w[2 * i]) * sc, T::to_float(v[2 * i + 1]) * T::to_float(w[2 * i + 1]) * sc);
+    uint4 u; u.x = r[0]; u.y = r[1]; u.z = r[2]; u.w = r[3];
+    return __builtin_bit_cast(s16x8, u);
+}
+
 MA_DEV int wave_id() { return __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)); }
 
 }  // namespace minfer_attn

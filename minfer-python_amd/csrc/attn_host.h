@@ -63,4 +63,9 @@ inline int check_common(int dtype, const void* q, const void* k, const void* v, 
     return MINFER_ATTN_OK;
 }
 
+// Dequantises K and V rows of Q8_0 blocks ([B, Hkv, L] rows of D/32 blocks; byte strides s0, s1 between batch
+// entries and heads; rows dense) into contiguous fp16 [B, Hkv, L, D] (csrc/quant.hip).
+int launch_dequant_q8_0_kv(const void* k, const void* v, void* k_out, void* v_out, int64_t B, int64_t Hkv, int64_t L,
+                           int64_t D, int64_t s0, int64_t s1, hipStream_t stream);
+
 }  // namespace minfer_attn

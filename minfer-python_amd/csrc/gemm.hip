@@ -41,19 +41,34 @@ using GemmSmall = GemmShape<2, 2, 2, 2>;
 constexpr int kRowTile = 8192;              // sub-tile [64 rows][64 k], 128-byte rows (A, and B as [N, K])
 constexpr int kColTile = 16384;             // sub-tile [64 k][128 n], 256-byte rows (B as [K, N])
 
+// Several weights that share A in one launch (the QKV projection): the column tiles (tiled kernel) or column groups
+// (few-row kernel) of weight s follow those of weight s - 1; `end` holds the cumulative counts.  No C operand.
+constexpr int kMaxGroup = 3;
+struct GemmGroup {
+    const void* B[kMaxGroup]; void* D[kMaxGroup];
+    int N[kMaxGroup], end[kMaxGroup];
+    int64_t ldb[kMaxGroup], ldd[kMaxGroup];
+};
 struct GemmParams {
     const void* A; const void* B; const void* C; void* D;
     int M, N, K;
     int64_t lda, ldb, ldc, ldd;   // row strides in elements
     float alpha, beta;
     int tiles_m, tiles_n, per_xcd;
+    GemmGroup grp;                // used by the GROUPED instantiations only
 };
+// Which weight column unit `c` (a tile column or a column group) belongs to, and its index inside that weight.
+MA_DEV int group_of_unit(const GemmGroup& g, int c, int& local) {
+    const int s = c < g.end[0] ? 0 : (c < g.end[1] ? 1 : 2);
+    local = c - (s == 0 ? 0 : (s == 1 ? g.end[0] : g.end[1]));
+    return s;
+}
 
 // swizzles: granule index of a row XORed with a function of the row (see the attention kernel's TileGeom)
 MA_DEV int swz_row_tile(int row) { return (row >> 1) & 7; }        // 128-byte rows, read 32 rows x 16 bytes
 MA_DEV int swz_col_tile(int row) { return (row & 3) << 2; }        // 256-byte rows, read 4 rows x 64 bytes (transposing)
 
-template <class T, bool NT, class SH>
+template <class T, bool NT, class SH, bool GROUPED = false>
 __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const GemmParams p) {
     constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB, NB = SH::NB, CA = SH::A_COPIES, CB = SH::B_COPIES;
     __shared__ __attribute__((aligned(1024))) char a_lds[2][SH::A_PANEL];
@@ -71,10 +86,24 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     constexpr int kGroupM = 4;
     const int band = t / (kGroupM * p.tiles_n), in_band = t % (kGroupM * p.tiles_n);
     const int first_m = band * kGroupM, gm = min(kGroupM, p.tiles_m - first_m);
-    const int m0 = (first_m + in_band % gm) * kBM, n0 = (in_band / gm) * kBN;
+    const int m0 = (first_m + in_band % gm) * kBM;
+    int n0 = (in_band / gm) * kBN;
 
     const short* Ag = (const short*)p.A;
     const short* Bg = (const short*)p.B;
+    short* Dg = (short*)p.D;
+    int N = p.N;
+    int64_t ldb = p.ldb, ldd = p.ldd;
+    if (GROUPED) {   // the tile column's weight, output and place inside them (all wave-uniform)
+        int local;
+        const int sg = group_of_unit(p.grp, in_band / gm, local);
+        n0 = local * kBN;
+        Bg = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]);
+        Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
+        N = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
+        ldb = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
+        ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
+    }
 
     // ---- global -> LDS copies: lane offsets (bytes) from the panel's first element ---------------------
     // Every wave issues 4 wave-wide copies (1 KB each) per panel and K step; copy q = j*NW + w of a panel covers
@@ -95,19 +124,19 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
         const int q = j * NW + w;
         if (NT) {
             const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
-            const int n = min(n0 + 64 * sub + row, p.N - 1) - n0;
-            b_off[j] = (uint32_t)((int64_t)n * p.ldb + 8 * (pg ^ swz_row_tile(row))) * 2u;
+            const int n = min(n0 + 64 * sub + row, N - 1) - n0;
+            b_off[j] = (uint32_t)((int64_t)n * ldb + 8 * (pg ^ swz_row_tile(row))) * 2u;
             b_dst[j] = sub * kRowTile + 8 * (q & 7) * 128;
         } else {
             const int sub = q >> 4, row = 4 * (q & 15) + (lane >> 4), pg = lane & 15;
-            const int col = min(n0 + 128 * sub + 8 * (pg ^ swz_col_tile(row)), p.N - 8) - n0;
-            b_off[j] = (uint32_t)((int64_t)row * p.ldb + col) * 2u;
+            const int col = min(n0 + 128 * sub + 8 * (pg ^ swz_col_tile(row)), N - 8) - n0;
+            b_off[j] = (uint32_t)((int64_t)row * ldb + col) * 2u;
             b_dst[j] = sub * kColTile + 4 * (q & 15) * 256;
         }
     }
     auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
         const short* abase = Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK;
-        const short* bbase = NT ? Bg + (int64_t)n0 * p.ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * p.ldb + n0;
+        const short* bbase = NT ? Bg + (int64_t)n0 * ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * ldb + n0;
 #pragma unroll
         for (int j = 0; j < CA; ++j) copy16_global_to_lds(abase, a_off[j], &a_lds[stage][a_dst[j]]);
 #pragma unroll
@@ -204,7 +233,6 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 
     // ---- epilogue: D = alpha * acc + beta * C; register r of a block is n = 8(r/4) + 4h + r%4, m = l32 ----
     const short* Cg = (const short*)p.C;
-    short* Dg = (short*)p.D;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const int m = m0 + 32 * MB * wm + 32 * mb + l32;
@@ -214,7 +242,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
                 const int n = n0 + 32 * NB * wn + 32 * nb + 8 * j + 4 * h;
-                if (n >= p.N) continue;
+                if (n >= N) continue;
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[nb][mb][4 * j + e];
@@ -226,7 +254,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
                 uint2 pk;
                 pk.x = T::pack2(v[0], v[1]);
                 pk.y = T::pack2(v[2], v[3]);
-                *reinterpret_cast<uint2*>(Dg + (int64_t)m * p.ldd + n) = pk;
+                *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
             }
         }
     }
@@ -240,17 +268,31 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 // of the contraction.  MB = ceil(M / 16) <= 4.
 constexpr int kSkinnyWaves = 8;
 // NR groups of 16 columns per workgroup (2 for wide weights: half as many workgroups, each A fragment used twice)
-template <class T, int MB, int NR>
+template <class T, int MB, int NR, bool GROUPED = false>
 __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const GemmParams p) {
     __shared__ f32x4 part[kSkinnyWaves][NR][MB][64];
     const int lane = threadIdx.x & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    const int n0 = (int)blockIdx.x * 16 * NR;
+    int n0 = (int)blockIdx.x * 16 * NR;
+    const short* Bg = (const short*)p.B;
+    short* Dg = (short*)p.D;
+    int N = p.N;
+    int64_t ldb = p.ldb, ldd = p.ldd;
+    if (GROUPED) {   // the workgroup's weight, output and place inside them (uniform)
+        int local;
+        const int sg = group_of_unit(p.grp, (int)blockIdx.x, local);
+        n0 = local * 16 * NR;
+        Bg = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]);
+        Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
+        N = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
+        ldb = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
+        ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
+    }
     const int steps = p.K / 64, per = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
     const int s0 = w * per, s1 = min(steps, s0 + per);
     const short* wrow[NR];
 #pragma unroll
-    for (int nr = 0; nr < NR; ++nr) wrow[nr] = (const short*)p.B + (int64_t)min(n0 + 16 * nr + l16, p.N - 1) * p.ldb + 16 * quad;
+    for (int nr = 0; nr < NR; ++nr) wrow[nr] = Bg + (int64_t)min(n0 + 16 * nr + l16, N - 1) * ldb + 16 * quad;
     const short* xrow[MB];
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) xrow[mb] = (const short*)p.A + (int64_t)min(16 * mb + l16, p.M - 1) * p.lda + 16 * quad;
@@ -291,7 +333,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const Ge
 #pragma unroll
     for (int ww = 1; ww < kSkinnyWaves; ++ww) sum += part[ww][nr][mb][lane];
     const int m = 16 * mb + l16, n = n0 + 16 * nr + 4 * quad;
-    if (m >= p.M || n >= p.N) return;
+    if (m >= p.M || n >= N) return;
     float v[4];
 #pragma unroll
     for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
@@ -303,7 +345,7 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_kernel(const Ge
     uint2 pk;
     pk.x = T::pack2(v[0], v[1]);
     pk.y = T::pack2(v[2], v[3]);
-    *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+    *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
 }
 
 template <class T, int NR>
@@ -361,9 +403,80 @@ static int launch_gemm(GemmParams& p, bool fast, hipStream_t stream) {
     return check_launch("gemm_plain_kernel");
 }
 
+// Up to three weights [N_s, K] against one A in one launch (alpha = 1, no C): the tiled kernel over the concatenated
+// column tiles of the weights, or, for a decode step's few rows, the few-row kernel over their column groups.
+template <class T>
+static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
+    int64_t n_sum = 0;
+    for (int s = 0; s < n_w; ++s) n_sum += p.grp.N[s];
+    auto fill_ends = [&](int unit) {
+        int acc = 0;
+        for (int s = 0; s < kMaxGroup; ++s) {
+            if (s < n_w) acc += (p.grp.N[s] + unit - 1) / unit;
+            p.grp.end[s] = acc;
+        }
+        return acc;
+    };
+    if (p.M <= 32 || (p.M <= 64 && n_sum * p.K <= (INT64_C(1) << 25))) {
+        const int nr = (p.M > 16 && n_sum >= 160 * 32) ? 2 : 1;
+        const int groups = fill_ends(16 * nr);
+        const dim3 grid(groups), block(kSkinnyWaves * 64);
+        const int mb = (p.M + 15) / 16;
+#define MINFER_SKINNY(MB, NR) hipLaunchKernelGGL((gemm_skinny_kernel<T, MB, NR, true>), grid, block, 0, stream, p)
+        if (nr == 1) { if (mb == 1) MINFER_SKINNY(1, 1); else if (mb == 2) MINFER_SKINNY(2, 1); else if (mb == 3) MINFER_SKINNY(3, 1); else MINFER_SKINNY(4, 1); }
+        else { if (mb == 2) MINFER_SKINNY(2, 2); else if (mb == 3) MINFER_SKINNY(3, 2); else MINFER_SKINNY(4, 2); }
+#undef MINFER_SKINNY
+        return check_launch("gemm_skinny_kernel (grouped)");
+    }
+    const int64_t big_tiles = (int64_t)((p.M + GemmBig::BM - 1) / GemmBig::BM) * ((n_sum + GemmBig::BN - 1) / GemmBig::BN);
+    const bool big = big_tiles >= 160;
+    const int bm = big ? GemmBig::BM : GemmSmall::BM, bn = big ? GemmBig::BN : GemmSmall::BN;
+    p.tiles_m = (p.M + bm - 1) / bm;
+    p.tiles_n = fill_ends(bn);
+    p.per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+    if (big) hipLaunchKernelGGL((gemm_kernel<T, true, GemmBig, true>), dim3(p.per_xcd * 8), dim3(GemmBig::WAVES * 64), 0, stream, p);
+    else hipLaunchKernelGGL((gemm_kernel<T, true, GemmSmall, true>), dim3(p.per_xcd * 8), dim3(GemmSmall::WAVES * 64), 0, stream, p);
+    return check_launch("gemm_kernel (grouped)");
+}
+
 }  // namespace minfer_attn
 
 using namespace minfer_attn;
+
+MINFER_ATTN_EXPORT int minfer_qkv(int dtype, const void* x, const void* wq, const void* wk, const void* wv,
+                                  void* q_out, void* k_out, void* v_out, int64_t M, int64_t K,
+                                  int64_t Nq, int64_t Nk, int64_t Nv, int64_t ldx, int64_t ldwq, int64_t ldwk, int64_t ldwv,
+                                  int64_t ldq, int64_t ldk, int64_t ldv, void* stream_v) {
+    clear_error();
+    if (dtype != MINFER_ATTN_F16 && dtype != MINFER_ATTN_BF16)
+        return fail(MINFER_ATTN_EINVAL, "qkv: dtype must be MINFER_ATTN_F16 or MINFER_ATTN_BF16");
+    const int64_t Ns[3] = {Nq, Nk, Nv}, ldw[3] = {ldwq, ldwk, ldwv}, ldo[3] = {ldq, ldk, ldv};
+    const void* W[3] = {wq, wk, wv};
+    void* O[3] = {q_out, k_out, v_out};
+    if (M < 0 || K < 0 || M > 0x7fffffffLL || K > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "qkv: bad M or K");
+    if (!x || ldx < K) return fail(MINFER_ATTN_EINVAL, "qkv: x is null or its leading dimension is smaller than K");
+    bool fast = K > 0 && K % kBK == 0 && ldx % 8 == 0 && aligned16(x) && (int64_t)GemmBig::BM * ldx < (1LL << 30);
+    for (int s = 0; s < 3; ++s) {
+        if (Ns[s] < 0 || Ns[s] > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "qkv: bad output width");
+        if (!W[s] || !O[s]) return fail(MINFER_ATTN_EINVAL, "qkv: null pointer");
+        if (ldw[s] < K || ldo[s] < Ns[s]) return fail(MINFER_ATTN_EINVAL, "qkv: a leading dimension is smaller than its row");
+        fast = fast && Ns[s] % 8 == 0 && ldw[s] % 8 == 0 && ldo[s] % 4 == 0 && aligned16(W[s]) && ((uintptr_t)O[s] & 7u) == 0 &&
+               (int64_t)std::max<int64_t>(GemmBig::BN, kBK) * ldw[s] < (1LL << 30);
+    }
+    if (M == 0) return MINFER_ATTN_OK;
+    if (!fast || Nq == 0 || Nk == 0 || Nv == 0) {   // shapes the tiled kernels cannot take: three separate launches
+        for (int s = 0; s < 3; ++s)
+            if (int rc = minfer_gemm(dtype, MINFER_GEMM_B_NK, x, W[s], nullptr, O[s], M, Ns[s], K, ldx, ldw[s], Ns[s], ldo[s], 1.0, 0.0, stream_v))
+                return rc;
+        return MINFER_ATTN_OK;
+    }
+    GemmParams p{};
+    p.A = x; p.M = (int)M; p.K = (int)K; p.lda = ldx; p.alpha = 1.f; p.beta = 0.f; p.C = nullptr;
+    p.B = wq; p.D = q_out; p.N = (int)Nq; p.ldb = ldwq; p.ldd = ldq; p.ldc = ldq;
+    for (int s = 0; s < 3; ++s) { p.grp.B[s] = W[s]; p.grp.D[s] = O[s]; p.grp.N[s] = (int)Ns[s]; p.grp.ldb[s] = ldw[s]; p.grp.ldd[s] = ldo[s]; }
+    hipStream_t stream = (hipStream_t)stream_v;
+    return dtype == MINFER_ATTN_F16 ? launch_grouped<F16>(p, 3, stream) : launch_grouped<BF16>(p, 3, stream);
+}
 
 MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
                                    int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,

@@ -96,6 +96,35 @@ __global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kernel(const char*
     }
 }
 
+// K and V rows of Q8_0 blocks, [B, Hkv, L] rows of D/32 blocks with byte strides s0, s1 between batch entries and
+// heads (rows dense), into two contiguous fp16 tensors [B, Hkv, L, D]: what prefill attention over quantised K/V
+// reads.  grid (pieces of one (batch, head), B * Hkv, 2): z = 0 is K, 1 is V.
+__global__ __launch_bounds__(kQuantThreads) void dequant_q8_0_kv_kernel(const char* k, const char* v, short* k_out, short* v_out,
+                                                                      int Hkv, int64_t s0, int64_t s1, int64_t pieces_per_head) {
+    const int bg = blockIdx.y, b = bg / Hkv, g = bg - b * Hkv;
+    const char* src = (blockIdx.z ? v : k) + (int64_t)b * s0 + (int64_t)g * s1;
+    s16x8* dst = (s16x8*)(blockIdx.z ? v_out : k_out) + (int64_t)bg * pieces_per_head;
+    for (int64_t i = (int64_t)blockIdx.x * kQuantThreads + threadIdx.x; i < pieces_per_head; i += (int64_t)gridDim.x * kQuantThreads) {
+        const char* blk = (const char*)__builtin_assume_aligned(src + (i >> 2) * 34, 2);
+        uint16_t d_bits;
+        uint2 q;
+        __builtin_memcpy(&d_bits, blk, 2);
+        __builtin_memcpy(&q, blk + 2 + 8 * (i & 3), 8);
+        const _Float16 dh = __builtin_bit_cast(_Float16, d_bits);
+        const h16x2 d2 = {dh, dh};
+        dst[i] = dequant8_words(q.x, q.y, d2);
+    }
+}
+
+int launch_dequant_q8_0_kv(const void* k, const void* v, void* k_out, void* v_out, int64_t B, int64_t Hkv, int64_t L,
+                           int64_t D, int64_t s0, int64_t s1, hipStream_t stream) {
+    const int64_t pieces = L * (D / 8);
+    const dim3 grid((unsigned)std::min<int64_t>((pieces + kQuantThreads - 1) / kQuantThreads, 4096), (unsigned)(B * Hkv), 2);
+    hipLaunchKernelGGL(dequant_q8_0_kv_kernel, grid, dim3(kQuantThreads), 0, stream, (const char*)k, (const char*)v,
+                       (short*)k_out, (short*)v_out, (int)Hkv, s0, s1, pieces);
+    return check_launch("dequant_q8_0_kv_kernel");
+}
+
 static int check_rows(const char* op, const void* x, const void* y, int64_t n_rows, int64_t k) {
     char msg[160];
     auto bad = [&](const char* what) {

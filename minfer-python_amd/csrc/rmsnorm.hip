@@ -27,21 +27,6 @@ struct NormParams {
     float eps, inv_dim;
 };
 
-template <class T> MA_DEV float sum_sq8(s16x8 v) {
-    float s = 0.f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) { const float f = T::to_float(v[i]); s += f * f; }
-    return s;
-}
-template <class T> MA_DEV s16x8 scale8w(s16x8 v, s16x8 w, float sc) {
-    uint32_t r[4];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-        r[i] = T::pack2(T::to_float(v[2 * i]) * T::to_float(w[2 * i]) * sc, T::to_float(v[2 * i + 1]) * T::to_float(w[2 * i + 1]) * sc);
-    uint4 u; u.x = r[0]; u.y = r[1]; u.z = r[2]; u.w = r[3];
-    return __builtin_bit_cast(s16x8, u);
-}
-
 // LANES lanes per vector, NCH 16-byte chunks per lane (dim <= LANES * 8 * NCH, dim % 8 == 0): chunk j of a
 // lane covers elements 8 * (j * LANES + lane_in_group) .., so a group reads contiguous 16 * LANES bytes.
 template <class T, int LANES, int NCH, bool STREAM>

@@ -280,6 +280,129 @@ __global__ __launch_bounds__(kRopeThreads) void rope_scalar_kernel(const RopePar
     }
 }
 
+// ------------------------------------------------------------------------------------------------
+// The producer with the per-head RMS normalisation of q and k in front of the rotation (reference: the optional
+// rmsnorm(q), rmsnorm(k) calls between the QKV projection and the rotary embedding, src/minfer/core.py:224-230).
+// A head is in registers between its load and its rotation anyway, so the normalisation costs no memory traffic:
+// G = D/8 neighbouring lanes hold one head (a 16-byte chunk each), sum their squares with lane exchanges, scale,
+// round to the element type exactly as rmsnorm_rows_kernel does (same grouping, same order of additions: the
+// result equals rmsnorm followed by the producer bit for bit), then rotate.  The NeoX partner of a chunk sits in
+// another lane of the group and is fetched by lane exchange.  v is copied (or quantised) as in the plain producer.
+// ------------------------------------------------------------------------------------------------
+struct NormRopeParams {
+    RopeParams r;
+    const void* wq; const void* wk;   // per-head weights [D]; null = that tensor is not normalised
+    float eps, inv_dim;
+};
+
+template <class T, int STYLE, bool Q8, int G, bool STREAM>
+__global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const NormRopeParams np) {
+    const RopeParams& p = np.r;
+    __shared__ f32x2 tab[2][kMaxPairs];
+    constexpr int D = 8 * G;
+    constexpr int UN = 4;             // chunks in flight per thread
+    const int tid = threadIdx.x;
+    const int half_rd = p.rd >> 1;
+    const int heads = p.H + 2 * p.Hkv;
+    const int units = heads * G;
+    const int c = tid & (G - 1);      // the lane's chunk inside its head: elements 8c..8c+7
+    const int rot_chunks = STYLE == ROPE_IL ? p.rd >> 3 : p.rd >> 4;   // IL: chunks that rotate; NeoX: chunks per half
+    // NeoX: chunk c < rd/16 holds the x0 of pairs 8c.., chunk c + rd/16 their x1
+    const bool neox_lo = STYLE == ROPE_NEOX && c < rot_chunks;
+    const bool neox_hi = STYLE == ROPE_NEOX && c >= rot_chunks && c < 2 * rot_chunks;
+    const int partner = neox_lo ? (int)(threadIdx.x & 63) + rot_chunks : neox_hi ? (int)(threadIdx.x & 63) - rot_chunks : (int)(threadIdx.x & 63);
+    const bool rotates = STYLE == ROPE_IL ? c < rot_chunks : (neox_lo || neox_hi);
+    const int pair0 = STYLE == ROPE_IL ? 4 * c : 8 * (neox_hi ? c - rot_chunks : c);   // first table entry of the chunk
+    const double my_freq = tid < half_rd ? p.inv_freq[tid] : 0.0;
+    const s16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+    const s16x8 wq8 = np.wq ? *reinterpret_cast<const s16x8*>((const short*)np.wq + 8 * c) : zero8;
+    const s16x8 wk8 = np.wk ? *reinterpret_cast<const s16x8*>((const short*)np.wk + 8 * c) : zero8;
+
+    const int tokens = p.B * p.L;
+    int parity = 0;
+    for (int tok = blockIdx.x; tok < tokens; tok += gridDim.x, parity ^= 1) {
+        const int b = tok / p.L, l = tok - b * p.L;
+        const int pos = p.positions[b] + l;
+        const bool row_ok = pos >= 0 && pos < p.Lmax;
+        short* xq = (short*)p.x + (int64_t)tok * p.H * D;
+        const short* xk = (const short*)p.k + (int64_t)tok * p.Hkv * D;
+        const short* xv = (const short*)p.v + (int64_t)tok * p.Hkv * D;
+        const int64_t crow = (int64_t)b * p.c0 + (int64_t)pos * p.c2;   // elements, or bytes into Q8_0 caches
+        for (int u0 = tid; u0 < ((units + kRopeThreads - 1) / kRopeThreads) * kRopeThreads; u0 += UN * kRopeThreads) {
+            s16x8 x[UN];
+            int head[UN];
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const int unit = u0 + u * kRopeThreads;
+                head[u] = unit < units ? unit / G : -1;
+                const int hd = head[u];
+                x[u] = zero8;
+                if (hd >= 0) {
+                    const short* src = hd < p.H ? xq + hd * D : hd < p.H + p.Hkv ? xk + (hd - p.H) * D : xv + (hd - p.H - p.Hkv) * D;
+                    if (hd < p.H || row_ok) x[u] = load_once<STREAM>(reinterpret_cast<const s16x8*>(src + 8 * c));
+                }
+            }
+            if (u0 == tid) {   // the token's table, while its first chunks are on their way; one barrier per token
+                if (tid < half_rd) tab[parity][tid] = table_entry(my_freq, pos);
+                __syncthreads();
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const int hd = head[u];
+                const bool is_q = hd >= 0 && hd < p.H, is_k = hd >= p.H && hd < p.H + p.Hkv;
+                // normalise: every lane takes part in the exchanges, the result is used by q and k heads only
+                float ss = sum_sq8<T>(x[u]);
+#pragma unroll
+                for (int m = 1; m < G; m <<= 1) ss += __shfl_xor(ss, m);
+                const float sc = rsqrtf(ss * np.inv_dim + np.eps);
+                s16x8 a = x[u];
+                if (is_q && np.wq) a = scale8w<T>(a, wq8, sc);
+                if (is_k && np.wk) a = scale8w<T>(a, wk8, sc);
+                // rotate
+                if (STYLE == ROPE_NEOX) {
+                    uint4 mine = __builtin_bit_cast(uint4, a), other;
+                    other.x = __shfl(mine.x, partner); other.y = __shfl(mine.y, partner);
+                    other.z = __shfl(mine.z, partner); other.w = __shfl(mine.w, partner);
+                    const s16x8 o = __builtin_bit_cast(s16x8, other);
+                    if ((is_q || is_k) && rotates) {
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) {
+                            const f32x2 cs = tab[parity][pair0 + j];
+                            const uint32_t pk = neox_lo ? rotate_pair<T>(cs[0], cs[1], a[j], o[j]) : rotate_pair<T>(cs[0], cs[1], o[j], a[j]);
+                            a[j] = (short)(neox_lo ? pk & 0xffffu : pk >> 16);
+                        }
+                    }
+                } else if ((is_q || is_k) && rotates) {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        const f32x2 cs = tab[parity][pair0 + j];
+                        const uint32_t pk = rotate_pair<T>(cs[0], cs[1], a[2 * j], a[2 * j + 1]);
+                        a[2 * j] = (short)(pk & 0xffffu);
+                        a[2 * j + 1] = (short)(pk >> 16);
+                    }
+                }
+                // store
+                if (is_q) {
+                    store_once<STREAM>(reinterpret_cast<s16x8*>(xq + hd * D + 8 * c), a);
+                } else if (hd >= 0 && row_ok) {
+                    const int g = is_k ? hd - p.H : hd - p.H - p.Hkv;
+                    void* cache = is_k ? p.k_cache : p.v_cache;
+                    if (Q8) {
+                        float f[8];
+#pragma unroll
+                        for (int j = 0; j < 8; ++j) f[j] = T::to_float(a[j]);
+                        uint16_t d_bits;
+                        const uint2 q8 = quant8_q8_0(f, d_bits);
+                        store_q8_piece((char*)cache + crow + (int64_t)g * p.c1 + (c >> 2) * 34, 8 * (c & 3), q8, d_bits);
+                    } else {
+                        store_once<STREAM>(reinterpret_cast<s16x8*>((short*)cache + crow + (int64_t)g * p.c1 + 8 * c), a);
+                    }
+                }
+            }
+        }
+    }
+}
+
 static int fill_rope(RopeParams& p, int dtype, int style, int64_t B, int64_t L, int64_t H, int64_t D,
                      int64_t rotary_dim, double freq_base, const char* op) {
     char msg[160];
@@ -400,4 +523,65 @@ MINFER_ATTN_EXPORT int minfer_rope_kv_append_q8_0(int dtype, int style, void* q,
     p.Hkv = (int)Hkv; p.Lmax = (int)Lmax;
     p.c0 = cache_stride_b; p.c1 = cache_stride_h; p.c2 = D / 32 * 34;
     return launch_rope<true, true>(dtype, style, p, (hipStream_t)stream_v);
+}
+
+namespace minfer_attn {
+template <class T, int STYLE, bool Q8>
+static void launch_norm_append_as(const NormRopeParams& np, int D, bool stream_hint, int grid, hipStream_t stream) {
+#define MINFER_NORM_APPEND(G, STREAM) \
+    hipLaunchKernelGGL((rope_norm_append_kernel<T, STYLE, Q8, G, STREAM>), dim3(grid), dim3(kRopeThreads), 0, stream, np)
+    if (D == 128) { if (stream_hint) MINFER_NORM_APPEND(16, true); else MINFER_NORM_APPEND(16, false); }
+    else { if (stream_hint) MINFER_NORM_APPEND(8, true); else MINFER_NORM_APPEND(8, false); }
+#undef MINFER_NORM_APPEND
+}
+}  // namespace minfer_attn
+
+MINFER_ATTN_EXPORT int minfer_rope_kv_append_norm(int dtype, int style, int cache_type, void* q, const void* k, const void* v,
+                                                  const void* wq_norm, const void* wk_norm, double eps,
+                                                  const int32_t* positions, void* k_cache, void* v_cache, int64_t B,
+                                                  int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
+                                                  int64_t cache_stride_b, int64_t cache_stride_h, int64_t cache_stride_row,
+                                                  int64_t rotary_dim, double freq_base, void* stream_v) {
+    clear_error();
+    NormRopeParams np{};
+    RopeParams& p = np.r;
+    if (int rc = fill_rope(p, dtype, style, B, L, Hq, D, rotary_dim, freq_base, "rope_kv_append_norm")) return rc;
+    const bool q8 = cache_type == MINFER_Q8_0;
+    if (!q8 && cache_type != dtype)
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: cache_type must be the activations' dtype or MINFER_Q8_0");
+    if (!q || !k || !v || !positions || !k_cache || !v_cache) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: null pointer");
+    if (!(eps >= 0.0)) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: eps must be non-negative");
+    if (Hkv <= 0 || Hkv > 65535 || Lmax < 0 || Lmax > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: bad n_kv_heads or Lmax");
+    if (D != 64 && D != 128) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: head_dim must be 64 or 128");
+    if (!vector_ok(style, D, rotary_dim))
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: rotary_dim must be a multiple of 8 (interleaved) or 16 (NeoX)");
+    if (!aligned16(q) || !aligned16(k) || !aligned16(v) || (wq_norm && !aligned16(wq_norm)) || (wk_norm && !aligned16(wk_norm)))
+        return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: q, k, v and the norm weights must be 16-byte aligned");
+    if (q8) {
+        if (((uintptr_t)k_cache | (uintptr_t)v_cache) & 1u) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: Q8_0 caches must be 2-byte aligned");
+        if (cache_stride_b % 2 || cache_stride_h % 2 || cache_stride_b < 0 || cache_stride_h < 0 || cache_stride_row != D / 32 * 34)
+            return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: Q8_0 cache strides are even byte counts, rows dense (D/32 * 34 bytes)");
+    } else {
+        if (!aligned16(k_cache) || !aligned16(v_cache)) return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: caches must be 16-byte aligned");
+        if (cache_stride_b % 8 || cache_stride_h % 8 || cache_stride_row % 8 || cache_stride_b < 0 || cache_stride_h < 0 || cache_stride_row < 0)
+            return fail(MINFER_ATTN_EINVAL, "rope_kv_append_norm: cache strides must be non-negative multiples of 8 elements");
+    }
+    if (B == 0 || L == 0) return MINFER_ATTN_OK;
+    p.x = q; p.k = k; p.v = v; p.k_cache = k_cache; p.v_cache = v_cache; p.positions = positions;
+    p.Hkv = (int)Hkv; p.Lmax = (int)Lmax;
+    p.c0 = cache_stride_b; p.c1 = cache_stride_h; p.c2 = cache_stride_row;
+    np.wq = wq_norm; np.wk = wk_norm; np.eps = (float)eps; np.inv_dim = (float)(1.0 / (double)D);
+    const int tokens = p.B * p.L;
+    const int grid = std::min(tokens, 256 * 16);
+    const int64_t touched = (int64_t)tokens * (2 * Hq * D * 2 + Hkv * D * 2 * (q8 ? 3 : 4));   // q in place (whole heads), k, v, cache rows
+    const bool hint = touched > kStreamBytes;
+    hipStream_t stream = (hipStream_t)stream_v;
+    if (dtype == MINFER_ATTN_F16) {
+        if (style == ROPE_IL) { if (q8) launch_norm_append_as<F16, ROPE_IL, true>(np, (int)D, hint, grid, stream); else launch_norm_append_as<F16, ROPE_IL, false>(np, (int)D, hint, grid, stream); }
+        else { if (q8) launch_norm_append_as<F16, ROPE_NEOX, true>(np, (int)D, hint, grid, stream); else launch_norm_append_as<F16, ROPE_NEOX, false>(np, (int)D, hint, grid, stream); }
+    } else {
+        if (style == ROPE_IL) { if (q8) launch_norm_append_as<BF16, ROPE_IL, true>(np, (int)D, hint, grid, stream); else launch_norm_append_as<BF16, ROPE_IL, false>(np, (int)D, hint, grid, stream); }
+        else { if (q8) launch_norm_append_as<BF16, ROPE_NEOX, true>(np, (int)D, hint, grid, stream); else launch_norm_append_as<BF16, ROPE_NEOX, false>(np, (int)D, hint, grid, stream); }
+    }
+    return check_launch("rope_norm_append_kernel");
 }

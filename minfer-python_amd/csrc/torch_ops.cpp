@@ -296,6 +296,49 @@ void rope_kv_append_hip(int64_t style, int64_t rotary_dim, double freq_base,
              "rope_kv_append");
 }
 
+// The same producer with the optional per-head normalisation of q and k in front of the rotation
+// (reference: src/minfer/core.py:224-230: rmsnorm(q), rmsnorm(k), then the two rope calls).
+void rope_kv_append_norm_hip(int64_t style, int64_t rotary_dim, double freq_base, double eps,
+                             Tensor& q,                 // [B, L, n_heads, head_dim], normalised and rotated in place
+                             const Tensor& k,           // [B, L, n_kv_heads, head_dim]
+                             const Tensor& v,           // [B, L, n_kv_heads, head_dim]
+                             const Tensor& wq_norm,     // [head_dim]
+                             const Tensor& wk_norm,     // [head_dim]
+                             const Tensor& positions,   // [B] int32
+                             Tensor& k_cache,           // [B, n_kv_heads, Lmax, head_dim] (or Q8_0 bytes)
+                             Tensor& v_cache) {
+    STD_TORCH_CHECK(on_gpu(q) && on_gpu(k) && on_gpu(v) && on_gpu(wq_norm) && on_gpu(wk_norm) && on_gpu(positions) &&
+                    on_gpu(k_cache) && on_gpu(v_cache), "rope_kv_append_norm: all tensors must be on the GPU");
+    STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && k_cache.dim() == 4 && v_cache.dim() == 4 &&
+                    positions.dim() == 1 && wq_norm.dim() == 1 && wk_norm.dim() == 1,
+                    "rope_kv_append_norm: q, k, v and the caches must be 4-D, positions and the norm weights 1-D");
+    STD_TORCH_CHECK(q.is_contiguous() && k.is_contiguous() && v.is_contiguous() && wq_norm.is_contiguous() && wk_norm.is_contiguous(),
+                    "rope_kv_append_norm: q, k, v and the norm weights must be contiguous");
+    STD_TORCH_CHECK(style == MINFER_ROPE_INTERLEAVED || style == MINFER_ROPE_NEOX, "rope_kv_append_norm: style must be 0 (interleaved) or 1 (NeoX)");
+    const bool q8 = k_cache.scalar_type() == ScalarType::Byte;
+    const int dtype = dtype_code(q, k, v, q8 ? q : k_cache, "rope_kv_append_norm");
+    STD_TORCH_CHECK(wq_norm.scalar_type() == q.scalar_type() && wk_norm.scalar_type() == q.scalar_type(),
+                    "rope_kv_append_norm: norm weights must have q's dtype");
+    STD_TORCH_CHECK(v_cache.scalar_type() == k_cache.scalar_type(), "rope_kv_append_norm: caches must share q's dtype, or both be uint8 (Q8_0)");
+    STD_TORCH_CHECK(positions.scalar_type() == ScalarType::Int && positions.is_contiguous(), "rope_kv_append_norm: positions must be contiguous int32");
+    STD_TORCH_CHECK(k.sizes().equals(v.sizes()) && k_cache.sizes().equals(v_cache.sizes()), "rope_kv_append_norm: k/v or cache shapes differ");
+    STD_TORCH_CHECK(k_cache.stride(-1) == 1 && v_cache.stride(-1) == 1 && k_cache.stride(0) == v_cache.stride(0) &&
+                    k_cache.stride(1) == v_cache.stride(1) && k_cache.stride(2) == v_cache.stride(2),
+                    "rope_kv_append_norm: caches must be contiguous in head_dim and share strides");
+    STD_TORCH_CHECK(q.size(0) == k.size(0) && q.size(1) == k.size(1) && q.size(3) == k.size(3) && q.size(0) == k_cache.size(0) &&
+                    k.size(2) == k_cache.size(1) && positions.size(0) == q.size(0) && wq_norm.size(0) == q.size(3) &&
+                    wk_norm.size(0) == q.size(3) && k_cache.size(3) == (q8 ? q.size(3) / 32 * 34 : q.size(3)),
+                    "rope_kv_append_norm: expected q [B,L,Hq,D], k/v [B,L,Hkv,D], weights [D], caches [B,Hkv,Lmax,D] (or [B,Hkv,Lmax,D/32*34] bytes), positions [B]");
+    STD_TORCH_CHECK(rotary_dim <= q.size(3), "rope_kv_append_norm: rotary_dim exceeds head_dim");
+    check_rc(minfer_rope_kv_append_norm(dtype, (int)style, q8 ? MINFER_Q8_0 : dtype, q.mutable_data_ptr(), k.const_data_ptr(),
+                                        v.const_data_ptr(), wq_norm.const_data_ptr(), wk_norm.const_data_ptr(), eps,
+                                        static_cast<const int32_t*>(positions.const_data_ptr()), k_cache.mutable_data_ptr(),
+                                        v_cache.mutable_data_ptr(), q.size(0), q.size(1), q.size(2), k.size(2), q.size(3),
+                                        k_cache.size(2), k_cache.stride(0), k_cache.stride(1), k_cache.stride(2), rotary_dim,
+                                        freq_base, current_stream()),
+             "rope_kv_append_norm");
+}
+
 // Same signature, argument meaning and checks as the reference's rmsnorm_cuda
 // (reference: src/minfer/kernels/torch_ext/csrc/cuda/rmsnorm/op.cuh:20-70); bfloat16 is admitted as well.
 void rmsnorm_hip(double eps,
@@ -372,6 +415,7 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
     const Tensor* ws[3] = {&wq, &wk, &wv};
     Tensor* outs[3] = {&q_out, &k_out, &v_out};
     const char* names[3] = {"qkv: q", "qkv: k", "qkv: v"};
+    bool all_nk = true;
     for (int i = 0; i < 3; ++i) {
         const Tensor& w = *ws[i];
         Tensor& o = *outs[i];
@@ -381,6 +425,21 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
         STD_TORCH_CHECK(o.size(0) == x.size(0) && o.size(1) == x.size(1), names[i], ": output must be [B, L, out_dim]");
         const bool nk = w.size(0) == N && w.size(1) == K;
         STD_TORCH_CHECK(nk || (w.size(0) == K && w.size(1) == N), names[i], ": weight must be [out_dim, hidden_dim] (or [hidden_dim, out_dim])");
+        all_nk = all_nk && nk;
+    }
+    if (all_nk) {   // the reference's layout: one launch for the three projections
+        const int64_t Nq = q_out.size(-1), Nk = k_out.size(-1), Nv = v_out.size(-1);
+        check_rc(minfer_qkv(dtype, x.const_data_ptr(), wq.const_data_ptr(), wk.const_data_ptr(), wv.const_data_ptr(),
+                            q_out.mutable_data_ptr(), k_out.mutable_data_ptr(), v_out.mutable_data_ptr(), M, K, Nq, Nk, Nv,
+                            K, K, K, K, Nq, Nk, Nv, stream),
+                 "qkv");
+        return;
+    }
+    for (int i = 0; i < 3; ++i) {
+        const Tensor& w = *ws[i];
+        Tensor& o = *outs[i];
+        const int64_t N = o.size(-1);
+        const bool nk = w.size(0) == N && w.size(1) == K;
         check_rc(minfer_gemm(dtype, nk ? MINFER_GEMM_B_NK : MINFER_GEMM_B_KN, x.const_data_ptr(), w.const_data_ptr(), nullptr,
                              o.mutable_data_ptr(), M, N, K, K, nk ? K : N, N, N, 1.0, 0.0, stream),
                  names[i]);
@@ -437,6 +496,7 @@ STABLE_TORCH_LIBRARY(minfer, m) {
     m.def("flash_attn_decode(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k_cache, Tensor v_cache, Tensor ctx_lens, Tensor(a!) out) -> ()");
     m.def("flash_attn_varlen(int qtype_int, int qblock_size, int qtype_size, Tensor q, Tensor k, Tensor v, Tensor cu_seqlens, int max_seqlen, Tensor(a!) out) -> ()");
     m.def("rope_kv_append(int style, int rotary_dim, float freq_base, Tensor(a!) q, Tensor k, Tensor v, Tensor positions, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
+    m.def("rope_kv_append_norm(int style, int rotary_dim, float freq_base, float eps, Tensor(a!) q, Tensor k, Tensor v, Tensor wq_norm, Tensor wk_norm, Tensor positions, Tensor(b!) k_cache, Tensor(c!) v_cache) -> ()");
 }
 
 STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-key name for ROCm devices too
@@ -451,6 +511,7 @@ STABLE_TORCH_LIBRARY_IMPL(minfer, CUDA, m) {  // "CUDA" is PyTorch's dispatch-ke
     m.impl("il_rope", TORCH_BOX(&il_rope_hip));
     m.impl("neox_rope", TORCH_BOX(&neox_rope_hip));
     m.impl("rope_kv_append", TORCH_BOX(&rope_kv_append_hip));
+    m.impl("rope_kv_append_norm", TORCH_BOX(&rope_kv_append_norm_hip));
 }
 
 }  // namespace minfer

@@ -9,5 +9,5 @@ except ImportError as e:  # pragma: no cover
         "(hipcc, gfx950) first"
     ) from e
 from .ops import (flash_attn, flash_attn_decode, flash_attn_varlen, gemm, il_rope, neox_rope,  # noqa: E402,F401
-                  qkv, rmsnorm, rope_kv_append)
+                  qkv, rmsnorm, rope_kv_append, rope_kv_append_norm)
 from .ops import dequant as _dequant, quant as _quant  # noqa: E402,F401  (reference: torch_ext/__init__.py:2)

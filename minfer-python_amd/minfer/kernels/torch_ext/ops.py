@@ -171,6 +171,38 @@ def _(style, rotary_dim, freq_base, q, k, v, positions, k_cache, v_cache):
     torch._check(rotary_dim <= q.size(3))
 
 
+def rope_kv_append_norm(
+    style: int,
+    rotary_dim: int,
+    freq_base: float,
+    eps: float,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    wq_norm: torch.Tensor,
+    wk_norm: torch.Tensor,
+    positions: torch.Tensor,
+    k_cache: torch.Tensor,
+    v_cache: torch.Tensor,
+):
+    """rope_kv_append with the per-head RMS normalisation of q (weight wq_norm [D]) and k (wk_norm [D]) in front of
+    the rotation: equals rmsnorm(q), rmsnorm(k), rope_kv_append in one pass (the reference model's optional q/k norm)."""
+    return torch.ops.minfer.rope_kv_append_norm.default(style, rotary_dim, freq_base, eps, q, k, v, wq_norm, wk_norm,
+                                                        positions, k_cache, v_cache)
+
+
+@torch.library.register_fake("minfer::rope_kv_append_norm")
+def _(style, rotary_dim, freq_base, eps, q, k, v, wq_norm, wk_norm, positions, k_cache, v_cache):
+    torch._check(q.dtype in _ACT_DTYPES)
+    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and wq_norm.dtype == q.dtype and wk_norm.dtype == q.dtype)
+    torch._check(k_cache.dtype in (q.dtype, torch.uint8) and v_cache.dtype == k_cache.dtype)
+    torch._check(positions.dtype == torch.int32)
+    torch._check(q.device.type == "cuda")
+    torch._check(q.dim() == 4 and k.dim() == 4 and v.dim() == 4 and k_cache.dim() == 4 and v_cache.dim() == 4)
+    torch._check(wq_norm.dim() == 1 and wk_norm.dim() == 1)
+    torch._check(rotary_dim <= q.size(3))
+
+
 def rmsnorm(eps: float, input: torch.Tensor, w: torch.Tensor, out: torch.Tensor):
     """RMS normalisation over vectors of length len(w) (the whole hidden dimension, or per head)."""
     return torch.ops.minfer.rmsnorm.default(eps, input, w, out)

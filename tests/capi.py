@@ -52,10 +52,15 @@ def lib():
         L.minfer_rope_kv_append.restype = ctypes.c_int
         L.minfer_rope_kv_append.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
                                             i64, i64, i64, i64, i64, dbl, vp]
+        L.minfer_rope_kv_append_norm.restype = ctypes.c_int
+        L.minfer_rope_kv_append_norm.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, dbl, vp, vp, vp,
+                                                 i64, i64, i64, i64, i64, i64, i64, i64, i64, i64, dbl, vp]
         L.minfer_rmsnorm.restype = ctypes.c_int
         L.minfer_rmsnorm.argtypes = [ctypes.c_int, vp, vp, vp, i64, i64, dbl, vp]
         L.minfer_gemm.restype = ctypes.c_int
         L.minfer_gemm.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, dbl, dbl, vp]
+        L.minfer_qkv.restype = ctypes.c_int
+        L.minfer_qkv.argtypes = [ctypes.c_int, vp, vp, vp, vp, vp, vp, vp] + [i64] * 12 + [vp]
         L.minfer_quant_q8_0.restype = ctypes.c_int
         L.minfer_quant_q8_0.argtypes = [ctypes.c_int, vp, vp, i64, i64, vp]
         L.minfer_dequant_q8_0.restype = ctypes.c_int
@@ -150,6 +155,19 @@ def rope_kv_append(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq
                                        k_cache.stride(2), rotary_dim, freq_base, _stream())
 
 
+def rope_kv_append_norm(style, q, k, v, wq_norm, wk_norm, eps, positions, k_cache, v_cache, rotary_dim, freq_base):
+    """rope_kv_append with per-head RMS normalisation of q and k first (a weight may be None); uint8 caches are Q8_0."""
+    import torch
+    B, L, Hq, D = q.shape
+    cache_type = Q8_0 if k_cache.dtype == torch.uint8 else _dtype_code(q)
+    return lib().minfer_rope_kv_append_norm(_dtype_code(q), style, cache_type, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                            wq_norm.data_ptr() if wq_norm is not None else None,
+                                            wk_norm.data_ptr() if wk_norm is not None else None, eps,
+                                            positions.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(), B, L, Hq,
+                                            k.shape[2], D, k_cache.shape[2], k_cache.stride(0), k_cache.stride(1),
+                                            k_cache.stride(2), rotary_dim, freq_base, _stream())
+
+
 def rmsnorm(x, w, out, eps):
     """RMS normalisation of contiguous x over vectors of length len(w), into out."""
     dim = w.shape[0]
@@ -164,6 +182,15 @@ def gemm(a, b, c, d, alpha, beta, b_layout=GEMM_B_KN):
     return lib().minfer_gemm(_dtype_code(a), b_layout, a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None,
                              d.data_ptr(), M, N, K, a.stride(0), b.stride(0), c.stride(0) if c is not None else N, d.stride(0),
                              alpha, beta, _stream())
+
+
+def qkv(x, wq, wk, wv, q_out, k_out, v_out):
+    """The three projections x [M,K] against weights [N,K] into outputs [M,N], one launch."""
+    M, K = x.shape
+    return lib().minfer_qkv(_dtype_code(x), x.data_ptr(), wq.data_ptr(), wk.data_ptr(), wv.data_ptr(), q_out.data_ptr(),
+                            k_out.data_ptr(), v_out.data_ptr(), M, K, wq.shape[0], wk.shape[0], wv.shape[0], x.stride(0),
+                            wq.stride(0), wk.stride(0), wv.stride(0), q_out.stride(0), k_out.stride(0), v_out.stride(0),
+                            _stream())
 
 
 def quant_q8_0(x, y):

@@ -121,6 +121,34 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
     assert torch.equal(d, out[0])
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,K,Nq,Nk,Nv", [
+    (4096, 4096, 4096, 1024, 1024),    # Llama-3-8B prefill: 256 x 256 tiles, 24 tile columns over three weights
+    (512, 6144, 6144, 1024, 1024),     # the reference test's head shape at a smaller batch: 128 x 128 tiles
+    (300, 256, 200, 72, 136),          # ragged rows, widths that end inside a tile
+    (1, 4096, 4096, 1024, 1024),       # a decode step: the few-row kernel over the three weights' column groups
+    (24, 1024, 5120, 1280, 1288),      # few rows, two column groups per workgroup, a ragged last group
+    (64, 512, 768, 256, 256),          # few-row kernel at its largest row count
+    (33, 50, 17, 17, 9),               # nothing tileable: three plain launches
+])
+def test_qkv_one_launch_equals_three_gemms(dtype, M, K, Nq, Nk, Nv):
+    """minfer_qkv (one grid over the column tiles of the three weights) against minfer_gemm per weight: the same
+    tiles run the same arithmetic, so the results are equal bit for bit; q additionally against the oracle."""
+    g = torch.Generator().manual_seed(M + K + Nq)
+    x = torch.randn(M, K, generator=g).to(dtype).to(DEV)
+    ws = [((1 / K ** 0.5) * torch.randn(n, K, generator=g)).to(dtype).to(DEV) for n in (Nq, Nk, Nv)]
+    outs = [torch.full((M, n), float("nan"), dtype=dtype, device=DEV) for n in (Nq, Nk, Nv)]
+    assert capi.qkv(x, *ws, *outs) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    for w, o, name in zip(ws, outs, "qkv"):
+        ref = torch.full_like(o, float("nan"))
+        assert capi.gemm(x, w, None, ref, 1.0, 0.0, NK) == capi.OK, capi.last_error()
+        torch.cuda.synchronize()
+        assert torch.equal(o, ref), name
+    rows = torch.arange(0, M, max(1, M // 24))
+    assert_close(outs[1][rows], oracle.gemm(x[rows].cpu(), ws[1].cpu(), None, 1.0, 0.0, NK), dtype, "k against the oracle")
+
+
 def test_qkv_op_and_reference_checks(kerns):
     """The QKV recipe of the reference's test at a smaller batch (test/kernels.py:173-214: hidden 6144, 48 query and
     8 KV heads of 128): x @ W^T for the three weights stored [out, hidden]."""
