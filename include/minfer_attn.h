@@ -251,6 +251,27 @@ int minfer_flash_attn_decode_q8_0(const void* q, const void* k_cache, const void
                                   size_t workspace_bytes, void* stream);
 
 /*
+ * minfer_flash_attn and minfer_flash_attn_varlen with k and v given as rows of Q8_0 blocks (prefill over a quantised
+ * KV cache): q and out are fp16; k, v are [B,Hkv,L] (varlen: [1,Hkv,T]) rows of D/32 blocks, 2-byte aligned, with
+ * st->kv0 and st->kv1 the BYTE strides of their first two dims (even) and st->kv2 = D/32 * 34 (rows dense), so a view of
+ * the first L rows of a longer cache is accepted.  One pass dequantises k and v into the workspace exactly as
+ * minfer_dequant_q8_0 does (every K/V row is read by many query tiles, so it is done once up front), then the fp16
+ * kernel runs: the result is that of minfer_flash_attn / minfer_flash_attn_varlen on the dequantised rows, bit for
+ * bit.  This is what the reference's unused (qtype_int, qblock_size, qtype_size) operator arguments are for
+ * (reference: cuda/flash_attn/op.cuh:22-24); it has no kernel for it.  The workspace holds the mask classification
+ * (dense call only) and the two fp16 copies.
+ */
+size_t minfer_flash_attn_q8_0_workspace_bytes(int64_t B, int64_t Hkv, int64_t L, int64_t D);
+int minfer_flash_attn_q8_0(const void* q, const void* k, const void* v, const uint8_t* mask, void* out,
+                           int64_t B, int64_t Hq, int64_t Hkv, int64_t L, int64_t D,
+                           const minfer_attn_strides* st, void* workspace, size_t workspace_bytes, void* stream);
+size_t minfer_flash_attn_varlen_q8_0_workspace_bytes(int64_t Hkv, int64_t T, int64_t D);
+int minfer_flash_attn_varlen_q8_0(const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                                  int64_t n_seqs, int64_t max_seqlen, void* out, int64_t Hq, int64_t Hkv,
+                                  int64_t T, int64_t D, const minfer_attn_strides* st, void* workspace,
+                                  size_t workspace_bytes, void* stream);
+
+/*
  * minfer_rope_kv_append into Q8_0 caches: q is rotated in place as there; the rotated k and v, rounded to
  * `dtype` as an fp16/bf16 cache would hold them, are quantised as minfer_quant_q8_0 does and written to row
  * positions[b] + l of caches laid out as minfer_flash_attn_decode_q8_0 reads them (cache_stride_b,

@@ -633,3 +633,87 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const 
     if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: problem too large for one launch");
     return dispatch_prefill<MODE_VARLEN>(dtype, D, p, (int)grid, stream);
 }
+
+// ------------------------------------------------------------------------------------------------
+// Prefill over K/V given as Q8_0 blocks (the operator's (qtype_int, qblock_size, qtype_size) = (8, 32, 34);
+// reference: the unused leading arguments of flash_attn_cuda, cuda/flash_attn/op.cuh:22-24).  In a prefill every K/V
+// tile is read by every query tile that attends it, so dequantising inside the attention kernel would repeat the work
+// once per query tile; instead one pass turns the rows into fp16 (exactly the values the reference's dequantiser gives,
+// cuda/quants/impls.cuh:121-143) in the caller's workspace, read back from the caches by the fp16 kernel.
+// ------------------------------------------------------------------------------------------------
+namespace minfer_attn {
+static size_t kv_f16_bytes(int64_t B, int64_t Hkv, int64_t L, int64_t D) {
+    return ((size_t)(B * Hkv * L * D * 2) + 255) / 256 * 256;
+}
+static int check_q8_kv(const char* op, int dtype, const void* q, const void* k, const void* v, const void* out, int64_t Hq,
+                       int64_t Hkv, int64_t D, const minfer_attn_strides* st) {
+    char msg[200];
+    auto bad = [&](const char* what) { snprintf(msg, sizeof msg, "%s: %s", op, what); return fail(MINFER_ATTN_EINVAL, msg); };
+    if (dtype != MINFER_ATTN_F16) return bad("q and out must be fp16 over Q8_0 k/v (the dequantiser produces fp16)");
+    if (D != 64 && D != 128) return bad("head_dim must be 64 or 128");
+    if (Hq <= 0 || Hkv <= 0 || Hq % Hkv != 0) return bad("n_heads must be a positive multiple of n_kv_heads");
+    if (!st) return bad("strides is null");
+    if (!q || !k || !v || !out) return bad("q, k, v and out must be non-null");
+    if (!aligned16(q) || !aligned16(out)) return bad("q and out must be 16-byte aligned");
+    if (((uintptr_t)k | (uintptr_t)v) & 1u) return bad("Q8_0 k and v must be 2-byte aligned");
+    const int64_t e[6] = {st->q0, st->q1, st->q2, st->o0, st->o1, st->o2};
+    for (int i = 0; i < 6; ++i)
+        if (e[i] % 8 != 0 || e[i] < 0) return bad("strides of q and out must be non-negative multiples of 8 elements");
+    if (st->kv2 != D / 32 * 34) return bad("Q8_0 rows must be dense (row stride = D/32 * 34 bytes)");
+    if (st->kv0 < 0 || st->kv1 < 0 || st->kv0 % 2 || st->kv1 % 2) return bad("Q8_0 k/v strides must be non-negative even byte counts");
+    return MINFER_ATTN_OK;
+}
+}  // namespace minfer_attn
+
+MINFER_ATTN_EXPORT size_t minfer_flash_attn_q8_0_workspace_bytes(int64_t B, int64_t Hkv, int64_t L, int64_t D) {
+    if (B <= 0 || Hkv <= 0 || L <= 0 || D <= 0) return 256;
+    return cls_bytes(B, L) + 2 * kv_f16_bytes(B, Hkv, L, D);
+}
+
+MINFER_ATTN_EXPORT int minfer_flash_attn_q8_0(const void* q, const void* k, const void* v, const uint8_t* mask, void* out,
+                                              int64_t B, int64_t Hq, int64_t Hkv, int64_t L, int64_t D,
+                                              const minfer_attn_strides* st, void* workspace, size_t workspace_bytes,
+                                              void* stream_v) {
+    clear_error();
+    if (int rc = check_q8_kv("flash_attn_q8_0", MINFER_ATTN_F16, q, k, v, out, Hq, Hkv, D, st)) return rc;
+    if (!mask) return fail(MINFER_ATTN_EINVAL, "flash_attn_q8_0: mask is null");
+    if (B < 0 || L < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_q8_0: negative B or L");
+    if (B == 0 || L == 0) return MINFER_ATTN_OK;
+    if (B * Hkv > 65535) return fail(MINFER_ATTN_EINVAL, "flash_attn_q8_0: B * n_kv_heads > 65535 unsupported");
+    const size_t cls = cls_bytes(B, L), kvb = kv_f16_bytes(B, Hkv, L, D);
+    if (!workspace || workspace_bytes < cls + 2 * kvb || !aligned16(workspace))
+        return fail(MINFER_ATTN_EWORKSPACE, "flash_attn_q8_0: workspace too small or misaligned (see minfer_flash_attn_q8_0_workspace_bytes)");
+    char* ws = (char*)workspace;
+    void* kf = ws + cls;
+    void* vf = ws + cls + kvb;
+    if (int rc = launch_dequant_q8_0_kv(k, v, kf, vf, B, Hkv, L, D, st->kv0, st->kv1, (hipStream_t)stream_v)) return rc;
+    minfer_attn_strides s2 = *st;
+    s2.kv0 = Hkv * L * D; s2.kv1 = L * D; s2.kv2 = D;
+    return minfer_flash_attn(MINFER_ATTN_F16, q, kf, vf, mask, out, B, Hq, Hkv, L, D, &s2, workspace, cls, stream_v);
+}
+
+MINFER_ATTN_EXPORT size_t minfer_flash_attn_varlen_q8_0_workspace_bytes(int64_t Hkv, int64_t T, int64_t D) {
+    if (Hkv <= 0 || T <= 0 || D <= 0) return 256;
+    return 2 * kv_f16_bytes(1, Hkv, T, D);
+}
+
+MINFER_ATTN_EXPORT int minfer_flash_attn_varlen_q8_0(const void* q, const void* k, const void* v, const int32_t* cu_seqlens,
+                                                     int64_t n_seqs, int64_t max_seqlen, void* out, int64_t Hq, int64_t Hkv,
+                                                     int64_t T, int64_t D, const minfer_attn_strides* st, void* workspace,
+                                                     size_t workspace_bytes, void* stream_v) {
+    clear_error();
+    if (int rc = check_q8_kv("flash_attn_varlen_q8_0", MINFER_ATTN_F16, q, k, v, out, Hq, Hkv, D, st)) return rc;
+    if (!cu_seqlens) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen_q8_0: cu_seqlens is null");
+    if (n_seqs < 0 || T < 0 || max_seqlen < 0) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen_q8_0: negative size");
+    if (n_seqs == 0 || T == 0) return MINFER_ATTN_OK;
+    if (Hkv > 65535) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen_q8_0: n_kv_heads > 65535 unsupported");
+    const size_t kvb = kv_f16_bytes(1, Hkv, T, D);
+    if (!workspace || workspace_bytes < 2 * kvb || !aligned16(workspace))
+        return fail(MINFER_ATTN_EWORKSPACE, "flash_attn_varlen_q8_0: workspace too small or misaligned (see minfer_flash_attn_varlen_q8_0_workspace_bytes)");
+    void* kf = workspace;
+    void* vf = (char*)workspace + kvb;
+    if (int rc = launch_dequant_q8_0_kv(k, v, kf, vf, 1, Hkv, T, D, 0, st->kv1, (hipStream_t)stream_v)) return rc;
+    minfer_attn_strides s2 = *st;
+    s2.kv0 = Hkv * T * D; s2.kv1 = T * D; s2.kv2 = D;
+    return minfer_flash_attn_varlen(MINFER_ATTN_F16, q, kf, vf, cu_seqlens, n_seqs, max_seqlen, out, Hq, Hkv, T, D, &s2, stream_v);
+}

@@ -70,6 +70,38 @@ minfer_attn_strides strides_of(const Tensor& q, const Tensor& k, const Tensor& o
 
 }  // namespace
 
+// Prefill over k and v given as Q8_0 blocks: uint8 [B, n_kv_heads, L, HEAD_DIM/32 * 34] (dims 0 and 1 may be strided,
+// e.g. the first L rows of a longer cache), q and out float16.
+static void flash_attn_q8_0(int64_t qblock_size, int64_t qtype_size, const Tensor& q, const Tensor& k, const Tensor& v,
+                            Tensor& mask, Tensor& out) {
+    STD_TORCH_CHECK(qblock_size == MINFER_Q8_0_BLOCK && qtype_size == MINFER_Q8_0_BLOCK_BYTES,
+                    "flash_attn: Q8_0 has qblock_size 32 and qtype_size 34");
+    STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && out.dim() == 4 && mask.dim() == 4,
+                    "flash_attn: q, k, v, mask and out must be 4-D");
+    STD_TORCH_CHECK(q.scalar_type() == ScalarType::Half && out.scalar_type() == ScalarType::Half,
+                    "flash_attn: q and out must be float16 over Q8_0 k/v");
+    STD_TORCH_CHECK(k.scalar_type() == ScalarType::Byte && v.scalar_type() == ScalarType::Byte, "flash_attn: Q8_0 k and v must be uint8");
+    STD_TORCH_CHECK(q.stride(-1) == 1 && k.stride(-1) == 1 && v.stride(-1) == 1 && out.stride(-1) == 1,
+                    "flash_attn: q, k, v and out must be contiguous in their last dimension");
+    STD_TORCH_CHECK(k.stride(0) == v.stride(0) && k.stride(1) == v.stride(1) && k.stride(2) == v.stride(2),
+                    "flash_attn: k and v must share strides");
+    STD_TORCH_CHECK(mask.is_contiguous() && mask.scalar_type() == ScalarType::Bool, "flash_attn: mask must be contiguous bool");
+    STD_TORCH_CHECK(q.sizes().equals(out.sizes()) && k.sizes().equals(v.sizes()), "flash_attn: q/out or k/v shapes differ");
+    const int64_t B = q.size(0), Hq = q.size(1), Hkv = k.size(1), L = q.size(2), D = q.size(3);
+    STD_TORCH_CHECK(D == 128 || D == 64, "flash_attn: head_dim must be 128 or 64");
+    STD_TORCH_CHECK(B == k.size(0) && B == mask.size(0) && mask.size(1) == 1 && L == k.size(2) && L == mask.size(2) &&
+                    L == mask.size(3) && k.size(3) == D / 32 * 34 && k.stride(2) == k.size(3),
+                    "flash_attn: expected q [B,Hq,L,D], Q8_0 k/v [B,Hkv,L,D/32*34] with dense rows, mask [B,1,L,L]");
+    if (B == 0 || L == 0) return;
+    const minfer_attn_strides st = strides_of(q, k, out);   // a byte tensor's strides are byte strides
+    const size_t ws_bytes = minfer_flash_attn_q8_0_workspace_bytes(B, Hkv, L, D);
+    Tensor ws = byte_workspace(q, ws_bytes);
+    check_rc(minfer_flash_attn_q8_0(q.const_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
+                                    static_cast<const uint8_t*>(mask.const_data_ptr()), out.mutable_data_ptr(), B, Hq, Hkv, L, D,
+                                    &st, ws.mutable_data_ptr(), ws_bytes, current_stream()),
+             "flash_attn");
+}
+
 // Same signature, argument meaning and checks as the reference's flash_attn_cuda
 // (reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/op.cuh:21-106); the dtype check
 // also admits bfloat16 and head_dim may be 64 as well as 128.
@@ -79,9 +111,15 @@ void flash_attn_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size,
                     const Tensor& v,   // [B, n_kv_heads, L, HEAD_DIM]
                     Tensor& mask,      // [B, 1, L, L] bool, True = attend
                     Tensor& out) {     // [B, n_heads, L, HEAD_DIM]
-    (void)qtype_int; (void)qblock_size; (void)qtype_size;  // unused by the reference as well
+    // The reference leaves its three leading arguments unused; here (8, 32, 34) announces k and v as Q8_0 blocks,
+    // any other value k and v of q's own type, as the reference's callers pass it (F16 = 1).
     STD_TORCH_CHECK(on_gpu(q) && on_gpu(k) && on_gpu(v) && on_gpu(mask) && on_gpu(out),
                     "flash_attn: all tensors must be on the GPU");
+    if (qtype_int == MINFER_Q8_0) {
+        flash_attn_q8_0(qblock_size, qtype_size, q, k, v, mask, out);
+        return;
+    }
+    STD_TORCH_CHECK(k.scalar_type() != ScalarType::Byte, "flash_attn: byte k/v need qtype_int = 8 (Q8_0)");
     STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && out.dim() == 4 && mask.dim() == 4,
                     "flash_attn: q, k, v, mask and out must be 4-D");
     STD_TORCH_CHECK(q.stride(-1) == 1 && k.stride(-1) == 1 && v.stride(-1) == 1 && out.stride(-1) == 1,
@@ -196,11 +234,39 @@ void flash_attn_varlen_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype
                            const Tensor& cu_seqlens,  // [n_seqs + 1] int32
                            int64_t max_seqlen,
                            Tensor& out) {             // [1, n_heads, T, HEAD_DIM]
-    (void)qtype_int; (void)qblock_size; (void)qtype_size;
     STD_TORCH_CHECK(on_gpu(q) && on_gpu(k) && on_gpu(v) && on_gpu(cu_seqlens) && on_gpu(out),
                     "flash_attn_varlen: all tensors must be on the GPU");
     STD_TORCH_CHECK(q.dim() == 4 && k.dim() == 4 && v.dim() == 4 && out.dim() == 4 && cu_seqlens.dim() == 1,
                     "flash_attn_varlen: q, k, v, out must be 4-D and cu_seqlens 1-D");
+    if (qtype_int == MINFER_Q8_0) {   // k and v as Q8_0 blocks: uint8 [1, n_kv_heads, T, HEAD_DIM/32 * 34], q and out float16
+        STD_TORCH_CHECK(qblock_size == MINFER_Q8_0_BLOCK && qtype_size == MINFER_Q8_0_BLOCK_BYTES,
+                        "flash_attn_varlen: Q8_0 has qblock_size 32 and qtype_size 34");
+        STD_TORCH_CHECK(q.scalar_type() == ScalarType::Half && out.scalar_type() == ScalarType::Half &&
+                        k.scalar_type() == ScalarType::Byte && v.scalar_type() == ScalarType::Byte,
+                        "flash_attn_varlen: over Q8_0 k/v, q and out must be float16 and k, v uint8");
+        STD_TORCH_CHECK(q.stride(-1) == 1 && k.stride(-1) == 1 && v.stride(-1) == 1 && out.stride(-1) == 1 &&
+                        k.stride(1) == v.stride(1) && k.stride(2) == v.stride(2),
+                        "flash_attn_varlen: tensors must be contiguous in their last dimension, k and v share strides");
+        STD_TORCH_CHECK(cu_seqlens.scalar_type() == ScalarType::Int && cu_seqlens.is_contiguous() && cu_seqlens.size(0) >= 1,
+                        "flash_attn_varlen: cu_seqlens must be contiguous int32 with at least one entry");
+        STD_TORCH_CHECK(q.sizes().equals(out.sizes()) && k.sizes().equals(v.sizes()), "flash_attn_varlen: q/out or k/v shapes differ");
+        const int64_t Hq8 = q.size(1), Hkv8 = k.size(1), T8 = q.size(2), D8 = q.size(3);
+        STD_TORCH_CHECK(D8 == 128 || D8 == 64, "flash_attn_varlen: head_dim must be 128 or 64");
+        STD_TORCH_CHECK(q.size(0) == 1 && k.size(0) == 1 && T8 == k.size(2) && k.size(3) == D8 / 32 * 34 && k.stride(2) == k.size(3),
+                        "flash_attn_varlen: expected q [1,Hq,T,D], Q8_0 k/v [1,Hkv,T,D/32*34] with dense rows");
+        const int64_t n8 = cu_seqlens.size(0) - 1;
+        if (n8 == 0 || T8 == 0) return;
+        const minfer_attn_strides st8 = strides_of(q, k, out);
+        const size_t ws_bytes = minfer_flash_attn_varlen_q8_0_workspace_bytes(Hkv8, T8, D8);
+        Tensor ws = byte_workspace(q, ws_bytes);
+        check_rc(minfer_flash_attn_varlen_q8_0(q.const_data_ptr(), k.const_data_ptr(), v.const_data_ptr(),
+                                               static_cast<const int32_t*>(cu_seqlens.const_data_ptr()), n8, max_seqlen,
+                                               out.mutable_data_ptr(), Hq8, Hkv8, T8, D8, &st8, ws.mutable_data_ptr(), ws_bytes,
+                                               current_stream()),
+                 "flash_attn_varlen");
+        return;
+    }
+    STD_TORCH_CHECK(k.scalar_type() != ScalarType::Byte, "flash_attn_varlen: byte k/v need qtype_int = 8 (Q8_0)");
     STD_TORCH_CHECK(q.stride(-1) == 1 && k.stride(-1) == 1 && v.stride(-1) == 1 && out.stride(-1) == 1,
                     "flash_attn_varlen: tensors must be contiguous in head_dim");
     STD_TORCH_CHECK(k.stride(1) == v.stride(1) && k.stride(2) == v.stride(2), "flash_attn_varlen: k and v must share strides");

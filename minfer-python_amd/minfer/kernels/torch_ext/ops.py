@@ -49,14 +49,16 @@ def flash_attn(
     out: torch.Tensor,
 ):
     """Fused GQA attention under a dense bool mask [B,1,L,L] (True = attend).
-    q/out [B,n_heads,L,D], k/v [B,n_kv_heads,L,D], any strides with unit stride on D."""
+    q/out [B,n_heads,L,D], k/v [B,n_kv_heads,L,D], any strides with unit stride on D.  With (qtype_int, qblock_size,
+    qtype_size) = (8, 32, 34), k and v are Q8_0 blocks, uint8 [B,n_kv_heads,L,D/32*34], and q/out float16."""
     return torch.ops.minfer.flash_attn.default(qtype_int, qblock_size, qtype_size, q, k, v, mask, out)
 
 
 @torch.library.register_fake("minfer::flash_attn")
 def _(qtype_int, qblock_size, qtype_size, q, k, v, mask, out):
     torch._check(q.dtype in _ACT_DTYPES)
-    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and out.dtype == q.dtype)
+    kv_dtype = torch.uint8 if qtype_int == _Q8_0 else q.dtype
+    torch._check(k.dtype == kv_dtype and v.dtype == kv_dtype and out.dtype == q.dtype)
     torch._check(mask.dtype == torch.bool)
     torch._check(q.device == k.device == v.device == out.device)
     torch._check(q.device.type == "cuda")
@@ -109,7 +111,8 @@ def flash_attn_varlen(
 @torch.library.register_fake("minfer::flash_attn_varlen")
 def _(qtype_int, qblock_size, qtype_size, q, k, v, cu_seqlens, max_seqlen, out):
     torch._check(q.dtype in _ACT_DTYPES)
-    torch._check(k.dtype == q.dtype and v.dtype == q.dtype and out.dtype == q.dtype)
+    kv_dtype = torch.uint8 if qtype_int == _Q8_0 else q.dtype
+    torch._check(k.dtype == kv_dtype and v.dtype == kv_dtype and out.dtype == q.dtype)
     torch._check(cu_seqlens.dtype == torch.int32)
     torch._check(q.device == k.device == v.device == cu_seqlens.device == out.device)
     torch._check(q.device.type == "cuda")

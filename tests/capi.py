@@ -68,6 +68,14 @@ def lib():
         L.minfer_flash_attn_decode_q8_0.restype = ctypes.c_int
         L.minfer_flash_attn_decode_q8_0.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64,
                                                     ctypes.POINTER(Strides), vp, sz, vp]
+        L.minfer_flash_attn_q8_0_workspace_bytes.restype = sz
+        L.minfer_flash_attn_q8_0_workspace_bytes.argtypes = [i64, i64, i64, i64]
+        L.minfer_flash_attn_q8_0.restype = ctypes.c_int
+        L.minfer_flash_attn_q8_0.argtypes = [vp, vp, vp, vp, vp, i64, i64, i64, i64, i64, ctypes.POINTER(Strides), vp, sz, vp]
+        L.minfer_flash_attn_varlen_q8_0_workspace_bytes.restype = sz
+        L.minfer_flash_attn_varlen_q8_0_workspace_bytes.argtypes = [i64, i64, i64]
+        L.minfer_flash_attn_varlen_q8_0.restype = ctypes.c_int
+        L.minfer_flash_attn_varlen_q8_0.argtypes = [vp, vp, vp, vp, i64, i64, vp, i64, i64, i64, i64, ctypes.POINTER(Strides), vp, sz, vp]
         L.minfer_rope_kv_append_q8_0.restype = ctypes.c_int
         L.minfer_rope_kv_append_q8_0.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, vp, vp, i64, i64, i64, i64,
                                                  i64, i64, i64, i64, i64, dbl, vp]
@@ -217,6 +225,29 @@ def flash_attn_decode_q8_0(q, k_cache, v_cache, ctx_lens, out, workspace=None):
     return lib().minfer_flash_attn_decode_q8_0(q.data_ptr(), k_cache.data_ptr(), v_cache.data_ptr(),
                                                ctx_lens.data_ptr(), out.data_ptr(), B, Hq, Hkv, Lmax, D,
                                                ctypes.byref(st), workspace.data_ptr(), workspace.numel(), _stream())
+
+
+def flash_attn_q8_0(q, k, v, mask, out):
+    """Dense-mask prefill with k, v as Q8_0 blocks, uint8 [B,Hkv,L,D/32*34] (dims 0, 1 may be strided)."""
+    import torch
+    B, Hq, L, D = q.shape
+    need = lib().minfer_flash_attn_q8_0_workspace_bytes(B, k.shape[1], L, D)
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    st = _strides(q, k, out)
+    return lib().minfer_flash_attn_q8_0(q.data_ptr(), k.data_ptr(), v.data_ptr(), mask.data_ptr(), out.data_ptr(), B, Hq,
+                                        k.shape[1], L, D, ctypes.byref(st), ws.data_ptr(), ws.numel(), _stream())
+
+
+def flash_attn_varlen_q8_0(q, k, v, cu_seqlens, max_seqlen, out):
+    """Packed ragged prefill with k, v as Q8_0 blocks, uint8 [1,Hkv,T,D/32*34]."""
+    import torch
+    _, Hq, T, D = q.shape
+    need = lib().minfer_flash_attn_varlen_q8_0_workspace_bytes(k.shape[1], T, D)
+    ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+    st = _strides(q, k, out)
+    return lib().minfer_flash_attn_varlen_q8_0(q.data_ptr(), k.data_ptr(), v.data_ptr(), cu_seqlens.data_ptr(),
+                                               cu_seqlens.numel() - 1, max_seqlen, out.data_ptr(), Hq, k.shape[1], T, D,
+                                               ctypes.byref(st), ws.data_ptr(), ws.numel(), _stream())
 
 
 def rope_kv_append_q8_0(style, q, k, v, positions, k_cache, v_cache, rotary_dim, freq_base):

@@ -223,3 +223,75 @@ def test_append_then_decode_over_q8_caches():
     evq = oracle.quant_q8_0(ev.astype(np.float16).astype(np.float32))
     want = oracle.flash_attn_decode_q8_0(qd, ekq, evq, ctx)
     assert float(np.abs(out.float().cpu().numpy() - want).max()) <= TOL
+
+
+# ------------------------------------------------------------------------------------------------
+# prefill over k, v given as Q8_0 blocks (the operator's (qtype_int, qblock_size, qtype_size) = (8, 32, 34))
+# ------------------------------------------------------------------------------------------------
+def _q8_rows(x):
+    """[..., D] values -> uint8 [..., D/32*34] Q8_0 rows (the oracle's quantiser), and the fp16 values they dequantise to."""
+    yq = torch.from_numpy(oracle.quant_q8_0(x.float()))
+    back = torch.from_numpy(oracle.dequant_q8_0(yq.numpy(), np.float16)).view(x.shape)
+    return yq, back
+
+
+@pytest.mark.parametrize("B,Hq,Hkv,L,D,kind,cache_rows", [
+    (2, 8, 2, 200, 128, "causal", 0),
+    (1, 12, 2, 333, 64, "window", 0),        # n_rep = 6, L not a multiple of anything
+    (2, 8, 4, 130, 128, "causal", 500),      # k, v are the first L rows of longer caches: strided batch and head dims
+    (1, 32, 8, 1024, 128, "causal", 0),
+])
+def test_prefill_over_q8_0_kv(B, Hq, Hkv, L, D, kind, cache_rows):
+    """Equal, bit for bit, to the fp16 operator on the dequantised rows (the same kernel reads the same fp16 values),
+    and within the fp16 attention tolerance of the oracle on those rows."""
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, torch.float16, seed=L + D, scale=1.0)
+    rows_total = max(L, cache_rows)
+    kq_all, k_back = _q8_rows(torch.cat([k, torch.zeros(B, Hkv, rows_total - L, D, dtype=torch.float16)], 2))
+    vq_all, v_back = _q8_rows(torch.cat([v, torch.zeros(B, Hkv, rows_total - L, D, dtype=torch.float16)], 2))
+    kq, vq = kq_all.to(DEV)[:, :, :L], vq_all.to(DEV)[:, :, :L]
+    assert kq.is_contiguous() == (cache_rows == 0)
+    mask = workloads.causal_mask(B, L) if kind == "causal" else workloads.window_mask(B, L, 50)
+    out = torch.full(q.shape, float("nan"), dtype=torch.float16, device=DEV)
+    assert capi.flash_attn_q8_0(q.to(DEV), kq, vq, mask.to(DEV), out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    ref = torch.full_like(out, float("nan"))
+    assert capi.flash_attn(q.to(DEV), k_back[:, :, :L].contiguous().to(DEV), v_back[:, :, :L].contiguous().to(DEV), mask.to(DEV), ref) == capi.OK
+    torch.cuda.synchronize()
+    assert torch.equal(out, ref)
+    want = oracle.flash_attn(q, k_back[:, :, :L], v_back[:, :, :L], mask)
+    assert float((out.float().cpu() - torch.from_numpy(want)).abs().max()) <= TOL
+
+
+def test_varlen_prefill_over_q8_0_kv_and_torch_ops(kerns):
+    from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
+    q8 = GGMLQuantizationType.Q8_0
+    qb, qs = GGML_QUANT_SIZES[q8]
+    qv, kv, vv, cu = workloads.ragged_prefill(seed=4, n_seqs=5, len_lo=1, len_hi=300, Hq=8, Hkv=2)
+    kq, k_back = _q8_rows(kv)
+    vq, v_back = _q8_rows(vv)
+    out = torch.full(qv.shape, float("nan"), dtype=torch.float16, device=DEV)
+    assert capi.flash_attn_varlen_q8_0(qv.to(DEV), kq.to(DEV), vq.to(DEV), cu.to(DEV), 300, out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    want = oracle.flash_attn_varlen(qv, k_back, v_back, cu)
+    assert float((out.float().cpu() - torch.from_numpy(want)).abs().max()) <= TOL
+    # the registered ops take the same tensors with the Q8_0 type triple and give the same bits
+    out2 = torch.zeros_like(out)
+    assert kerns.flash_attn_varlen(q8, qb, qs, qv.to(DEV), kq.to(DEV), vq.to(DEV), cu.to(DEV), 300, out2) is None
+    torch.cuda.synchronize()
+    assert torch.equal(out, out2)
+    B, Hq, Hkv, L, D = 2, 8, 2, 192, 128
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, torch.float16, seed=8, scale=1.0, device=DEV)
+    kq, _ = _q8_rows(k.cpu())
+    vq, _ = _q8_rows(v.cpu())
+    mask = workloads.causal_mask(B, L, device=DEV)
+    a, b = torch.zeros_like(q), torch.zeros_like(q)
+    assert kerns.flash_attn(q8, qb, qs, q, kq.to(DEV), vq.to(DEV), mask, a) is None
+    assert capi.flash_attn_q8_0(q, kq.to(DEV), vq.to(DEV), mask, b) == capi.OK
+    torch.cuda.synchronize()
+    assert torch.equal(a, b)
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(1, 1, 2, q, kq.to(DEV), vq.to(DEV), mask, a)            # byte k/v without the Q8_0 type
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(q8, qb, qs, q.bfloat16(), kq.to(DEV), vq.to(DEV), mask, a.bfloat16())   # q must be float16
+    with pytest.raises(RuntimeError):
+        kerns.flash_attn(q8, qb, qs, q, k, v, mask, a)                           # float k/v with the Q8_0 type
