@@ -89,6 +89,49 @@ __global__ __launch_bounds__(256) void classify_mask_kernel(const uint8_t* __res
     }
 }
 
+// The same for masks whose rows can be read in aligned 16-byte pieces, 64 rows x 256 columns (4 key tiles) per workgroup:
+// a lane takes 16 bytes of one row, the workgroup 16 rows per pass, 4 passes, all requested before any is used.  Four times
+// the workgroups of the general kernel and a quarter of the loads per lane: the pass is latency-bound, not byte-bound
+// (16 MiB at S=4096: 4.4 us instead of 5.1).  grid (ceil(NKT/4), NQT, B).
+__global__ __launch_bounds__(256) void classify_mask_kernel_256(const uint8_t* __restrict__ mask, uint8_t* __restrict__ cls,
+                                                                int L, int NQT, int NKT) {
+    __shared__ uint32_t any_s[4][4], all_s[4][4];
+    const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+    const int strip = blockIdx.x, qt = blockIdx.y, b = blockIdx.z;
+    const uint8_t* mb = mask + (size_t)b * L * L;
+    const int col0 = strip * 256 + (tid & 15) * 16;     // this lane's 16 key columns
+    const int r0 = tid >> 4;                            // row inside a pass of 16 rows
+    uint32_t any_acc = 0u, all_acc = 0x01010101u;
+    if (col0 < L) {
+        uint4 x[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int row = min(qt * 64 + 16 * i + r0, L - 1);
+            x[i] = *reinterpret_cast<const uint4*>(mb + (size_t)row * L + col0);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            any_acc |= x[i].x | x[i].y | x[i].z | x[i].w;
+            all_acc &= x[i].x & x[i].y & x[i].z & x[i].w;
+        }
+    }
+    // lanes 4t..4t+3 (mod 16) cover key tile t of the strip; rows differ across lane / 16 and across waves
+    any_acc |= __shfl_xor(any_acc, 1); any_acc |= __shfl_xor(any_acc, 2);
+    all_acc &= __shfl_xor(all_acc, 1); all_acc &= __shfl_xor(all_acc, 2);
+    any_acc |= __shfl_xor(any_acc, 16); any_acc |= __shfl_xor(any_acc, 32);
+    all_acc &= __shfl_xor(all_acc, 16); all_acc &= __shfl_xor(all_acc, 32);
+    if (lane < 16 && (lane & 3) == 0) { any_s[w][lane >> 2] = any_acc; all_s[w][lane >> 2] = all_acc; }
+    __syncthreads();
+    if (tid < 4) {
+        const int kt = strip * 4 + tid;
+        if (kt < NKT) {
+            const uint32_t a = any_s[0][tid] | any_s[1][tid] | any_s[2][tid] | any_s[3][tid];
+            const uint32_t l = all_s[0][tid] & all_s[1][tid] & all_s[2][tid] & all_s[3][tid];
+            cls[((size_t)b * NQT + qt) * NKT + kt] = (uint8_t)(a == 0u ? TILE_NONE : (l == 0x01010101u ? TILE_ALL : TILE_MIXED));
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------
 // Main kernel
 // ------------------------------------------------------------------------------------------
@@ -138,6 +181,9 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     __shared__ __attribute__((aligned(1024))) char v_lds[2][GEO::TILE_BYTES];
     __shared__ uint32_t tile_list[MODE == MODE_DENSE ? kMaxKeyTiles : 1];
     __shared__ int n_active_s;
+    // A wave's own 32 query rows on their way in (whole rows, copied global->LDS) and its 32 output rows on their way
+    // out (so that a store instruction writes whole rows): no other wave touches a wave's area, so it needs no barrier.
+    __shared__ __attribute__((aligned(1024))) char q_lds[kWaves][32 * GEO::RB];
 
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
     const int h = lane >> 5, l32 = lane & 31;
@@ -205,12 +251,15 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     short* Oh = (short*)p.out + (MODE == MODE_DENSE ? (int64_t)b * p.o0 : 0) + (int64_t)head * p.o1 + (int64_t)seq_lo * p.o2;
     const uint8_t* mrow = MODE == MODE_DENSE ? p.mask + ((size_t)b * p.L + min(qrow, last_row)) * p.L : nullptr;
 
-    // the wave's Q rows are requested now and used after the tile list is built, so that the two latencies overlap
-    s16x8 q_raw[KC];
-    {
-        const short* src = Qh + (int64_t)min(qrow, last_row) * p.q2 + 8 * h;
+    // The wave's Q rows are requested now and used after the tile list is built, so that the two latencies overlap.
+    // They are copied global->LDS as whole rows (RPI rows per instruction, with the K tile's swizzle) and read back as
+    // fragments: fetched straight into fragment registers every instruction would touch 32 rows for 32 bytes each.
+    // Rows past the end of the sequence re-read its last row.
 #pragma unroll
-        for (int c = 0; c < KC; ++c) q_raw[c] = *reinterpret_cast<const s16x8*>(src + 16 * c);
+    for (int j = 0; j < 32 / RPI; ++j) {
+        const int row = j * RPI + lane / G, pg = lane % G;
+        const short* src = Qh + (int64_t)min(q_row0 + row, last_row) * p.q2 + 8 * (pg ^ GEO::swz_k(row));
+        copy16_global_to_lds(src, &q_lds[w][j * RPI * RB]);
     }
 
     // ---- list of key tiles this workgroup visits ---------------------------------------------
@@ -248,11 +297,16 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
     // Q is multiplied by scale*log2(e) once, here, so that the MFMA accumulator of Q K^T is directly
     // the base-2 exponent of the softmax weight (minus the running reference it is initialised with).
-    // (The loads were requested before the tile list was built.)
+    // (The rows were requested before the tile list was built.)
     const float c2 = p.scale_log2;
     s16x8 qf[KC];
+    wait_vmcnt<0>();   // the wave's own rows have landed (nobody else reads them)
+    {
+        const uint32_t qa = lds_addr(&q_lds[w][0]) + l32 * RB;
+        const int sw = GEO::swz_k(l32);
 #pragma unroll
-    for (int c = 0; c < KC; ++c) qf[c] = T::scale8(q_raw[c], c2);
+        for (int c = 0; c < KC; ++c) qf[c] = T::scale8(lds_read_b128(qa + 16 * ((2 * c + h) ^ sw), 0), c2);
+    }
 
     // ---- global -> LDS tile copy ----------------------------------------------------------
     // Instruction j of this wave fills rows (j*kWaves + w)*RPI .. +RPI-1 of the tile; the lane's byte
@@ -366,23 +420,37 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         const int key0 = kt * 64;
 
         // S^T = K Q^T, accumulated on top of -reference: register r of block kb is key 32kb + 8(r/4) + 4h + r%4.
-        // All K fragments are requested before the first MFMA: the LDS latency is paid once per tile.
-        s16x8 ka[KC], kb_[KC];
-#pragma unroll
-        for (int c = 0; c < KC; ++c) {
-            ka[c] = lds_read_b128(k_rd[c], SOFF);
-            kb_[c] = lds_read_b128(k_rd[c], SOFF + 32 * RB);
-        }
-        __builtin_amdgcn_sched_barrier(0);
-        // the accumulators start from -reference (neg_ref, a register block that changes only when the
-        // reference does), so the MFMA output is the exponent relative to the reference
+        // K fragments go through two register buffers of two contraction chunks each (both key blocks): the buffer just
+        // consumed is refilled while the other one feeds the matrix pipe (all sixteen fragments requested up front ran
+        // at the same speed and held 24 registers more).  The accumulators start from -reference (neg_ref, a register
+        // block that changes only when the reference does), so the MFMA output is the exponent relative to the reference.
         f32x16 e_acc[2];
-        e_acc[0] = T::mfma32(ka[0], qf[0], neg_ref);
-        e_acc[1] = T::mfma32(kb_[0], qf[0], neg_ref);
+        {
+            s16x8 kf[2][2][2];   // [buffer][chunk in buffer][key block]
+            auto load_k = [&](int buf, int c0) __attribute__((always_inline)) {
 #pragma unroll
-        for (int c = 1; c < KC; ++c) {
-            e_acc[0] = T::mfma32(ka[c], qf[c], e_acc[0]);
-            e_acc[1] = T::mfma32(kb_[c], qf[c], e_acc[1]);
+                for (int i = 0; i < 2; ++i) {
+                    kf[buf][i][0] = lds_read_b128(k_rd[c0 + i], SOFF);
+                    kf[buf][i][1] = lds_read_b128(k_rd[c0 + i], SOFF + 32 * RB);
+                }
+            };
+            load_k(0, 0);
+            load_k(1, 2);
+#pragma unroll
+            for (int c0 = 0; c0 < KC; c0 += 2) {
+                const int buf = (c0 >> 1) & 1;
+#pragma unroll
+                for (int i = 0; i < 2; ++i) {
+                    if (c0 + i == 0) {
+                        e_acc[0] = T::mfma32(kf[buf][i][0], qf[0], neg_ref);
+                        e_acc[1] = T::mfma32(kf[buf][i][1], qf[0], neg_ref);
+                    } else {
+                        e_acc[0] = T::mfma32(kf[buf][i][0], qf[c0 + i], e_acc[0]);
+                        e_acc[1] = T::mfma32(kf[buf][i][1], qf[c0 + i], e_acc[1]);
+                    }
+                }
+                if (c0 + 4 < KC) load_k(buf, c0 + 4);
+            }
         }
         // first two chunks of V^T fragments: their latency hides behind the max and the first exponentials
         s16x8 va[2][DB];
@@ -502,21 +570,34 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         if (it + 1 < n_active) iteration(std::integral_constant<int, 1>{}, it + 1);
     }
 
-    // ---- epilogue: normalise and store -----------------------------------------------------
+    // ---- epilogue: normalise, transpose through the wave's staging area, store whole rows ---------------
+    // A lane holds 4 consecutive columns of ONE row per register quadruple: stored from the registers, an instruction
+    // would write 16 bytes to each of 32 rows (2.2 us per item for the 16 stores of a wave).  Written to LDS (8 bytes
+    // per lane, granules XOR-swizzled by row) and read back 16 bytes per lane, RPI whole rows per instruction, the same
+    // data leaves in 32/RPI stores of whole rows.
     if (!wave_on) return;
     const float l = sum_across_halves(l_sum);
     const float inv = l > 0.f ? 1.f / l : 0.f;
-    if (qrow < seq_len) {
-        short* orow = Oh + (int64_t)qrow * p.o2;
+    {
+        const uint32_t so = lds_addr(&q_lds[w][0]);
+        typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+        typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                uint2 pk;
+                u32x2 pk;
                 pk.x = T::pack2(o_acc[db][4 * j + 0] * inv, o_acc[db][4 * j + 1] * inv);
                 pk.y = T::pack2(o_acc[db][4 * j + 2] * inv, o_acc[db][4 * j + 3] * inv);
-                *reinterpret_cast<uint2*>(orow + 32 * db + 8 * j + 4 * h) = pk;
+                const int gi = 4 * db + j;   // 16-byte granule of the row: columns 8gi..8gi+7, this lane's half 4h..4h+3
+                *(lds_u32x2*)(uintptr_t)(so + l32 * RB + 16 * (gi ^ (l32 & (G - 1))) + 8 * h) = pk;
             }
+        }
+#pragma unroll
+        for (int i = 0; i < 32 / RPI; ++i) {
+            const int r = i * RPI + lane / G, gi = lane % G;
+            const s16x8 val = lds_read_b128(so + r * RB + 16 * (gi ^ (r & (G - 1))), 0);
+            if (q_row0 + r < seq_len) *reinterpret_cast<s16x8*>(Oh + (int64_t)(q_row0 + r) * p.o2 + 8 * gi) = val;
         }
     }
 }
@@ -602,8 +683,12 @@ MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k
     const int64_t grid = (int64_t)p.NQ * B * Hkv * p.n_hg;
     if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn: problem too large for one launch");
 
-    hipLaunchKernelGGL(classify_mask_kernel, dim3((p.NKT + 15) / 16, p.NQT, (unsigned)B), dim3(256), 0, stream,
-                       mask, (uint8_t*)workspace, p.L, p.NQT, p.NKT, p.mask_vec);
+    if (p.mask_vec)
+        hipLaunchKernelGGL(classify_mask_kernel_256, dim3((p.NKT + 3) / 4, p.NQT, (unsigned)B), dim3(256), 0, stream,
+                           mask, (uint8_t*)workspace, p.L, p.NQT, p.NKT);
+    else
+        hipLaunchKernelGGL(classify_mask_kernel, dim3((p.NKT + 15) / 16, p.NQT, (unsigned)B), dim3(256), 0, stream,
+                           mask, (uint8_t*)workspace, p.L, p.NQT, p.NKT, p.mask_vec);
     if (int rc = check_launch("classify_mask_kernel")) return rc;
     return dispatch_prefill<MODE_DENSE>(dtype, D, p, (int)grid, stream);
 }
