@@ -5,7 +5,8 @@ S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmi
 (4*D*Hq*attended pairs), inputs resident in HBM, every kernel the op launches inside the timed
 region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
 under "decode" with its own HBM roofline (and again over Q8_0 caches under "decode_q8_0"), the steps that feed
-attention under "rope", "rope_kv_append" (into Q8_0 caches: "rope_kv_append_q8_0"), "rmsnorm" and "gemm", and the
+attention under "rope", "rope_kv_append" (into Q8_0 caches: "rope_kv_append_q8_0"; with the per-head q/k norm: "rope_kv_append_norm"),
+"rmsnorm", "gemm" and "qkv", and the
 reference's CPU attention path (torch SDPA in fp32 on the host cores) under "cpu_baseline".  Prints ONE JSON line.
 """
 import argparse
@@ -28,7 +29,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
 # These are figures from those earlier counter runs, not measured in the run that prints them.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels_pmc.md (rocprofv3 --pmc runs of the same workloads; not re-measured by this run)"
-PREFILL_TRAFFIC_BYTES = 107374 * 1024
+PREFILL_TRAFFIC_BYTES = 107531 * 1024
 DECODE_TRAFFIC_BYTES = 1092838 * 1024
 ROPE_TRAFFIC_BYTES = 393312 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
@@ -36,6 +37,8 @@ NORM_TRAFFIC_BYTES = 786659 * 1024          # rmsnorm on [8,4096,6144]
 GEMM_TRAFFIC_BYTES = 230579 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
 DECODE_Q8_TRAFFIC_BYTES = 598453 * 1024     # decode over Q8_0 caches (split + combine)
 APPEND_Q8_TRAFFIC_BYTES = 737585 * 1024     # rope_kv_append into Q8_0 caches
+APPEND_NORM_TRAFFIC_BYTES = 786620 * 1024   # rope_kv_append_norm, the same shape
+QKV_TRAFFIC_BYTES = 377657 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
 
 
 class HipEvents:
@@ -273,6 +276,15 @@ def main():
     a_avg_ms, a_med_ms = ev.time_each(astep, stream, 50)
     abytes = workloads.kv_append_bytes(8, 4096, 32, 8, 128, 128)
     a_gbs = abytes / (a_avg_ms * 1e-3) / 1e9
+    # the same producer with the per-head q/k RMSNorm (Qwen3/Gemma3-style) applied first, in the same launch
+    wqn = torch.ones(128, dtype=torch.float16, device=dev)
+    wkn = torch.ones(128, dtype=torch.float16, device=dev)
+    anstep = lambda: kerns.rope_kv_append_norm(1, 128, 5e5, 1e-6, aq, ak, av, wqn, wkn, apos, akc, avc)
+    for _ in range(100):
+        anstep()
+    torch.cuda.synchronize()
+    an_avg_ms, an_med_ms = ev.time_each(anstep, stream, 50)
+    an_gbs = abytes / (an_avg_ms * 1e-3) / 1e9
     del akc, avc
     akq = torch.zeros(8, 8, 4096, 128 // 32 * 34, dtype=torch.uint8, device=dev)
     avq = torch.zeros_like(akq)
@@ -306,6 +318,22 @@ def main():
     gflops = workloads.gemm_flops(4096, 4096, 4096)
     g_tf = gflops / (g_avg_ms * 1e-3) / 1e12
     del ga, gw, gbias, gout
+    # the QKV projection of the prefill shape, three weight matrices in one launch
+    px = workloads.gemm_input(4096, 4096, 4096, seed=1, device=dev)[0]
+    pwq = workloads.gemm_input(4096, 4096, 4096, seed=2, device=dev)[1].t().contiguous()   # [out, hidden]
+    pwk = pwq[:1024].clone()
+    pwv = pwq[1024:2048].clone()
+    pq = torch.empty(1, 4096, 4096, dtype=torch.float16, device=dev)
+    pk = torch.empty(1, 4096, 1024, dtype=torch.float16, device=dev)
+    pv = torch.empty_like(pk)
+    pstep = lambda: kerns.qkv(qt, qt, qt, qb, qb, qb, qs, qs, qs, px, pwq, pwk, pwv, pq, pk, pv)
+    for _ in range(100):
+        pstep()
+    torch.cuda.synchronize()
+    p_avg_ms, p_med_ms = ev.time_each(pstep, stream, 50)
+    pflops = workloads.gemm_flops(4096, 6144, 4096)
+    p_tf = pflops / (p_avg_ms * 1e-3) / 1e12
+    del px, pwq, pwk, pwv, pq, pk, pv
 
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
@@ -353,6 +381,14 @@ def main():
                              "workload": "NeoX rope(q) in place + rope(k), v appended to the cache: B=8 L=4096 Hq=32 Hkv=8 D=128 fp16, rotary_dim 128, base 5e5",
                              "roofline": {"bound": "hbm", "achieved": a_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a_gbs / PEAK_HBM_GBS,
                                           "traffic": APPEND_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rope_kernel<F16,neox,fused append>", "algorithmic_bytes": abytes}}
+    rec["rope_kv_append_norm"] = {"value": an_gbs, "unit": "GB/s", "ms": an_avg_ms, "median_ms": an_med_ms,
+                                  "workload": "the rope_kv_append workload with per-head RMSNorm of q and k (eps 1e-6) applied before the rotation, one launch",
+                                  "roofline": {"bound": "hbm", "achieved": an_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": an_gbs / PEAK_HBM_GBS,
+                                               "traffic": APPEND_NORM_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rope_norm_append_kernel<F16,neox>", "algorithmic_bytes": abytes}}
+    rec["qkv"] = {"value": p_tf, "unit": "TFLOP/s", "ms": p_avg_ms, "median_ms": p_med_ms,
+                  "workload": "q,k,v = x wq^T, x wk^T, x wv^T in one launch: x [1,4096,4096], wq [4096,4096], wk and wv [1024,4096] fp16 (Llama-3-8B prefill)",
+                  "roofline": {"bound": "mfma", "achieved": p_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": p_tf / PEAK_MFMA_TFLOPS,
+                               "traffic": QKV_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_kernel<F16,[N,K],256x256,grouped>", "algorithmic_flops": pflops}}
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,

@@ -148,6 +148,25 @@ def rope_kv_append_q8_0(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def rope_kv_append_norm(backend: str, which: str, workload: str, repeat: int):
+    """rope_kv_append at the same shape with the per-head RMSNorm of q and k in front (the models whose attention
+    normalises q and k per head: reference src/minfer/core.py:134-141); `ref` is the three separate steps."""
+    kerns = KernelBackend(backend)
+    q, k, v, pos, kc, vc = workloads.kv_append(device="cuda", B=8, L=4096)
+    wq = torch.ones(128, dtype=q.dtype, device="cuda")
+    wk = torch.ones(128, dtype=q.dtype, device="cuda")
+    if which == "minfer":
+        fn = lambda: kerns.rope_kv_append_norm(1, 128, 5e5, 1e-6, q, k, v, wq, wk, pos, kc, vc)
+    else:
+        def fn():
+            kerns.rmsnorm(1e-6, q, wq, q)
+            kerns.rmsnorm(1e-6, k, wk, k)
+            kerns.rope_kv_append(1, 128, 5e5, q, k, v, pos, kc, vc)
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def quant(backend: str, which: str, workload: str, repeat: int):
     """The reference test's larger shape (reference: test/kernels.py:25): fp32 [16384, 6144] into Q8_0 rows and back."""
     kerns = KernelBackend(backend)
@@ -184,6 +203,27 @@ def gemm(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def qkv(backend: str, which: str, workload: str, repeat: int):
+    """The Llama-3-8B QKV projection of a 4096-token prefill: x [1,4096,4096], wq [4096,4096], wk and wv [1024,4096];
+    `ref` is three separate gemm calls."""
+    kerns = KernelBackend(backend)
+    x, w, _ = workloads.gemm_input(4096, 4096, 4096, device="cuda")
+    wq = w.t().contiguous()
+    wk, wv = wq[:1024].clone(), wq[1024:2048].clone()
+    qo = torch.empty(1, 4096, 4096, dtype=x.dtype, device="cuda")
+    ko = torch.empty(1, 4096, 1024, dtype=x.dtype, device="cuda")
+    vo = torch.empty_like(ko)
+    if which == "minfer":
+        fn = lambda: kerns.qkv(QT, QT, QT, QB, QB, QB, QS, QS, QS, x, wq, wk, wv, qo, ko, vo)
+    else:
+        def fn():
+            for wt, o in ((wq, qo), (wk, ko), (wv, vo)):
+                kerns.gemm(QT, QB, QS, 1.0, 0.0, x, wt, o, o)
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def copy(backend: str, which: str, workload: str, repeat: int):
     """A plain device-to-device copy of 1 GiB: the known-size kernel that HBM byte counters
     (FETCH_SIZE / WRITE_SIZE) are calibrated against."""
@@ -197,7 +237,7 @@ def copy(backend: str, which: str, workload: str, repeat: int):
 if __name__ == "__main__":
     KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
                "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "il_rope": il_rope, "rope_kv_append": rope_kv_append,
-               "rope_kv_append_q8_0": rope_kv_append_q8_0, "quant": quant, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
+               "rope_kv_append_q8_0": rope_kv_append_q8_0, "rope_kv_append_norm": rope_kv_append_norm, "qkv": qkv, "quant": quant, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)
