@@ -239,7 +239,8 @@ int minfer_dequant_q8_0(int dst_dtype, const void* x, void* y, int64_t n_rows, i
  * st->o0, o1; k_cache and v_cache are [B,Hkv,Lmax] rows of D/32 blocks, 2-byte aligned, with st->kv0 and
  * st->kv1 the BYTE strides of their first two dims (even) and st->kv2 = D/32 * 34 (rows are dense).  The kernel
  * reads whole aligned 16-byte pieces, so up to 15 bytes on either side of a (sequence, head)'s rows, inside the
- * same 16-byte lines, are read and ignored.  Every
+ * same 16-byte lines, are read and ignored (an aligned 16-byte line never straddles a page, so those bytes lie in pages
+ * that hold bytes of the cache itself and the read cannot fault).  Every
  * block is dequantised to fp16 exactly as minfer_dequant_q8_0 does and the result is that of
  * minfer_flash_attn_decode on the dequantised cache; workspace as for minfer_flash_attn_decode.  This is what
  * the reference's unused (qtype_int, qblock_size, qtype_size) operator arguments are for (reference:

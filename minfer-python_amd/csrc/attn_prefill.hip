@@ -11,7 +11,15 @@
 // exchange with lane^32.  The exponentiated scores are, without any data movement, the B operand
 // of O^T += V^T P^T; V^T fragments come from LDS transpose reads.  K and V tiles are copied
 // global->LDS directly (no VGPR staging) and double-buffered: the copy of tile t+1 is issued
-// right after the barrier that opens tile t.
+// right after the barrier that opens tile t.  The K fragments of a tile pass through a ring of
+// two register buffers, so the next fragment is requested while the current one feeds its MFMAs.
+//
+// Query rows in, output rows out.  Every wave has a private 8 KiB LDS area.  Its 32 query rows
+// are copied there global->LDS as whole rows (full 128/256-byte lines per request) and read back
+// as MFMA fragments; at the end the normalised output goes through the same area so that the
+// wave stores whole rows as well.  Read straight into fragment layout, a load or store
+// instruction would touch 32 different rows with 16 bytes each.  The area is the wave's own:
+// no barrier is involved.
 //
 // Masking.  The reference operator takes an arbitrary dense bool mask [B,1,L,L]
 // (reference: src/minfer/kernels/torch_ext/csrc/cuda/flash_attn/op.cuh:28).  A pre-pass
