@@ -46,9 +46,24 @@ struct RopeParams {
 };
 
 // The rotated pair, rounded to the element type: low half = cos*x0 - sin*x1, high half = sin*x0 + cos*x1.
+// Each output is one product and one fused multiply-add, written out so that every kernel rounds alike:
+// cos*x0 - sin*x1 = fma(cos, x0, -(sin*x1)), sin*x0 + cos*x1 = fma(cos, x1, sin*x0).
+MA_DEV float fma_of_product(float c, float mine, float s, float other) {
+    float t;
+    {
+#pragma clang fp contract(off)
+        t = s * other;
+    }
+    return __builtin_fmaf(c, mine, t);
+}
 template <class T> MA_DEV uint32_t rotate_pair(float c, float s, short a, short b) {
     const float x0 = T::to_float(a), x1 = T::to_float(b);
-    return T::pack2(c * x0 - s * x1, s * x0 + c * x1);
+    return T::pack2(fma_of_product(c, x0, -s, x1), fma_of_product(c, x1, s, x0));
+}
+// One output of a pair for a lane that holds one element and has fetched the other: signed_s is -sin for the lane
+// with x0, +sin for the lane with x1.
+template <class T> MA_DEV float rotate_one(float c, float signed_s, short mine, short other) {
+    return fma_of_product(c, T::to_float(mine), signed_s, T::to_float(other));
 }
 
 // cos/sin of pos * inv_freq[i]: the product and its reduction to a fraction of a turn are done in fp64
@@ -295,111 +310,175 @@ struct NormRopeParams {
     float eps, inv_dim;
 };
 
+// A lane's value from another lane of its row of 16 (quad permutation, mirror or rotation, chosen by CTRL).
+template <int CTRL> MA_DEV uint32_t row_exchange(uint32_t v) {
+    return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, true);
+}
+// ss summed over the G lanes of a head.  The partners are those of `ss += __shfl_xor(ss, m)`, m = 1, 2, 4, 8 (after
+// the quad steps every lane of a quad holds the same sum, so mirroring the half row or the row reads the same value
+// as the lane m away), the additions therefore the same, at a few cycles each instead of a trip through the LDS.
+template <int G> MA_DEV float sum_over_head(float ss) {
+    ss += __builtin_bit_cast(float, row_exchange<0xB1>(__builtin_bit_cast(uint32_t, ss)));            // lanes 1 0 3 2
+    ss += __builtin_bit_cast(float, row_exchange<0x4E>(__builtin_bit_cast(uint32_t, ss)));            // lanes 2 3 0 1
+    ss += __builtin_bit_cast(float, row_exchange<0x141>(__builtin_bit_cast(uint32_t, ss)));           // half row mirrored
+    if (G == 16) ss += __builtin_bit_cast(float, row_exchange<0x140>(__builtin_bit_cast(uint32_t, ss)));   // row mirrored
+    return ss;
+}
+
 template <class T, int STYLE, bool Q8, int G, bool STREAM>
 __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const NormRopeParams np) {
     const RopeParams& p = np.r;
     __shared__ f32x2 tab[2][kMaxPairs];
+    static_assert(G == 8 || G == 16, "a head is 8 or 16 chunks");
     constexpr int D = 8 * G;
-    constexpr int UN = 4;             // chunks in flight per thread
+    constexpr int UN = 4;             // chunks in flight per thread and batch
     const int tid = threadIdx.x;
     const int half_rd = p.rd >> 1;
     const int heads = p.H + 2 * p.Hkv;
     const int units = heads * G;
+    const int batches = (units + UN * kRopeThreads - 1) / (UN * kRopeThreads);
     const int c = tid & (G - 1);      // the lane's chunk inside its head: elements 8c..8c+7
     const int rot_chunks = STYLE == ROPE_IL ? p.rd >> 3 : p.rd >> 4;   // IL: chunks that rotate; NeoX: chunks per half
     // NeoX: chunk c < rd/16 holds the x0 of pairs 8c.., chunk c + rd/16 their x1
     const bool neox_lo = STYLE == ROPE_NEOX && c < rot_chunks;
     const bool neox_hi = STYLE == ROPE_NEOX && c >= rot_chunks && c < 2 * rot_chunks;
     const int partner = neox_lo ? (int)(threadIdx.x & 63) + rot_chunks : neox_hi ? (int)(threadIdx.x & 63) - rot_chunks : (int)(threadIdx.x & 63);
+    const bool partner_half_row = STYLE == ROPE_NEOX && G == 16 && rot_chunks == 8;   // the partner is the lane 8 further round the row
     const bool rotates = STYLE == ROPE_IL ? c < rot_chunks : (neox_lo || neox_hi);
     const int pair0 = STYLE == ROPE_IL ? 4 * c : 8 * (neox_hi ? c - rot_chunks : c);   // first table entry of the chunk
     const double my_freq = tid < half_rd ? p.inv_freq[tid] : 0.0;
     const s16x8 zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
-    const s16x8 wq8 = np.wq ? *reinterpret_cast<const s16x8*>((const short*)np.wq + 8 * c) : zero8;
-    const s16x8 wk8 = np.wk ? *reinterpret_cast<const s16x8*>((const short*)np.wk + 8 * c) : zero8;
-
+    float wq32[8], wk32[8];           // the lane's share of the two weights
+    {
+        const s16x8 wq8 = np.wq ? *reinterpret_cast<const s16x8*>((const short*)np.wq + 8 * c) : zero8;
+        const s16x8 wk8 = np.wk ? *reinterpret_cast<const s16x8*>((const short*)np.wk + 8 * c) : zero8;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { wq32[j] = T::to_float(wq8[j]); wk32[j] = T::to_float(wk8[j]); }
+    }
     const int tokens = p.B * p.L;
-    int parity = 0;
-    for (int tok = blockIdx.x; tok < tokens; tok += gridDim.x, parity ^= 1) {
+
+    // the chunks of batch `bi` of a token: unit (bi*UN + u)*threads + tid is chunk c of head unit / G
+    auto request = [&](int tok, int bi, s16x8 (&x)[UN]) __attribute__((always_inline)) {
+        const int b = tok / p.L, l = tok - b * p.L;
+        const int pos = p.positions[b] + l;
+        const bool row_ok = pos >= 0 && pos < p.Lmax;
+        const uintptr_t xq = (uintptr_t)((const short*)p.x + (int64_t)tok * p.H * D);
+        const uintptr_t xk = (uintptr_t)((const short*)p.k + (int64_t)tok * p.Hkv * D);
+        const uintptr_t xv = (uintptr_t)((const short*)p.v + (int64_t)tok * p.Hkv * D);
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int unit = (bi * UN + u) * kRopeThreads + tid;
+            const int hd = unit / G;
+            x[u] = zero8;
+            if (unit < units) {
+                const bool from_k = hd >= p.H, from_v = hd >= p.H + p.Hkv;
+                const uintptr_t src = from_v ? xv : from_k ? xk : xq;
+                const int local = hd - (from_v ? p.H + p.Hkv : from_k ? p.H : 0);
+                if (!from_k || row_ok) x[u] = load_once<STREAM>(reinterpret_cast<const s16x8*>((const short*)src + local * D + 8 * c));
+            }
+        }
+    };
+
+    // The work is the sequence of (token, batch) items of this workgroup; the chunks of the next item are requested
+    // before the current one is worked on.
+    int tok = blockIdx.x, bi = 0, parity = 0;
+    if (tok >= tokens) return;
+    s16x8 x[UN], xn[UN];
+    request(tok, 0, x);
+    float cs_c[8], cs_s[8];           // the lane's cos and signed sin: out = cos * mine + sin * partner's (NeoX)
+    while (tok < tokens) {
         const int b = tok / p.L, l = tok - b * p.L;
         const int pos = p.positions[b] + l;
         const bool row_ok = pos >= 0 && pos < p.Lmax;
         short* xq = (short*)p.x + (int64_t)tok * p.H * D;
-        const short* xk = (const short*)p.k + (int64_t)tok * p.Hkv * D;
-        const short* xv = (const short*)p.v + (int64_t)tok * p.Hkv * D;
         const int64_t crow = (int64_t)b * p.c0 + (int64_t)pos * p.c2;   // elements, or bytes into Q8_0 caches
-        for (int u0 = tid; u0 < ((units + kRopeThreads - 1) / kRopeThreads) * kRopeThreads; u0 += UN * kRopeThreads) {
-            s16x8 x[UN];
-            int head[UN];
+        int ntok = tok, nbi = bi + 1;
+        if (nbi == batches) { ntok = tok + gridDim.x; nbi = 0; }
+        if (ntok < tokens) request(ntok, nbi, xn);
+        if (bi == 0) {   // the token's table; one barrier per token (the next token writes the other buffer)
+            if (tid < half_rd) tab[parity][tid] = table_entry(my_freq, pos);
+            __syncthreads();
+            if (rotates) {
 #pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                const int unit = u0 + u * kRopeThreads;
-                head[u] = unit < units ? unit / G : -1;
-                const int hd = head[u];
-                x[u] = zero8;
-                if (hd >= 0) {
-                    const short* src = hd < p.H ? xq + hd * D : hd < p.H + p.Hkv ? xk + (hd - p.H) * D : xv + (hd - p.H - p.Hkv) * D;
-                    if (hd < p.H || row_ok) x[u] = load_once<STREAM>(reinterpret_cast<const s16x8*>(src + 8 * c));
-                }
-            }
-            if (u0 == tid) {   // the token's table, while its first chunks are on their way; one barrier per token
-                if (tid < half_rd) tab[parity][tid] = table_entry(my_freq, pos);
-                __syncthreads();
-            }
-#pragma unroll
-            for (int u = 0; u < UN; ++u) {
-                const int hd = head[u];
-                const bool is_q = hd >= 0 && hd < p.H, is_k = hd >= p.H && hd < p.H + p.Hkv;
-                // normalise: every lane takes part in the exchanges, the result is used by q and k heads only
-                float ss = sum_sq8<T>(x[u]);
-#pragma unroll
-                for (int m = 1; m < G; m <<= 1) ss += __shfl_xor(ss, m);
-                const float sc = rsqrtf(ss * np.inv_dim + np.eps);
-                s16x8 a = x[u];
-                if (is_q && np.wq) a = scale8w<T>(a, wq8, sc);
-                if (is_k && np.wk) a = scale8w<T>(a, wk8, sc);
-                // rotate
-                if (STYLE == ROPE_NEOX) {
-                    uint4 mine = __builtin_bit_cast(uint4, a), other;
-                    other.x = __shfl(mine.x, partner); other.y = __shfl(mine.y, partner);
-                    other.z = __shfl(mine.z, partner); other.w = __shfl(mine.w, partner);
-                    const s16x8 o = __builtin_bit_cast(s16x8, other);
-                    if ((is_q || is_k) && rotates) {
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) {
-                            const f32x2 cs = tab[parity][pair0 + j];
-                            const uint32_t pk = neox_lo ? rotate_pair<T>(cs[0], cs[1], a[j], o[j]) : rotate_pair<T>(cs[0], cs[1], o[j], a[j]);
-                            a[j] = (short)(neox_lo ? pk & 0xffffu : pk >> 16);
-                        }
-                    }
-                } else if ((is_q || is_k) && rotates) {
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {
-                        const f32x2 cs = tab[parity][pair0 + j];
-                        const uint32_t pk = rotate_pair<T>(cs[0], cs[1], a[2 * j], a[2 * j + 1]);
-                        a[2 * j] = (short)(pk & 0xffffu);
-                        a[2 * j + 1] = (short)(pk >> 16);
-                    }
-                }
-                // store
-                if (is_q) {
-                    store_once<STREAM>(reinterpret_cast<s16x8*>(xq + hd * D + 8 * c), a);
-                } else if (hd >= 0 && row_ok) {
-                    const int g = is_k ? hd - p.H : hd - p.H - p.Hkv;
-                    void* cache = is_k ? p.k_cache : p.v_cache;
-                    if (Q8) {
-                        float f[8];
-#pragma unroll
-                        for (int j = 0; j < 8; ++j) f[j] = T::to_float(a[j]);
-                        uint16_t d_bits;
-                        const uint2 q8 = quant8_q8_0(f, d_bits);
-                        store_q8_piece((char*)cache + crow + (int64_t)g * p.c1 + (c >> 2) * 34, 8 * (c & 3), q8, d_bits);
-                    } else {
-                        store_once<STREAM>(reinterpret_cast<s16x8*>((short*)cache + crow + (int64_t)g * p.c1 + 8 * c), a);
-                    }
+                for (int j = 0; j < (STYLE == ROPE_IL ? 4 : 8); ++j) {
+                    const f32x2 e = tab[parity][pair0 + j];
+                    cs_c[j] = e[0];
+                    cs_s[j] = neox_lo ? -e[1] : e[1];
                 }
             }
         }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const int unit = (bi * UN + u) * kRopeThreads + tid;
+            if (__builtin_amdgcn_readfirstlane(unit) >= units) continue;   // units grow with the lane: none of this wave's is real
+            const bool valid = unit < units;
+            const int hd = unit / G;
+            const bool is_q = valid && hd < p.H, is_k = valid && hd >= p.H && hd < p.H + p.Hkv;
+            // normalise: every lane takes part in the exchanges, the result is used by q and k heads only
+            const float ss = sum_over_head<G>(sum_sq8<T>(x[u]));
+            const float sc = rsqrtf(ss * np.inv_dim + np.eps);
+            s16x8 a = x[u];
+            if ((is_q && np.wq) || (is_k && np.wk)) {
+                uint32_t r[4];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float w0 = is_q ? wq32[2 * j] : wk32[2 * j], w1 = is_q ? wq32[2 * j + 1] : wk32[2 * j + 1];
+                    r[j] = T::pack2(T::to_float(a[2 * j]) * w0 * sc, T::to_float(a[2 * j + 1]) * w1 * sc);
+                }
+                uint4 v4; v4.x = r[0]; v4.y = r[1]; v4.z = r[2]; v4.w = r[3];
+                a = __builtin_bit_cast(s16x8, v4);
+            }
+            // rotate
+            if (STYLE == ROPE_NEOX) {
+                const uint4 mine = __builtin_bit_cast(uint4, a);
+                uint4 other;
+                if (partner_half_row) {
+                    other.x = row_exchange<0x128>(mine.x); other.y = row_exchange<0x128>(mine.y);
+                    other.z = row_exchange<0x128>(mine.z); other.w = row_exchange<0x128>(mine.w);
+                } else {
+                    other.x = __shfl(mine.x, partner); other.y = __shfl(mine.y, partner);
+                    other.z = __shfl(mine.z, partner); other.w = __shfl(mine.w, partner);
+                }
+                const s16x8 o = __builtin_bit_cast(s16x8, other);
+                if ((is_q || is_k) && rotates) {
+                    uint32_t r[4];
+#pragma unroll
+                    for (int j = 0; j < 4; ++j)
+                        r[j] = T::pack2(rotate_one<T>(cs_c[2 * j], cs_s[2 * j], a[2 * j], o[2 * j]),
+                                        rotate_one<T>(cs_c[2 * j + 1], cs_s[2 * j + 1], a[2 * j + 1], o[2 * j + 1]));
+                    uint4 v4; v4.x = r[0]; v4.y = r[1]; v4.z = r[2]; v4.w = r[3];
+                    a = __builtin_bit_cast(s16x8, v4);
+                }
+            } else if ((is_q || is_k) && rotates) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint32_t pk = rotate_pair<T>(cs_c[j], cs_s[j], a[2 * j], a[2 * j + 1]);
+                    a[2 * j] = (short)(pk & 0xffffu);
+                    a[2 * j + 1] = (short)(pk >> 16);
+                }
+            }
+            // store
+            if (is_q) {
+                store_once<STREAM>(reinterpret_cast<s16x8*>(xq + hd * D + 8 * c), a);
+            } else if (valid && row_ok) {
+                const int g = is_k ? hd - p.H : hd - p.H - p.Hkv;
+                void* cache = is_k ? p.k_cache : p.v_cache;
+                if (Q8) {
+                    float f[8];
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) f[j] = T::to_float(a[j]);
+                    uint16_t d_bits;
+                    const uint2 q8 = quant8_q8_0(f, d_bits);
+                    store_q8_piece((char*)cache + crow + (int64_t)g * p.c1 + (c >> 2) * 34, 8 * (c & 3), q8, d_bits);
+                } else {
+                    store_once<STREAM>(reinterpret_cast<s16x8*>((short*)cache + crow + (int64_t)g * p.c1 + 8 * c), a);
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) x[u] = xn[u];
+        if (nbi == 0) parity ^= 1;
+        tok = ntok; bi = nbi;
     }
 }
 
