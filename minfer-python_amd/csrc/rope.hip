@@ -356,11 +356,16 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
         for (int j = 0; j < 8; ++j) { wq32[j] = T::to_float(wq8[j]); wk32[j] = T::to_float(wk8[j]); }
     }
     const int tokens = p.B * p.L;
+    const uintptr_t kc_addr = (uintptr_t)p.k_cache, vc_addr = (uintptr_t)p.v_cache;   // chosen per lane by value, not by a table in memory
 
     // the chunks of batch `bi` of a token: unit (bi*UN + u)*threads + tid is chunk c of head unit / G
+    // (the token's position comes back: it is read through the scalar cache, once per token)
     auto request = [&](int tok, int bi, s16x8 (&x)[UN]) __attribute__((always_inline)) {
-        const int b = tok / p.L, l = tok - b * p.L;
-        const int pos = p.positions[b] + l;
+        const int b = __builtin_amdgcn_readfirstlane(tok / p.L), l = tok - b * p.L;
+        // positions is an input nothing writes: read it as constant memory, so that the load is a scalar one and
+        // waiting for it does not wait for the chunk loads in flight
+        typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+        const int pos = *((const_i32_ptr)(uintptr_t)p.positions + b) + l;
         const bool row_ok = pos >= 0 && pos < p.Lmax;
         const uintptr_t xq = (uintptr_t)((const short*)p.x + (int64_t)tok * p.H * D);
         const uintptr_t xk = (uintptr_t)((const short*)p.k + (int64_t)tok * p.Hkv * D);
@@ -368,7 +373,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
             const int unit = (bi * UN + u) * kRopeThreads + tid;
-            const int hd = unit / G;
+            const int hd = (int)((unsigned)unit / G);
             x[u] = zero8;
             if (unit < units) {
                 const bool from_k = hd >= p.H, from_v = hd >= p.H + p.Hkv;
@@ -377,6 +382,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
                 if (!from_k || row_ok) x[u] = load_once<STREAM>(reinterpret_cast<const s16x8*>((const short*)src + local * D + 8 * c));
             }
         }
+        return pos;
     };
 
     // The work is the sequence of (token, batch) items of this workgroup; the chunks of the next item are requested
@@ -384,17 +390,16 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
     int tok = blockIdx.x, bi = 0, parity = 0;
     if (tok >= tokens) return;
     s16x8 x[UN], xn[UN];
-    request(tok, 0, x);
+    int pos = request(tok, 0, x), npos = 0;
     float cs_c[8], cs_s[8];           // the lane's cos and signed sin: out = cos * mine + sin * partner's (NeoX)
     while (tok < tokens) {
-        const int b = tok / p.L, l = tok - b * p.L;
-        const int pos = p.positions[b] + l;
+        const int b = __builtin_amdgcn_readfirstlane(tok / p.L);
         const bool row_ok = pos >= 0 && pos < p.Lmax;
         short* xq = (short*)p.x + (int64_t)tok * p.H * D;
         const int64_t crow = (int64_t)b * p.c0 + (int64_t)pos * p.c2;   // elements, or bytes into Q8_0 caches
         int ntok = tok, nbi = bi + 1;
         if (nbi == batches) { ntok = tok + gridDim.x; nbi = 0; }
-        if (ntok < tokens) request(ntok, nbi, xn);
+        if (ntok < tokens) npos = request(ntok, nbi, xn);
         if (bi == 0) {   // the token's table; one barrier per token (the next token writes the other buffer)
             if (tid < half_rd) tab[parity][tid] = table_entry(my_freq, pos);
             __syncthreads();
@@ -412,7 +417,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
             const int unit = (bi * UN + u) * kRopeThreads + tid;
             if (__builtin_amdgcn_readfirstlane(unit) >= units) continue;   // units grow with the lane: none of this wave's is real
             const bool valid = unit < units;
-            const int hd = unit / G;
+            const int hd = (int)((unsigned)unit / G);
             const bool is_q = valid && hd < p.H, is_k = valid && hd >= p.H && hd < p.H + p.Hkv;
             // normalise: every lane takes part in the exchanges, the result is used by q and k heads only
             const float ss = sum_over_head<G>(sum_sq8<T>(x[u]));
@@ -462,7 +467,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
                 store_once<STREAM>(reinterpret_cast<s16x8*>(xq + hd * D + 8 * c), a);
             } else if (valid && row_ok) {
                 const int g = is_k ? hd - p.H : hd - p.H - p.Hkv;
-                void* cache = is_k ? p.k_cache : p.v_cache;
+                void* cache = (void*)(is_k ? kc_addr : vc_addr);
                 if (Q8) {
                     float f[8];
 #pragma unroll
@@ -478,7 +483,7 @@ __global__ __launch_bounds__(kRopeThreads) void rope_norm_append_kernel(const No
 #pragma unroll
         for (int u = 0; u < UN; ++u) x[u] = xn[u];
         if (nbi == 0) parity ^= 1;
-        tok = ntok; bi = nbi;
+        tok = ntok; bi = nbi; pos = npos;
     }
 }
 
