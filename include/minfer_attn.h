@@ -196,6 +196,20 @@ int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const voi
                 double alpha, double beta, void* stream);
 
 /*
+ * minfer_gemm with a workspace.  A problem of a few dozen rows against a wide weight (a batch of decode steps, a short
+ * prefill chunk) has too few output tiles to occupy the chip; given minfer_gemm_workspace_bytes(M, N, K) bytes of
+ * device memory (16-byte aligned; 0 = this shape does not use any), the K dimension is cut into slices that run as
+ * separate workgroups and meet in the workspace as fp32 partial sums, which a second kernel adds up (alpha, beta and
+ * C applied there, one rounding).  With a null or smaller workspace the call is minfer_gemm.  No counterpart in the
+ * reference, whose gemm_cuda takes no scratch memory (reference: gemm/op.cuh:218-316); same contract for the
+ * workspace as the attention entry points (contents need not be initialised; one per stream).
+ */
+size_t minfer_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int minfer_gemm_ws(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
+                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                   double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The QKV projection in one launch: q_out[M,Nq] = x[M,K] wq^T, k_out[M,Nk] = x wk^T, v_out[M,Nv] = x wv^T, the three
  * weights stored [N, K] (the reference's layout for them), 16-bit operands, fp32 accumulation, one rounding; ld* are
  * row strides in elements.  What the reference's fused qkv operator is meant to be (reference:

@@ -55,6 +55,8 @@ struct GemmParams {
     int64_t lda, ldb, ldc, ldd;   // row strides in elements
     float alpha, beta;
     int tiles_m, tiles_n, per_xcd;
+    int splits;                   // SPLIT instantiations: K is cut into this many slices, one workgroup per (tile, slice)
+    float* part;                  // their fp32 partial products, [splits][M][N]
     GemmGroup grp;                // used by the GROUPED instantiations only
 };
 // Which weight column unit `c` (a tile column or a column group) belongs to, and its index inside that weight.
@@ -68,7 +70,7 @@ MA_DEV int group_of_unit(const GemmGroup& g, int c, int& local) {
 MA_DEV int swz_row_tile(int row) { return (row >> 1) & 7; }        // 128-byte rows, read 32 rows x 16 bytes
 MA_DEV int swz_col_tile(int row) { return (row & 3) << 2; }        // 256-byte rows, read 4 rows x 64 bytes (transposing)
 
-template <class T, bool NT, class SH, bool GROUPED = false>
+template <class T, bool NT, class SH, bool GROUPED = false, bool SPLIT = false>
 __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const GemmParams p) {
     constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB, NB = SH::NB, CA = SH::A_COPIES, CB = SH::B_COPIES;
     __shared__ __attribute__((aligned(1024))) char a_lds[2][SH::A_PANEL];
@@ -79,7 +81,10 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     const int wm = w & 1, wn = w >> 1;   // wave's place in the tile: rows 32*MB*wm .., columns 64*wn ..
 
     // ---- which tile ----------------------------------------------------------------------------------
-    const int t = (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
+    // (SPLIT: consecutive workgroup ids are the K slices of one tile, so the slices of a tile run on different XCDs)
+    const int unit = SPLIT ? (int)blockIdx.x : (int)(blockIdx.x & 7) * p.per_xcd + (int)(blockIdx.x >> 3);
+    const int slice = SPLIT ? unit % p.splits : 0;
+    const int t = SPLIT ? unit / p.splits : unit;
     if (t >= p.tiles_m * p.tiles_n) return;
     // Tiles are numbered down bands of kGroupM tile rows, so that the tiles an XCD runs at one time form a block that
     // shares A row panels as well as B column panels in its L2 (row-major numbering made every XCD read all of B).
@@ -134,7 +139,12 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
             b_dst[j] = sub * kColTile + 4 * (q & 15) * 256;
         }
     }
-    auto issue = [&](int kt, int stage) __attribute__((always_inline)) {
+    // K steps of this workgroup: all of them, or its slice
+    const int kt_all = p.K / kBK;
+    const int kt_first = SPLIT ? (int)((int64_t)slice * kt_all / p.splits) : 0;
+    const int KT = SPLIT ? (int)((int64_t)(slice + 1) * kt_all / p.splits) - kt_first : kt_all;
+    auto issue = [&](int kt_rel, int stage) __attribute__((always_inline)) {
+        const int kt = kt_first + kt_rel;
         const short* abase = Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK;
         const short* bbase = NT ? Bg + (int64_t)n0 * ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * ldb + n0;
 #pragma unroll
@@ -198,7 +208,6 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     // of the next stage's copy has landed; after the barrier it issues the copy of the step after next into the
     // stage just vacated and reads the next step's first fragments, all of which overlaps with the last slice's
     // MFMAs, so the matrix pipe does not drain at step boundaries.
-    const int KT = p.K / kBK;
     s16x8 nf[2][NB], mf[2][MB];
     auto mfmas = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
@@ -243,6 +252,11 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
             for (int j = 0; j < 4; ++j) {
                 const int n = n0 + 32 * NB * wn + 32 * nb + 8 * j + 4 * h;
                 if (n >= N) continue;
+                if (SPLIT) {   // the slice's raw sums; gemm_reduce_kernel adds the slices up and applies alpha, beta and C
+                    const f32x4 raw = {acc[nb][mb][4 * j], acc[nb][mb][4 * j + 1], acc[nb][mb][4 * j + 2], acc[nb][mb][4 * j + 3]};
+                    *reinterpret_cast<f32x4*>(p.part + ((int64_t)slice * p.M + m) * N + n) = raw;
+                    continue;
+                }
                 float v[4];
 #pragma unroll
                 for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[nb][mb][4 * j + e];
@@ -382,6 +396,53 @@ __global__ __launch_bounds__(256) void gemm_plain_kernel(const GemmParams p) {
     }
 }
 
+// D = alpha * (sum of the K slices' partial products) + beta * C, four columns per thread.
+template <class T>
+__global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
+    const int n4 = p.N >> 2;
+    const int64_t total = (int64_t)p.M * n4;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (int64_t)gridDim.x * 256) {
+        const int m = (int)(i / n4), n = 4 * (int)(i % n4);
+        f32x4 sum = *reinterpret_cast<const f32x4*>(p.part + (int64_t)m * p.N + n);
+        for (int sl = 1; sl < p.splits; ++sl) sum += *reinterpret_cast<const f32x4*>(p.part + ((int64_t)sl * p.M + m) * p.N + n);
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
+        if (p.beta != 0.f) {
+            const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+        }
+        uint2 pk;
+        pk.x = T::pack2(v[0], v[1]);
+        pk.y = T::pack2(v[2], v[3]);
+        *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+    }
+}
+
+// How many K slices a problem is cut into when a workspace is at hand: problems whose 128 x 128 tiles would leave most
+// of the chip idle (a few dozen rows against a wide weight), every slice at least 4 steps of 64 long.  1 = no split.
+static int gemm_splits(int64_t M, int64_t N, int64_t K) {
+    if (K % kBK != 0 || N % 8 != 0) return 1;
+    const int64_t tiles = ((M + GemmSmall::BM - 1) / GemmSmall::BM) * ((N + GemmSmall::BN - 1) / GemmSmall::BN);
+    const int64_t kt = K / kBK;
+    if (tiles >= 128 || kt < 8) return 1;
+    return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, kt / 4), 32));
+}
+
+template <class T, bool NT>
+static int launch_split(GemmParams& p, hipStream_t stream) {
+    using SH = GemmSmall;
+    p.tiles_m = (p.M + SH::BM - 1) / SH::BM;
+    p.tiles_n = (p.N + SH::BN - 1) / SH::BN;
+    p.per_xcd = 0;
+    hipLaunchKernelGGL((gemm_kernel<T, NT, SH, false, true>), dim3(p.tiles_m * p.tiles_n * p.splits), dim3(SH::WAVES * 64), 0, stream, p);
+    if (int rc = check_launch("gemm_kernel (K slices)")) return rc;
+    const int grid = (int)std::min<int64_t>(((int64_t)p.M * (p.N / 4) + 255) / 256, 256 * 8);
+    hipLaunchKernelGGL((gemm_reduce_kernel<T>), dim3(grid), dim3(256), 0, stream, p);
+    return check_launch("gemm_reduce_kernel");
+}
+
 template <class T, bool NT, class SH>
 static int launch_tiled(GemmParams& p, hipStream_t stream) {
     p.tiles_m = (p.M + SH::BM - 1) / SH::BM;
@@ -478,9 +539,9 @@ MINFER_ATTN_EXPORT int minfer_qkv(int dtype, const void* x, const void* wq, cons
     return dtype == MINFER_ATTN_F16 ? launch_grouped<F16>(p, 3, stream) : launch_grouped<BF16>(p, 3, stream);
 }
 
-MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
-                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
-                                   double alpha, double beta, void* stream_v) {
+static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
+                     int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                     double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream_v) {
     clear_error();
     if (dtype != MINFER_ATTN_F16 && dtype != MINFER_ATTN_BF16)
         return fail(MINFER_ATTN_EINVAL, "gemm: dtype must be MINFER_ATTN_F16 or MINFER_ATTN_BF16");
@@ -503,9 +564,35 @@ MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const
     hipStream_t stream = (hipStream_t)stream_v;
     // a decode step's few tokens against an [N, K] weight: stream the weight once
     // (up to 32 rows it beats the tiled kernel at every weight size measured, 7-34 us against 40-133 us; with 33-64 rows,
-    // whose fragments are re-read from L2 for every 16 columns, only while the weight is small)
-    if (fast && nt && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))
+    // whose fragments are re-read from L2 for every 16 columns, only while the weight is small and no workspace allows K slices)
+    const int splits = fast && workspace && aligned16(workspace) ? gemm_splits(M, N, K) : 1;
+    const bool can_split = splits > 1 && workspace_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
+    // (with a workspace, K slices of the tiled kernel overtake it from 17 rows on: 32 rows against 4096 x 14336, 28 us against 52)
+    if (fast && nt && (M <= 16 || (!can_split && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))))
         return dtype == MINFER_ATTN_F16 ? launch_skinny<F16>(p, stream) : launch_skinny<BF16>(p, stream);
+    if (can_split) {
+        p.splits = splits; p.part = (float*)workspace;
+        if (dtype == MINFER_ATTN_F16) return nt ? launch_split<F16, true>(p, stream) : launch_split<F16, false>(p, stream);
+        return nt ? launch_split<BF16, true>(p, stream) : launch_split<BF16, false>(p, stream);
+    }
     if (dtype == MINFER_ATTN_F16) return nt ? launch_gemm<F16, true>(p, fast, stream) : launch_gemm<F16, false>(p, fast, stream);
     return nt ? launch_gemm<BF16, true>(p, fast, stream) : launch_gemm<BF16, false>(p, fast, stream);
+}
+
+MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
+                                   int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                                   double alpha, double beta, void* stream_v) {
+    return gemm_impl(dtype, b_layout, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, nullptr, 0, stream_v);
+}
+
+MINFER_ATTN_EXPORT size_t minfer_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
+    const int splits = gemm_splits(M, N, K);
+    return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
+}
+
+MINFER_ATTN_EXPORT int minfer_gemm_ws(int dtype, int b_layout, const void* A, const void* B, const void* C, void* D,
+                                      int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
+                                      double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream_v) {
+    return gemm_impl(dtype, b_layout, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, workspace, workspace_bytes, stream_v);
 }

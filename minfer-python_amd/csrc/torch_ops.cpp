@@ -450,9 +450,12 @@ void gemm_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size, double
     STD_TORCH_CHECK(A.size(0) * A.size(1) == C.size(0) * C.size(1) && C.size(-1) == N, "gemm: C does not have the shape of A B");
     STD_TORCH_CHECK(C.sizes().equals(D.sizes()), "gemm: C and D shapes differ");
     STD_TORCH_CHECK(alpha != 0.0, "gemm: alpha must not be 0");
-    check_rc(minfer_gemm(t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16, kn ? MINFER_GEMM_B_KN : MINFER_GEMM_B_NK,
-                         A.const_data_ptr(), B.const_data_ptr(), C.const_data_ptr(), D.mutable_data_ptr(), M, N, K, K,
-                         kn ? N : K, N, N, alpha, beta, current_stream()),
+    // a few dozen rows against a wide weight run as K slices that meet in a workspace
+    const size_t ws_bytes = minfer_gemm_workspace_bytes(M, N, K);
+    Tensor ws = byte_workspace(A, ws_bytes);
+    check_rc(minfer_gemm_ws(t == ScalarType::Half ? MINFER_ATTN_F16 : MINFER_ATTN_BF16, kn ? MINFER_GEMM_B_KN : MINFER_GEMM_B_NK,
+                            A.const_data_ptr(), B.const_data_ptr(), C.const_data_ptr(), D.mutable_data_ptr(), M, N, K, K,
+                            kn ? N : K, N, N, alpha, beta, ws_bytes ? ws.mutable_data_ptr() : nullptr, ws_bytes, current_stream()),
              "gemm");
 }
 

@@ -116,7 +116,8 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
     assert_close(out[0, rows], oracle.gemm(a[0, rows].cpu(), w.cpu(), bias[0, rows].cpu(), alpha, beta), torch.float16, "op")
     assert torch.allclose((alpha * (a @ w) + beta * bias).float(), out.float(), atol=6e-1)
     d = torch.empty(S, S, dtype=torch.float16, device=DEV)
-    assert capi.gemm(a[0], w, bias[0], d, alpha, beta) == capi.OK
+    ws = torch.empty(max(capi.lib().minfer_gemm_workspace_bytes(S, S, S), 16), dtype=torch.uint8, device=DEV)   # the op brings one too
+    assert capi.gemm_ws(a[0], w, bias[0], d, alpha, beta, ws) == capi.OK
     torch.cuda.synchronize()
     assert torch.equal(d, out[0])
 
@@ -186,3 +187,56 @@ def test_qkv_op_and_reference_checks(kerns):
         kerns.gemm(1, 1, 2, 1.0, 0.0, a, w.float(), bias, out)
     with pytest.raises((RuntimeError, NotImplementedError)):
         kerns.gemm(1, 1, 2, 1.0, 0.0, a.cpu(), w.cpu(), bias.cpu(), out.cpu())
+
+
+# ---- K slices through a workspace (minfer_gemm_ws) -------------------------------------------------------------
+@pytest.mark.parametrize("layout", [KN, NK])
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K,alpha,beta", [
+    (64, 4096, 4096, 1.0, 0.0),      # 32 tiles, 8 slices of 8 steps
+    (100, 1032, 2048, 2.0, 3.0),     # ragged rows and columns, C read by the second kernel
+    (256, 2048, 1024, 0.5, 1.0),     # two tile rows
+    (40, 512, 1984, 1.0, 0.0),       # K steps (31) not a multiple of the slice count
+    (1, 4096, 4096, 1.0, 1.0),       # one row: with [K, N] the sliced tiles, with [N, K] still the few-row kernel
+])
+def test_gemm_k_slices_against_oracle(layout, dtype, M, N, K, alpha, beta):
+    a, b, c = make(M, N, K, layout, dtype, seed=M + N + K)
+    need = capi.lib().minfer_gemm_workspace_bytes(M, N, K)
+    assert need > 0 and need % (4 * M * N) == 0, need
+    exact = oracle.gemm(a.float().numpy(), b.float().numpy(), c.float().numpy(), alpha, beta, layout)
+    da, db, dc = a.to(DEV), b.to(DEV), c.to(DEV)
+    d = torch.zeros(M, N, dtype=dtype, device=DEV)
+    ws = torch.full((need,), 0xFF, dtype=torch.uint8, device=DEV)      # NaN patterns: every slot read must have been written
+    assert capi.gemm_ws(da, db, dc, d, alpha, beta, ws, layout) == capi.OK, capi.last_error()
+    assert_close(d, exact, dtype, "k slices")
+    # a workspace that is too small, or none, is the plain call
+    d2 = torch.zeros_like(d)
+    assert capi.gemm_ws(da, db, dc, d2, alpha, beta, ws[: need // 2], layout) == capi.OK, capi.last_error()
+    d3 = torch.zeros_like(d)
+    assert capi.gemm(da, db, dc, d3, alpha, beta, layout) == capi.OK, capi.last_error()
+    assert torch.equal(d2, d3)
+    assert_close(d2, exact, dtype, "fallback")
+
+
+def test_gemm_workspace_bytes_is_zero_where_tiles_fill_the_chip():
+    L = capi.lib()
+    assert L.minfer_gemm_workspace_bytes(4096, 4096, 4096) == 0
+    assert L.minfer_gemm_workspace_bytes(64, 4096, 100) == 0       # K not a multiple of 64
+    assert L.minfer_gemm_workspace_bytes(64, 4096, 256) == 0       # too few K steps to slice
+    assert L.minfer_gemm_workspace_bytes(0, 4096, 4096) == 0
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_gemm_op_uses_k_slices_and_matches_oracle(dtype):
+    from minfer.kernels import KernelBackend
+    from minfer.const import GGMLQuantizationType, GGML_QUANT_SIZES
+    kerns = KernelBackend("torch_ext")
+    qt = GGMLQuantizationType.F16 if dtype == torch.float16 else GGMLQuantizationType.BF16
+    qb, qs = GGML_QUANT_SIZES[qt]
+    M, N, K = 96, 2048, 4096
+    a, b, c = make(M, N, K, KN, dtype, seed=5)
+    exact = oracle.gemm(a.float().numpy(), b.float().numpy(), c.float().numpy(), 1.0, 1.0, KN)
+    A, Cc = a.view(2, 48, K).to(DEV), c.view(2, 48, N).to(DEV)
+    D = torch.empty_like(Cc)
+    kerns.gemm(qt, qb, qs, 1.0, 1.0, A, b.to(DEV), Cc, D)
+    assert_close(D.view(M, N), exact, dtype, "gemm op, k slices")
