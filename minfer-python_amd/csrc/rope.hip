@@ -119,8 +119,11 @@ __global__ __launch_bounds__(kRopeThreads, FUSED ? 1 : 8) void rope_kernel(const
     };
     auto token_at = [&](int tok) __attribute__((always_inline)) {
         Token k;
-        const int b = tok / p.L, l = tok - b * p.L;
-        k.pos = FUSED ? p.positions[b] + l : p.start_pos + l;
+        const int b = __builtin_amdgcn_readfirstlane(tok / p.L), l = tok - b * p.L;
+        // positions is an input nothing writes: read as constant memory the load is a scalar one, and waiting for it
+        // does not wait for the chunk loads and stores in flight
+        typedef const __attribute__((address_space(4))) int32_t* const_i32_ptr;
+        k.pos = FUSED ? *((const_i32_ptr)(uintptr_t)p.positions + b) + l : p.start_pos + l;
         k.row_ok = !FUSED || (k.pos >= 0 && k.pos < p.Lmax);   // cache row exists
         k.xq = (short*)p.x + (int64_t)tok * p.H * p.D;
         k.xk = FUSED ? (const short*)p.k + (int64_t)tok * p.Hkv * p.D : nullptr;
