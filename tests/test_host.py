@@ -147,6 +147,22 @@ def test_gemm_validation_rejects_before_launch():
     assert gemm(lda=32) == capi.EINVAL and "leading" in capi.last_error()
     assert gemm(N=128, ldd=64) == capi.EINVAL
     assert gemm(M=0) == capi.OK and gemm(N=0) == capi.OK and capi.last_error() == ""
+    # the entry point with a workspace checks the same things first
+    gemm_ws = lambda dtype=capi.F16, layout=0, a=0x1000, b=0x2000, d=0x4000, M=64, N=4096, K=4096, lda=4096, ldd=4096: \
+        L.minfer_gemm_ws(dtype, layout, a, b, None, d, M, N, K, lda, N, N, ldd, 1.0, 0.0, 0x10000, 1 << 30, None)
+    assert gemm_ws(dtype=2) == capi.EINVAL and "dtype" in capi.last_error()
+    assert gemm_ws(a=0) == capi.EINVAL and gemm_ws(lda=64) == capi.EINVAL and gemm_ws(ldd=64) == capi.EINVAL
+    assert gemm_ws(M=0) == capi.OK
+
+
+def test_gemm_workspace_sizes():
+    L = capi.lib()
+    ws = L.minfer_gemm_workspace_bytes
+    assert ws(64, 4096, 4096) == 8 * 64 * 4096 * 4            # 32 tiles of 128 x 128: 8 slices of 8 steps
+    assert ws(256, 4096, 4096) == 4 * 256 * 4096 * 4          # 64 tiles: 4 slices
+    assert ws(100, 14336, 4096) == 2 * 100 * 14336 * 4
+    assert ws(4096, 4096, 4096) == 0 and ws(64, 4096, 256) == 0 and ws(64, 4096, 100) == 0 and ws(64, 4100, 4096) == 0
+    assert ws(0, 4096, 4096) == 0 and ws(-1, 4096, 4096) == 0 and ws(64, 4096, 1 << 40) == 0
 
 
 def test_q8_0_validation_rejects_before_launch():
