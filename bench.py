@@ -6,7 +6,7 @@ S=4096, D=128, fp16, causal dense mask); `value` is its throughput in algorithmi
 region.  The decode workload (B=64, ctx in [512,8192]) is timed in the same run and reported
 under "decode" with its own HBM roofline (and again over Q8_0 caches under "decode_q8_0"), the steps that feed
 attention under "rope", "rope_kv_append" (into Q8_0 caches: "rope_kv_append_q8_0"; with the per-head q/k norm: "rope_kv_append_norm"),
-"rmsnorm", "gemm" and "qkv", and the
+"rmsnorm", "gemm", "qkv" and "gemm_q8_0" (a decode step's projection against a weight of Q8_0 blocks), and the
 reference's CPU attention path (torch SDPA in fp32 on the host cores) under "cpu_baseline".  Prints ONE JSON line.
 """
 import argparse
@@ -334,6 +334,23 @@ def main():
     pflops = workloads.gemm_flops(4096, 6144, 4096)
     p_tf = pflops / (p_avg_ms * 1e-3) / 1e12
     del px, pwq, pwk, pwv, pq, pk, pv
+    # a decode step's projection against a weight kept as Q8_0 blocks (Llama-3-8B FFN up: 14336 x 4096), one token
+    q8 = GGMLQuantizationType.Q8_0
+    q8b, q8s = GGML_QUANT_SIZES[q8]
+    wf = workloads.gemm_input(16, 14336, 4096, seed=3, device=dev)[1].t().contiguous()       # [14336, 4096] fp16
+    wq8 = torch.empty(14336, 4096 // 32 * 34, dtype=torch.uint8, device=dev)
+    kerns._quant(q8, q8b, q8s, wf, wq8)
+    del wf
+    xa = workloads.gemm_input(1, 16, 4096, seed=4, device=dev)[0]                              # [1, 1, 4096]
+    xo = torch.zeros(1, 1, 14336, dtype=torch.float16, device=dev)
+    q8step = lambda: kerns.gemm(q8, q8b, q8s, 1.0, 0.0, xa, wq8, xo, xo)
+    for _ in range(100):
+        q8step()
+    torch.cuda.synchronize()
+    q8_avg_ms, q8_med_ms = ev.time_each(q8step, stream, 50)
+    q8bytes = 14336 * (4096 // 32 * 34) + 4096 * 2 + 14336 * 2
+    q8_gbs = q8bytes / (q8_avg_ms * 1e-3) / 1e9
+    del wq8, xa, xo
 
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
@@ -389,6 +406,10 @@ def main():
                   "workload": "q,k,v = x wq^T, x wk^T, x wv^T in one launch: x [1,4096,4096], wq [4096,4096], wk and wv [1024,4096] fp16 (Llama-3-8B prefill)",
                   "roofline": {"bound": "mfma", "achieved": p_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": p_tf / PEAK_MFMA_TFLOPS,
                                "traffic": QKV_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_kernel<F16,[N,K],256x256,grouped>", "algorithmic_flops": pflops}}
+    rec["gemm_q8_0"] = {"value": q8_gbs, "unit": "GB/s", "ms": q8_avg_ms, "median_ms": q8_med_ms,
+                        "workload": "one token against a weight of Q8_0 blocks: x [1,1,4096] fp16, W uint8 [14336, 4352] (Llama-3-8B FFN up), out fp16",
+                        "roofline": {"bound": "hbm", "achieved": q8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": q8_gbs / PEAK_HBM_GBS,
+                                     "traffic": None, "kernel": "gemm_skinny_q8_kernel<1,1>", "algorithmic_bytes": q8bytes}}
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,

@@ -210,6 +210,22 @@ int minfer_gemm_ws(int dtype, int b_layout, const void* A, const void* B, const 
                    double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream);
 
 /*
+ * The projection against a weight stored as Q8_0 blocks: D[M,N] = alpha * A[M,K] x W^T + beta * C[M,N] with W given as N
+ * dense rows of K/32 blocks of 34 bytes (4-byte aligned), every weight dequantised to fp16 exactly as
+ * minfer_dequant_q8_0 does, fp16 A, C and D, fp32 accumulation, one rounding: the result is that of minfer_gemm
+ * (MINFER_GEMM_B_NK) on the dequantised weight, element for element up to the order of the fp32 sums.  Up to 64 rows of A
+ * and an even number of blocks per weight row, a kernel streams the blocks once (34 bytes per 32 weights instead of
+ * 64: the projections of a decode step) and no workspace is needed; other shapes dequantise the weight into the
+ * workspace (minfer_gemm_q8_0_workspace_bytes) and run the fp16 kernels on it.  This is the case the reference's
+ * gemm_cuda routes to dispatch_quant_abt, whose body is empty (reference: gemm/op.cuh:199-210, 299-312); block format
+ * common/types.hpp:141-146, dequantisation cuda/quants/impls.cuh:121-143.
+ */
+size_t minfer_gemm_q8_0_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int minfer_gemm_q8_0(const void* A, const void* Bq, const void* C, void* D, int64_t M, int64_t N, int64_t K,
+                     int64_t lda, int64_t ldc, int64_t ldd, double alpha, double beta,
+                     void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * The QKV projection in one launch: q_out[M,Nq] = x[M,K] wq^T, k_out[M,Nk] = x wk^T, v_out[M,Nv] = x wv^T, the three
  * weights stored [N, K] (the reference's layout for them), 16-bit operands, fp32 accumulation, one rounding; ld* are
  * row strides in elements.  What the reference's fused qkv operator is meant to be (reference:

@@ -21,6 +21,7 @@
 
 #include "attn_common.h"
 #include "attn_host.h"
+#include "quant_q8.h"
 
 namespace minfer_attn {
 
@@ -380,6 +381,115 @@ static int launch_skinny(const GemmParams& p, hipStream_t stream) {
     return check_launch("gemm_skinny_kernel");
 }
 
+// The few-row kernel over a weight stored as rows of Q8_0 blocks, [N][K/32] blocks of 34 bytes (an fp16 scale and 32
+// int8; reference block format: csrc/common/types.hpp:141-146): every weight is dequantised to fp16 exactly as
+// minfer_dequant_q8_0 does (reference: cuda/quants/impls.cuh:121-143) on its way into the MFMA, so the result is that of
+// the fp16 kernel on the dequantised weight while the launch streams 34 bytes per 32 weights instead of 64.
+// A K step is 128 wide: lane (row n, quad q) owns block 4s + q of its weight row, which is one MFMA A fragment per
+// 8 values, and the activations of the same k for the B operand (64 contiguous bytes of row m).  Blocks start on
+// 2-byte boundaries; a lane reads its block as the nine aligned words that cover it, and whether the block starts on a
+// word or in the middle of one depends only on q (rows are multiples of 4 bytes), so one byte permute per quant word with
+// a per-lane constant selector undoes the shift (dequant8_shifted).  fp16 activations only.
+// The weight loads carry no non-temporal hint, unlike the fp16 kernel's: a 128-byte line of a weight row holds 3.8
+// blocks, so the line a step ends in is the line the next step starts in, and a line loaded with the hint is not kept
+// for that second touch (14336 x 4096 at one row: 31 us with the hint, 17.5 us without).
+template <int MB, int NR>
+__global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_q8_kernel(const GemmParams p) {
+    using T = F16;
+    __shared__ f32x4 part[kSkinnyWaves][NR][MB][64];
+    const int lane = threadIdx.x & 63, w = wave_id();
+    const int l16 = lane & 15, quad = lane >> 4;
+    const int n0 = (int)blockIdx.x * 16 * NR;
+    const int nblk = p.K / 32;                                  // blocks per weight row
+    const int steps = (nblk + 3) / 4, per = (steps + kSkinnyWaves - 1) / kSkinnyWaves;
+    const int s0 = w * per, s1 = min(steps, s0 + per);
+    const bool odd = (quad & 1) != 0;                           // block 4s + q starts 2 bytes past a word boundary
+    const uint32_t sel = odd ? kQ8SelOdd : kQ8SelEven;
+    const char* wrow[NR];
+#pragma unroll
+    for (int nr = 0; nr < NR; ++nr) wrow[nr] = (const char*)p.B + (int64_t)min(n0 + 16 * nr + l16, p.N - 1) * p.ldb;   // ldb in bytes here
+    const short* xrow[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) xrow[mb] = (const short*)p.A + (int64_t)min(16 * mb + l16, p.M - 1) * p.lda;
+    f32x4 acc[NR][MB];
+#pragma unroll
+    for (int nr = 0; nr < NR; ++nr)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[nr][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+    for (int s = s0; s < s1; ++s) {
+        const int blk = 4 * s + quad;
+        const bool real = blk < nblk;                           // K need not be a multiple of 128: the last step may be short
+        const int bc = real ? blk : (quad & 1);               // a block of the same alignment class that exists (nblk is even)
+        uint32_t wq[NR][9];
+#pragma unroll
+        for (int nr = 0; nr < NR; ++nr) {
+            const uint32_t* src = reinterpret_cast<const uint32_t*>(wrow[nr] + (int64_t)bc * 34 - (odd ? 2 : 0));
+            const u32x4 a = *reinterpret_cast<const u32x4*>(src);
+            const u32x4 b = *reinterpret_cast<const u32x4*>(src + 4);
+            wq[nr][0] = a[0]; wq[nr][1] = a[1]; wq[nr][2] = a[2]; wq[nr][3] = a[3];
+            wq[nr][4] = b[0]; wq[nr][5] = b[1]; wq[nr][6] = b[2]; wq[nr][7] = b[3];
+            wq[nr][8] = src[8];
+        }
+        s16x8 x[MB][4];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) x[mb][j] = *reinterpret_cast<const s16x8*>(xrow[mb] + 32 * bc + 8 * j);
+#pragma unroll
+        for (int nr = 0; nr < NR; ++nr) {
+            const uint16_t bits = (uint16_t)(odd ? wq[nr][0] >> 16 : wq[nr][0]);
+            const _Float16 dh = real ? __builtin_bit_cast(_Float16, bits) : (_Float16)0.f;
+            const h16x2 d2 = {dh, dh};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const s16x8 wf = dequant8_shifted(wq[nr][2 * j], wq[nr][2 * j + 1], wq[nr][2 * j + 2], sel, d2);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) acc[nr][mb] = T::mfma16(wf, x[mb][j], acc[nr][mb]);
+            }
+        }
+    }
+#pragma unroll
+    for (int nr = 0; nr < NR; ++nr)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) part[w][nr][mb][lane] = acc[nr][mb];
+    __syncthreads();
+    // wave j adds up block (nr, mb) = (j / MB, j % MB): register r of a lane is n = n0 + 16*nr + 4*quad + r, m = 16*mb + l16
+    if (w >= NR * MB) return;
+    const int nr = w / MB, mb = w - nr * MB;
+    f32x4 sum = part[0][nr][mb][lane];
+#pragma unroll
+    for (int ww = 1; ww < kSkinnyWaves; ++ww) sum += part[ww][nr][mb][lane];
+    const int m = 16 * mb + l16, n = n0 + 16 * nr + 4 * quad;
+    if (m >= p.M || n >= p.N) return;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
+    if (p.beta != 0.f) {
+        const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+    }
+    uint2 pk;
+    pk.x = T::pack2(v[0], v[1]);
+    pk.y = T::pack2(v[2], v[3]);
+    *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+}
+
+static int launch_skinny_q8(const GemmParams& p, hipStream_t stream) {
+    const int mb = (p.M + 15) / 16;
+    // two column groups per workgroup as soon as there is more than one row and the weight is wide enough to leave 160
+    // workgroups: the activations are re-read from L2 for every group of columns, and from 8 rows on they are more bytes than
+    // a group's blocks (14336 columns, 8 / 16 rows: 22.2 -> 18.4 us, 27.1 -> 20.7 us)
+    const bool two = p.M > 1 && p.N >= 160 * 32;
+    const dim3 grid((p.N + (two ? 32 : 16) - 1) / (two ? 32 : 16)), block(kSkinnyWaves * 64);
+#define MINFER_SKINNY_Q8(MB, NR) hipLaunchKernelGGL((gemm_skinny_q8_kernel<MB, NR>), grid, block, 0, stream, p)
+    if (!two) { if (mb == 1) MINFER_SKINNY_Q8(1, 1); else if (mb == 2) MINFER_SKINNY_Q8(2, 1); else if (mb == 3) MINFER_SKINNY_Q8(3, 1); else MINFER_SKINNY_Q8(4, 1); }
+    else { if (mb == 1) MINFER_SKINNY_Q8(1, 2); else if (mb == 2) MINFER_SKINNY_Q8(2, 2); else if (mb == 3) MINFER_SKINNY_Q8(3, 2); else MINFER_SKINNY_Q8(4, 2); }
+#undef MINFER_SKINNY_Q8
+    return check_launch("gemm_skinny_q8_kernel");
+}
+
 // Any shape and alignment: one thread per element of D, fp32 accumulation.  Small or odd problems only.
 template <class T, bool NT>
 __global__ __launch_bounds__(256) void gemm_plain_kernel(const GemmParams p) {
@@ -595,4 +705,50 @@ MINFER_ATTN_EXPORT int minfer_gemm_ws(int dtype, int b_layout, const void* A, co
                                       int64_t M, int64_t N, int64_t K, int64_t lda, int64_t ldb, int64_t ldc, int64_t ldd,
                                       double alpha, double beta, void* workspace, size_t workspace_bytes, void* stream_v) {
     return gemm_impl(dtype, b_layout, A, B, C, D, M, N, K, lda, ldb, ldc, ldd, alpha, beta, workspace, workspace_bytes, stream_v);
+}
+
+// ---- weights stored as Q8_0 blocks ------------------------------------------------------------------------------
+constexpr int64_t kQ8SkinnyRows = 64;    // up to here the kernel that streams the blocks; above, dequantise once and run the tiles
+
+static size_t q8_dequant_bytes(int64_t N, int64_t K) { return ((size_t)N * (size_t)K * 2 + 255) & ~(size_t)255; }
+
+// the streaming kernel takes up to 64 rows and needs weight rows that are multiples of 4 bytes (an even number of blocks)
+static bool q8_streams(int64_t M, int64_t K) { return M <= kQ8SkinnyRows && (K / 32) % 2 == 0; }
+
+MINFER_ATTN_EXPORT size_t minfer_gemm_q8_0_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+    if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
+    if (q8_streams(M, K)) return 0;
+    return q8_dequant_bytes(N, K) + minfer_gemm_workspace_bytes(M, N, K);
+}
+
+MINFER_ATTN_EXPORT int minfer_gemm_q8_0(const void* A, const void* Bq, const void* C, void* D, int64_t M, int64_t N, int64_t K,
+                                        int64_t lda, int64_t ldc, int64_t ldd, double alpha, double beta,
+                                        void* workspace, size_t workspace_bytes, void* stream_v) {
+    clear_error();
+    if (M < 0 || N < 0 || K < 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL)
+        return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: bad M, N or K");
+    if (K % 32 != 0) return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: K must be a multiple of the block size 32");
+    if (!A || !Bq || !D || (beta != 0.0 && !C)) return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: null pointer");
+    if (lda < K || ldd < N || (beta != 0.0 && ldc < N)) return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: a leading dimension is smaller than its row");
+    if (M == 0 || N == 0) return MINFER_ATTN_OK;
+    if (K == 0) return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: K must be positive");
+    hipStream_t stream = (hipStream_t)stream_v;
+    const int64_t row_bytes = K / 32 * 34;
+    if (((uintptr_t)Bq & 3u) != 0) return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: the weight must be 4-byte aligned");
+    if (q8_streams(M, K)) {
+        // the streaming kernel reads aligned words of the weight, 16-byte pieces of A, and stores 8-byte pieces of D
+        if (!aligned16(A) || lda % 8 != 0 || ldc % 4 != 0 || ldd % 4 != 0 || ((uintptr_t)D & 7u) != 0 || ((uintptr_t)C & 7u) != 0 || N % 4 != 0)
+            return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: A must be 16-byte aligned with lda a multiple of 8; C, D 8-byte aligned with strides and N multiples of 4");
+        GemmParams p{};
+        p.A = A; p.B = Bq; p.C = C; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
+        p.lda = lda; p.ldb = row_bytes; p.ldc = ldc; p.ldd = ldd; p.alpha = (float)alpha; p.beta = (float)beta;
+        return launch_skinny_q8(p, stream);
+    }
+    // otherwise: the weight as fp16 in the workspace, then the fp16 kernels on it
+    const size_t deq = q8_dequant_bytes(N, K);
+    if (!workspace || !aligned16(workspace) || workspace_bytes < deq)
+        return fail(MINFER_ATTN_EWORKSPACE, "gemm_q8_0: this shape needs a workspace of N*K*2 bytes (rounded up to 256) for the dequantised weight");
+    if (int rc = minfer_dequant_q8_0(MINFER_ATTN_F16, Bq, workspace, N, K, stream_v)) return rc;
+    return gemm_impl(MINFER_ATTN_F16, MINFER_GEMM_B_NK, A, workspace, C, D, M, N, K, lda, K, ldc, ldd, alpha, beta,
+                     (char*)workspace + deq, workspace_bytes - deq, stream_v);
 }

@@ -435,9 +435,32 @@ void gemm_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size, double
               const Tensor& B,   // [in_dim, out_dim] or [out_dim, in_dim]
               const Tensor& C,   // [B, L, out_dim]
               Tensor& D) {       // [B, L, out_dim]
-    (void)qblock_size; (void)qtype_size;
-    STD_TORCH_CHECK(qtype_int == 1 || qtype_int == 30, "gemm: only 16-bit weights (qtype F16 = 1, BF16 = 30) are implemented");
+    STD_TORCH_CHECK(qtype_int == 1 || qtype_int == 30 || qtype_int == 8,
+                    "gemm: weights must be 16-bit (qtype F16 = 1, BF16 = 30) or Q8_0 blocks (qtype 8)");
     STD_TORCH_CHECK(on_gpu(A) && on_gpu(B) && on_gpu(C) && on_gpu(D), "gemm: all tensors must be on the GPU");
+    if (qtype_int == 8) {
+        // B [out_dim, in_dim / 32 * 34] bytes: alpha * A B^T + beta * C over the dequantised weight (reference:
+        // gemm/op.cuh:299-312 routes this case to dispatch_quant_abt, which is empty there)
+        STD_TORCH_CHECK(qblock_size == 32 && qtype_size == 34, "gemm: Q8_0 is (qblock_size, qtype_size) = (32, 34)");
+        STD_TORCH_CHECK(A.scalar_type() == ScalarType::Half && C.scalar_type() == ScalarType::Half && D.scalar_type() == ScalarType::Half,
+                        "gemm: A, C and D must be float16 with a Q8_0 weight");
+        STD_TORCH_CHECK(B.scalar_type() == ScalarType::Byte, "gemm: a Q8_0 weight is a uint8 tensor");
+        STD_TORCH_CHECK(A.dim() == 3 && B.dim() == 2 && C.dim() == 3 && D.dim() == 3, "gemm: A, C, D must be 3-D and B 2-D");
+        STD_TORCH_CHECK(A.is_contiguous() && B.is_contiguous() && C.is_contiguous() && D.is_contiguous(), "gemm: tensors must be contiguous");
+        const int64_t K = A.size(-1), M = A.numel() / (K > 0 ? K : 1), N = B.size(0);
+        STD_TORCH_CHECK(K % 32 == 0, "gemm: in_dim must be a multiple of the block size");
+        STD_TORCH_CHECK(B.size(1) == K / 32 * 34, "Unsupported dims for quant matmul");
+        STD_TORCH_CHECK(A.size(0) * A.size(1) == C.size(0) * C.size(1) && C.size(-1) == N, "gemm: C does not have the shape of A B^T");
+        STD_TORCH_CHECK(C.sizes().equals(D.sizes()), "gemm: C and D shapes differ");
+        STD_TORCH_CHECK(alpha != 0.0, "gemm: alpha must not be 0");
+        const size_t ws_bytes = minfer_gemm_q8_0_workspace_bytes(M, N, K);
+        Tensor ws = byte_workspace(A, ws_bytes);
+        check_rc(minfer_gemm_q8_0(A.const_data_ptr(), B.const_data_ptr(), C.const_data_ptr(), D.mutable_data_ptr(), M, N, K, K, N, N,
+                                  alpha, beta, ws_bytes ? ws.mutable_data_ptr() : nullptr, ws_bytes, current_stream()),
+                 "gemm");
+        return;
+    }
+    (void)qblock_size; (void)qtype_size;
     const ScalarType t = A.scalar_type();
     STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, "gemm: A must be float16 or bfloat16");
     STD_TORCH_CHECK(B.scalar_type() == t && C.scalar_type() == t && D.scalar_type() == t, "gemm: A, B, C and D must share one dtype");
@@ -472,9 +495,8 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
              Tensor& q_out,      // [B, L, q_dim]
              Tensor& k_out,      // [B, L, kv_dim]
              Tensor& v_out) {    // [B, L, kv_dim]
-    (void)q_qblock_size; (void)k_qblock_size; (void)v_qblock_size; (void)q_qtype_size; (void)k_qtype_size; (void)v_qtype_size;
-    STD_TORCH_CHECK((q_qtype_int == 1 || q_qtype_int == 30) && k_qtype_int == q_qtype_int && v_qtype_int == q_qtype_int,
-                    "qkv: only 16-bit weights (qtype F16 = 1, BF16 = 30) are implemented");
+    const int64_t qtypes[3] = {q_qtype_int, k_qtype_int, v_qtype_int};
+    const int64_t qblocks[3] = {q_qblock_size, k_qblock_size, v_qblock_size}, qsizes[3] = {q_qtype_size, k_qtype_size, v_qtype_size};
     const ScalarType t = x.scalar_type();
     STD_TORCH_CHECK(t == ScalarType::Half || t == ScalarType::BFloat16, "qkv: x must be float16 or bfloat16");
     STD_TORCH_CHECK(x.dim() == 3 && x.is_contiguous() && on_gpu(x), "qkv: x must be a contiguous 3-D GPU tensor");
@@ -484,6 +506,38 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
     const Tensor* ws[3] = {&wq, &wk, &wv};
     Tensor* outs[3] = {&q_out, &k_out, &v_out};
     const char* names[3] = {"qkv: q", "qkv: k", "qkv: v"};
+    if (qtypes[0] == MINFER_Q8_0 || qtypes[1] == MINFER_Q8_0 || qtypes[2] == MINFER_Q8_0) {
+        // weights as rows of Q8_0 blocks, uint8 [out_dim, hidden_dim / 32 * 34] (each may also be 16-bit): one projection per weight
+        STD_TORCH_CHECK(t == ScalarType::Half, "qkv: x must be float16 with a Q8_0 weight");
+        STD_TORCH_CHECK(K % 32 == 0, "qkv: hidden_dim must be a multiple of the block size");
+        for (int i = 0; i < 3; ++i) {
+            const Tensor& w = *ws[i];
+            Tensor& o = *outs[i];
+            STD_TORCH_CHECK(on_gpu(w) && on_gpu(o) && o.scalar_type() == t, names[i], ": dtype or device mismatch");
+            STD_TORCH_CHECK(w.dim() == 2 && o.dim() == 3 && w.is_contiguous() && o.is_contiguous(), names[i], ": weight must be contiguous 2-D, output contiguous 3-D");
+            STD_TORCH_CHECK(o.size(0) == x.size(0) && o.size(1) == x.size(1), names[i], ": output must be [B, L, out_dim]");
+            const int64_t N = o.size(-1);
+            if (qtypes[i] == MINFER_Q8_0) {
+                STD_TORCH_CHECK(qblocks[i] == MINFER_Q8_0_BLOCK && qsizes[i] == MINFER_Q8_0_BLOCK_BYTES, names[i], ": Q8_0 is (qblock_size, qtype_size) = (32, 34)");
+                STD_TORCH_CHECK(w.scalar_type() == ScalarType::Byte && w.size(0) == N && w.size(1) == K / 32 * 34, names[i],
+                                ": a Q8_0 weight is uint8 [out_dim, hidden_dim / 32 * 34]");
+                const size_t ws_bytes = minfer_gemm_q8_0_workspace_bytes(M, N, K);
+                Tensor wsp = byte_workspace(x, ws_bytes);
+                check_rc(minfer_gemm_q8_0(x.const_data_ptr(), w.const_data_ptr(), nullptr, o.mutable_data_ptr(), M, N, K, K, N, N, 1.0, 0.0,
+                                          ws_bytes ? wsp.mutable_data_ptr() : nullptr, ws_bytes, stream),
+                         names[i]);
+            } else {
+                STD_TORCH_CHECK(qtypes[i] == 1 && w.scalar_type() == t && w.size(0) == N && w.size(1) == K, names[i],
+                                ": next to a Q8_0 weight, a 16-bit weight must be float16 [out_dim, hidden_dim]");
+                check_rc(minfer_gemm(dtype, MINFER_GEMM_B_NK, x.const_data_ptr(), w.const_data_ptr(), nullptr, o.mutable_data_ptr(), M, N, K, K, K, N, N,
+                                     1.0, 0.0, stream),
+                         names[i]);
+            }
+        }
+        return;
+    }
+    STD_TORCH_CHECK((q_qtype_int == 1 || q_qtype_int == 30) && k_qtype_int == q_qtype_int && v_qtype_int == q_qtype_int,
+                    "qkv: weights must be 16-bit (qtype F16 = 1, BF16 = 30), all alike, or Q8_0 blocks (qtype 8)");
     bool all_nk = true;
     for (int i = 0; i < 3; ++i) {
         const Tensor& w = *ws[i];

@@ -225,14 +225,16 @@ def _(eps, input, w, out):
 def gemm(qtype_int: int, qblock_size: int, qtype_size: int, alpha: float, beta: float,
          A: torch.Tensor, B: torch.Tensor, C: torch.Tensor, D: torch.Tensor):
     """D = alpha * A B + beta * C; A [B,L,in_dim], weight B [in_dim,out_dim] (or [out_dim,in_dim]: A B^T), C and D
-    [B,L,out_dim]."""
+    [B,L,out_dim].  With (qtype_int, qblock_size, qtype_size) = (8, 32, 34) the weight is uint8 [out_dim, in_dim/32*34],
+    rows of Q8_0 blocks, and the product is A B^T over the dequantised weight."""
     return torch.ops.minfer.gemm.default(qtype_int, qblock_size, qtype_size, alpha, beta, A, B, C, D)
 
 
 @torch.library.register_fake("minfer::gemm")
 def _(qtype_int, qblock_size, qtype_size, alpha, beta, A, B, C, D):
     torch._check(A.dtype in _ACT_DTYPES)
-    torch._check(B.dtype == A.dtype and C.dtype == A.dtype and D.dtype == A.dtype)
+    torch._check(C.dtype == A.dtype and D.dtype == A.dtype)
+    torch._check(B.dtype == (torch.uint8 if qtype_int == 8 else A.dtype))
     torch._check(A.device == B.device == C.device == D.device)
     torch._check(A.device.type == "cuda")
     torch._check(A.dim() == 3 and B.dim() == 2 and C.dim() == 3 and D.dim() == 3)
@@ -246,7 +248,8 @@ def qkv(q_qtype_int: int, k_qtype_int: int, v_qtype_int: int, q_qblock_size: int
         q_qtype_size: int, k_qtype_size: int, v_qtype_size: int,
         x: torch.Tensor, wq: torch.Tensor, wk: torch.Tensor, wv: torch.Tensor,
         q_out: torch.Tensor, k_out: torch.Tensor, v_out: torch.Tensor):
-    """The three projections q_out = x wq^T, k_out = x wk^T, v_out = x wv^T; x [B,L,hidden], weights [out,hidden]."""
+    """The three projections q_out = x wq^T, k_out = x wk^T, v_out = x wv^T; x [B,L,hidden], weights [out,hidden]; a
+    weight whose type triple is (8, 32, 34) is uint8 [out, hidden/32*34], rows of Q8_0 blocks."""
     return torch.ops.minfer.qkv.default(q_qtype_int, k_qtype_int, v_qtype_int, q_qblock_size, k_qblock_size, v_qblock_size,
                                         q_qtype_size, k_qtype_size, v_qtype_size, x, wq, wk, wv, q_out, k_out, v_out)
 
@@ -255,7 +258,8 @@ def qkv(q_qtype_int: int, k_qtype_int: int, v_qtype_int: int, q_qblock_size: int
 def _(q_qtype_int, k_qtype_int, v_qtype_int, q_qblock_size, k_qblock_size, v_qblock_size, q_qtype_size, k_qtype_size,
       v_qtype_size, x, wq, wk, wv, q_out, k_out, v_out):
     torch._check(x.dtype in _ACT_DTYPES)
-    torch._check(all(t.dtype == x.dtype for t in (wq, wk, wv, q_out, k_out, v_out)))
+    torch._check(all(t.dtype == x.dtype for t in (q_out, k_out, v_out)))
+    torch._check(all(w.dtype == (torch.uint8 if qt == 8 else x.dtype) for w, qt in ((wq, q_qtype_int), (wk, k_qtype_int), (wv, v_qtype_int))))
     torch._check(x.device == wq.device == wk.device == wv.device == q_out.device == k_out.device == v_out.device)
     torch._check(x.device.type == "cuda")
     torch._check(x.dim() == 3 and q_out.dim() == 3 and k_out.dim() == 3 and v_out.dim() == 3)

@@ -63,6 +63,10 @@ def lib():
         L.minfer_gemm_ws.argtypes = [ctypes.c_int, ctypes.c_int, vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, i64, dbl, dbl, vp, ctypes.c_size_t, vp]
         L.minfer_gemm_workspace_bytes.restype = ctypes.c_size_t
         L.minfer_gemm_workspace_bytes.argtypes = [i64, i64, i64]
+        L.minfer_gemm_q8_0.restype = ctypes.c_int
+        L.minfer_gemm_q8_0.argtypes = [vp, vp, vp, vp, i64, i64, i64, i64, i64, i64, dbl, dbl, vp, ctypes.c_size_t, vp]
+        L.minfer_gemm_q8_0_workspace_bytes.restype = ctypes.c_size_t
+        L.minfer_gemm_q8_0_workspace_bytes.argtypes = [i64, i64, i64]
         L.minfer_qkv.restype = ctypes.c_int
         L.minfer_qkv.argtypes = [ctypes.c_int, vp, vp, vp, vp, vp, vp, vp] + [i64] * 12 + [vp]
         L.minfer_quant_q8_0.restype = ctypes.c_int
@@ -203,6 +207,15 @@ def gemm_ws(a, b, c, d, alpha, beta, ws, b_layout=GEMM_B_KN):
     return lib().minfer_gemm_ws(_dtype_code(a), b_layout, a.data_ptr(), b.data_ptr(), c.data_ptr() if c is not None else None,
                                 d.data_ptr(), M, N, K, a.stride(0), b.stride(0), c.stride(0) if c is not None else N, d.stride(0),
                                 alpha, beta, ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream())
+
+
+def gemm_q8_0(a, bq, c, d, alpha, beta, ws=None):
+    """d[M,N] = alpha * a[M,K] x dequant(bq)^T + beta * c; bq uint8 [N, K/32*34] rows of Q8_0 blocks; fp16 a, c, d."""
+    M, K = a.shape
+    N = d.shape[1]
+    return lib().minfer_gemm_q8_0(a.data_ptr(), bq.data_ptr(), c.data_ptr() if c is not None else None, d.data_ptr(), M, N, K,
+                                  a.stride(0), c.stride(0) if c is not None else N, d.stride(0), alpha, beta,
+                                  ws.data_ptr() if ws is not None else None, ws.numel() if ws is not None else 0, _stream())
 
 
 def qkv(x, wq, wk, wv, q_out, k_out, v_out):

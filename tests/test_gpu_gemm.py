@@ -240,3 +240,84 @@ def test_gemm_op_uses_k_slices_and_matches_oracle(dtype):
     D = torch.empty_like(Cc)
     kerns.gemm(qt, qb, qs, 1.0, 1.0, A, b.to(DEV), Cc, D)
     assert_close(D.view(M, N), exact, dtype, "gemm op, k slices")
+
+
+# ---- weights stored as Q8_0 blocks (minfer_gemm_q8_0; the gemm op with the type triple (8, 32, 34)) -----------------
+def make_q8(M, N, K, seed):
+    g = torch.Generator().manual_seed(seed)
+    a = torch.randn(M, K, generator=g).half()
+    w = (1 / K ** 0.5) * torch.randn(N, K, generator=g)
+    c = torch.randn(M, N, generator=g).half()
+    wq = torch.from_numpy(oracle.quant_q8_0(w.numpy()))                        # uint8 [N, K/32*34]
+    w_deq = torch.from_numpy(oracle.dequant_q8_0(wq.numpy(), np.float16))      # what every kernel must multiply with
+    return a, wq, c, w_deq
+
+
+@pytest.mark.parametrize("M,N,K,alpha,beta", [
+    (1, 4096, 4096, 1.0, 0.0),       # a decode step against a Llama-3-8B projection: the kernel that streams the blocks
+    (8, 1024, 4096, 1.0, 1.0),
+    (16, 256, 14336, 2.0, 3.0),      # a long contraction split over the eight waves
+    (17, 5152, 256, 1.0, 0.0),       # two column groups per workgroup, a ragged last one
+    (4, 5200, 512, 1.0, 1.0),        # the same with one block of rows
+    (64, 264, 192, 0.5, 1.0),        # its largest row count; K a multiple of 64 but not of 128: a short last step
+    (37, 24, 64, 1.0, 1.0),          # one step, half-empty column group
+    (65, 256, 256, 1.0, 2.0),        # above 64 rows: dequantise into the workspace, then the fp16 kernels
+    (300, 1032, 512, 2.0, 0.0),
+    (5, 64, 96, 1.0, 1.0),           # an odd number of blocks per row: workspace path at any row count
+])
+def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
+    a, wq, c, w_deq = make_q8(M, N, K, seed=M * 7 + N + K)
+    exact = oracle.gemm(a.float().numpy(), w_deq.float().numpy(), c.float().numpy(), alpha, beta, NK)
+    da, dwq, dc = a.to(DEV), wq.to(DEV), c.to(DEV)
+    d = torch.zeros(M, N, dtype=torch.float16, device=DEV)
+    need = capi.lib().minfer_gemm_q8_0_workspace_bytes(M, N, K)
+    assert (need == 0) == (M <= 64 and (K // 32) % 2 == 0)
+    ws = torch.full((max(need, 16),), 0xFF, dtype=torch.uint8, device=DEV)
+    assert capi.gemm_q8_0(da, dwq, dc, d, alpha, beta, ws if need else None) == capi.OK, capi.last_error()
+    assert_close(d, exact, torch.float16, "q8_0 weight")
+    # the same numbers as the fp16 kernel on the dequantised weight, up to the order of the fp32 sums
+    d_ref = torch.zeros_like(d)
+    assert capi.gemm(da, w_deq.to(DEV), dc, d_ref, alpha, beta, NK) == capi.OK, capi.last_error()
+    assert_close(d_ref, exact, torch.float16, "fp16 kernel on the dequantised weight")
+    if need:
+        assert capi.gemm_q8_0(da, dwq, dc, d, alpha, beta, None) == capi.EWORKSPACE and "workspace" in capi.last_error()
+
+
+def test_gemm_op_with_q8_0_weight(kerns):
+    M, N, K = 8, 2048, 4096
+    a, wq, c, w_deq = make_q8(M, N, K, seed=3)
+    exact = oracle.gemm(a.float().numpy(), w_deq.float().numpy(), c.float().numpy(), 1.0, 1.0, NK)
+    A, Cc = a.view(2, 4, K).to(DEV), c.view(2, 4, N).to(DEV)
+    D = torch.empty_like(Cc)
+    assert kerns.gemm(8, 32, 34, 1.0, 1.0, A, wq.to(DEV), Cc, D) is None
+    assert_close(D.view(M, N), exact, torch.float16, "gemm op, q8_0 weight")
+    A2 = torch.randn(1, 200, K, dtype=torch.float16, device=DEV)
+    C2 = torch.zeros(1, 200, N, dtype=torch.float16, device=DEV)
+    D2 = torch.empty_like(C2)
+    kerns.gemm(8, 32, 34, 1.0, 0.0, A2, wq.to(DEV), C2, D2)                      # prefill-sized: workspace path
+    exact2 = oracle.gemm(A2[0].float().cpu().numpy(), w_deq.float().numpy(), None, 1.0, 0.0, NK)
+    assert_close(D2[0], exact2, torch.float16, "gemm op, q8_0 weight, 200 rows")
+    with pytest.raises(RuntimeError, match="Unsupported dims"):
+        kerns.gemm(8, 32, 34, 1.0, 0.0, A2, wq.to(DEV)[:, :-34].contiguous(), C2, D2)
+    with pytest.raises(RuntimeError, match="float16"):
+        kerns.gemm(8, 32, 34, 1.0, 0.0, A2.bfloat16(), wq.to(DEV), C2.bfloat16(), D2.bfloat16())
+
+
+def test_qkv_op_with_q8_0_weights(kerns):
+    """The reference's QKV recipe (test/kernels.py:173-214) with the k and v weights as Q8_0 blocks and q as float16."""
+    B, L, K, Nq, Nkv = 2, 3, 2048, 1024, 256
+    g = torch.Generator().manual_seed(11)
+    x = torch.randn(B, L, K, generator=g).half()
+    wq = ((1 / K ** 0.5) * torch.randn(Nq, K, generator=g)).half()
+    wk = (1 / K ** 0.5) * torch.randn(Nkv, K, generator=g)
+    wv = (1 / K ** 0.5) * torch.randn(Nkv, K, generator=g)
+    wk8, wv8 = (torch.from_numpy(oracle.quant_q8_0(w.numpy())) for w in (wk, wv))
+    q, k, v = (torch.empty(B, L, n, dtype=torch.float16, device=DEV) for n in (Nq, Nkv, Nkv))
+    assert kerns.qkv(1, 8, 8, 1, 32, 32, 2, 34, 34, x.to(DEV), wq.to(DEV), wk8.to(DEV), wv8.to(DEV), q, k, v) is None
+    x2 = x.view(B * L, K).float().numpy()
+    assert_close(q.view(B * L, Nq), oracle.gemm(x2, wq.float().numpy(), None, 1.0, 0.0, NK), torch.float16, "q")
+    for out, w8, name in ((k, wk8, "k"), (v, wv8, "v")):
+        w_deq = torch.from_numpy(oracle.dequant_q8_0(w8.numpy(), np.float16)).float().numpy()
+        assert_close(out.view(B * L, Nkv), oracle.gemm(x2, w_deq, None, 1.0, 0.0, NK), torch.float16, name)
+    with pytest.raises(RuntimeError, match="Q8_0 weight is uint8"):
+        kerns.qkv(1, 8, 8, 1, 32, 32, 2, 34, 34, x.to(DEV), wq.to(DEV), wk8.to(DEV)[:, :-34].contiguous(), wv8.to(DEV), q, k, v)
