@@ -155,6 +155,25 @@ def test_gemm_validation_rejects_before_launch():
     assert gemm_ws(M=0) == capi.OK
 
 
+def test_gemm_q8_0_validation_rejects_before_launch():
+    L = capi.lib()
+    g = lambda a=0x1000, b=0x2000, c=None, d=0x4000, M=4, N=64, K=256, lda=256, ldc=64, ldd=64, alpha=1.0, beta=0.0, ws=None, wsb=0: \
+        L.minfer_gemm_q8_0(a, b, c, d, M, N, K, lda, ldc, ldd, alpha, beta, ws, wsb, None)
+    assert g(K=100) == capi.EINVAL and "multiple of the block size" in capi.last_error()
+    assert g(a=0) == capi.EINVAL and "null" in capi.last_error()
+    assert g(beta=1.0) == capi.EINVAL                                  # beta != 0 needs C
+    assert g(lda=128) == capi.EINVAL and "leading" in capi.last_error()
+    assert g(b=0x2002) == capi.EINVAL and "4-byte" in capi.last_error()
+    assert g(a=0x1008) == capi.EINVAL and "16-byte" in capi.last_error()   # the streaming kernel's alignment
+    assert g(M=100) == capi.EWORKSPACE and "workspace" in capi.last_error()   # more than 64 rows: needs the dequantised weight
+    assert g(K=96, lda=96) == capi.EWORKSPACE                               # an odd number of blocks per row as well
+    assert g(M=0) == capi.OK and g(N=0) == capi.OK and capi.last_error() == ""
+    ws = L.minfer_gemm_q8_0_workspace_bytes
+    assert ws(1, 4096, 4096) == 0 and ws(64, 14336, 4096) == 0
+    assert ws(65, 4096, 4096) == 4096 * 4096 * 2 + L.minfer_gemm_workspace_bytes(65, 4096, 4096)
+    assert ws(4, 64, 96) == (64 * 96 * 2 + 255) // 256 * 256 and ws(4, 64, 100) == 0 and ws(0, 64, 128) == 0
+
+
 def test_gemm_workspace_sizes():
     L = capi.lib()
     ws = L.minfer_gemm_workspace_bytes
