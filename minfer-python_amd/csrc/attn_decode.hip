@@ -33,6 +33,8 @@
 #include <atomic>
 #include <mutex>
 
+#include <type_traits>
+
 #include "attn_common.h"
 #include "attn_host.h"
 #include "quant_q8.h"
@@ -431,22 +433,32 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
         const int rel_last = real ? (int)min(last - group_off, (int64_t)16 * (NG - 1)) : 0;   // >= 0
         return min(16 * (64 * j + lane), rel_last);
     };
-    auto load_group = [&](int t, Stage& st) {
+    // A group that is not the wave's last lies wholly inside the chunk: its pieces need no clamping (their offsets are
+    // constants of the lane) and its keys no masking.  `inner_tag` says so at compile time; the loop below runs such
+    // groups through code without the clamps and falls back to the general code for the last ones.
+    int inner_off[NL];
+#pragma unroll
+    for (int j = 0; j < NL; ++j) inner_off[j] = min(16 * (64 * j + lane), 16 * (NG - 1));
+    auto load_group = [&](auto inner_tag, int t, Stage& st) __attribute__((always_inline)) {
+        constexpr bool INNER = decltype(inner_tag)::value;
+        const int64_t inner_goff = (int64_t)(row_lo + t * GR) * ROWB;
 #pragma unroll
         for (int j = 0; j < NL; ++j) {
-            int64_t goff;
-            const int off = piece_offset(t, j, last_k, goff);
+            int64_t goff = inner_goff;
+            const int off = INNER ? inner_off[j] : piece_offset(t, j, last_k, goff);
             st.k[j] = stream_load(reinterpret_cast<const u32x4*>(kb16 + goff + off));
         }
 #pragma unroll
         for (int j = 0; j < NL; ++j) {
-            int64_t goff;
-            const int off = piece_offset(t, j, last_v, goff);
+            int64_t goff = inner_goff;
+            const int off = INNER ? inner_off[j] : piece_offset(t, j, last_v, goff);
             st.v[j] = stream_load(reinterpret_cast<const u32x4*>(vb16 + goff + off));
         }
     };
+    const std::false_type general_tag{};
+    const std::true_type inner_group_tag{};
 #pragma unroll
-    for (int s = 0; s < NS; ++s) load_group(s, ring[s]);
+    for (int s = 0; s < NS; ++s) load_group(general_tag, s, ring[s]);
 
     f32x4 o_acc[DB];
 #pragma unroll
@@ -468,13 +480,14 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
         return h16x2{dh, dh};
     };
 
-    auto consume = [&](int t, const Stage& st) {
+    auto consume = [&](auto inner_tag, int t, const Stage& st) __attribute__((always_inline)) {
+        constexpr bool INNER = decltype(inner_tag)::value;
         const int r0 = row_lo + t * GR;
         int64_t goff;
         // ---- the group's pieces into the wave's raw areas ----------------------------------------------
 #pragma unroll
         for (int j = 0; j < NL; ++j) {
-            const int off = piece_offset(t, j, last_k, goff);
+            const int off = INNER ? inner_off[j] : piece_offset(t, j, last_k, goff);
             *reinterpret_cast<u32x4*>(raw_k + off) = st.k[j];
         }
         // ---- S^T = K Q^T for the two 16-key halves: lane gets head l16, keys 16h + 4*quad + r ---------------
@@ -485,7 +498,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
             // the lane's share of its key's row: D/4 values starting at D/4 * quad (one block at D = 128, half a block at 64)
             const int at = pre_k + row * ROWB + (D == 128 ? quad : quad >> 1) * 34;
             const uint32_t* wp = reinterpret_cast<const uint32_t*>(raw_k + (at & ~3));
-            const h16x2 d2 = scale_of(wp[0], k_odd, r0 + row < row_hi);
+            const h16x2 d2 = scale_of(wp[0], k_odd, INNER || r0 + row < row_hi);
             constexpr int NW = D / 16;                       // quant words of the lane's share
             const uint32_t* qp = wp + (D == 128 ? 0 : 4 * (quad & 1));
             uint32_t wq[NW + 1];
@@ -495,14 +508,16 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
 #pragma unroll
             for (int c = 0; c < KC; ++c)
                 s[h] = T::mfma16(dequant8_shifted(wq[2 * c], wq[2 * c + 1], wq[2 * c + 2], k_sel, d2), qf[c], s[h]);
-            const int key0 = r0 + 16 * h + 4 * quad;
+            if (!INNER) {
+                const int key0 = r0 + 16 * h + 4 * quad;
 #pragma unroll
-            for (int r = 0; r < 4; ++r) s[h][r] = (key0 + r < row_hi) ? s[h][r] : -INFINITY;
+                for (int r = 0; r < 4; ++r) s[h][r] = (key0 + r < row_hi) ? s[h][r] : -INFINITY;
+            }
         }
         // ---- V: its pieces over K's, then every lane dequantises GR * BPR / 64 blocks and parks them as fp16 rows (swizzled)
 #pragma unroll
         for (int j = 0; j < NL; ++j) {
-            const int off = piece_offset(t, j, last_v, goff);
+            const int off = INNER ? inner_off[j] : piece_offset(t, j, last_v, goff);
             *reinterpret_cast<u32x4*>(raw_v + off) = st.v[j];
         }
 #pragma unroll
@@ -513,7 +528,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
             uint32_t wv[9];
 #pragma unroll
             for (int j = 0; j < 9; ++j) wv[j] = wp[j];
-            const h16x2 d2 = scale_of(wv[0], v_odd, r0 + row < row_hi);
+            const h16x2 d2 = scale_of(wv[0], v_odd, INNER || r0 + row < row_hi);
             char* rowp = park_v + row * RB;
             const int sw = GEO::swz_v(row);
 #pragma unroll
@@ -564,11 +579,20 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
         }
     };
 
-    for (int t0 = 0; t0 < n_groups; t0 += NS) {
+    int t0 = 0;
+    // rounds in which every group consumed and every group requested is an inner one
+    for (; t0 + 2 * NS < n_groups; t0 += NS) {
 #pragma unroll
         for (int s = 0; s < NS; ++s) {
-            if (t0 + s < n_groups) consume(t0 + s, ring[s]);
-            load_group(t0 + s + NS, ring[s]);
+            consume(inner_group_tag, t0 + s, ring[s]);
+            load_group(inner_group_tag, t0 + s + NS, ring[s]);
+        }
+    }
+    for (; t0 < n_groups; t0 += NS) {
+#pragma unroll
+        for (int s = 0; s < NS; ++s) {
+            if (t0 + s < n_groups) consume(general_tag, t0 + s, ring[s]);
+            load_group(general_tag, t0 + s + NS, ring[s]);
         }
     }
 
