@@ -3,7 +3,7 @@ through the registered torch ops), against the CPU oracle on identical seeded in
 
 Tolerances are the ones the task fixes: max-abs error <= 2e-3 for fp16 and <= 1e-2 for bf16 against
 an fp32-or-better reference.  Masking and the GQA head mapping are checked for exact equality.
-At full BASELINE sizes the oracle is evaluated on a sample of query rows (it is a scalar CPU
+At the full benchmark sizes the oracle is evaluated on a sample of query rows (it is a scalar CPU
 program) and the whole output is additionally compared with a plain fp32 torch evaluation of the
 same formula on the GPU.
 """
@@ -101,7 +101,7 @@ def test_golden_decode_and_varlen():
 # ------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("B,Hq,Hkv,L,D,kind,views", [
-    (1, 8, 2, 256, 64, "causal", False),     # BASELINE config 1 shape
+    (1, 8, 2, 256, 64, "causal", False),     # benchmark configuration 1 shape
     (2, 8, 2, 320, 128, "causal", True),     # reference-style transposed views
     (2, 6, 2, 200, 128, "window", False),    # n_rep = 3, symmetric window (reference test case B)
     (2, 4, 4, 333, 128, "random", False),    # L % 4 != 0: byte-wise mask path, per-batch masks
@@ -125,7 +125,7 @@ def test_dense_matches_oracle(dtype, B, Hq, Hkv, L, D, kind, views):
 
 
 def test_cpu_plumbing_config_on_gpu():
-    """BASELINE config 1 (fp32 N(0,1) inputs, S=256, D=64): the same seeded inputs rounded to fp16."""
+    """benchmark configuration 1 (fp32 N(0,1) inputs, S=256, D=64): the same seeded inputs rounded to fp16."""
     q, k, v, mask = workloads.cpu_plumbing(seed=0)
     want = oracle.flash_attn(q.half(), k.half(), v.half(), mask)
     out = run_prefill(q.half().to(DEV), k.half().to(DEV), v.half().to(DEV), mask.to(DEV))
@@ -184,7 +184,7 @@ def test_masking_and_gqa_mapping_exact(dtype):
 
 
 # ------------------------------------------------------------------------------------------------
-# BASELINE configs at full size
+# the benchmark configurations at full size
 # ------------------------------------------------------------------------------------------------
 def sample_rows(L, n, gen):
     fixed = [0, 1, 31, 32, 63, 64, 65, L // 2, L - 65, L - 2, L - 1]
@@ -194,7 +194,7 @@ def sample_rows(L, n, gen):
 
 @pytest.mark.parametrize("views", [False, True])
 def test_llama8b_prefill_full(views):
-    """BASELINE config 2: B=1, Hq=32, Hkv=8, S=4096, D=128, fp16, causal, 0.5*N(0,1)."""
+    """benchmark configuration 2: B=1, Hq=32, Hkv=8, S=4096, D=128, fp16, causal, 0.5*N(0,1)."""
     q, k, v, mask = workloads.llama8b_prefill(seed=0, device=DEV, views=views)
     out = run_prefill(q, k, v, mask)
     assert max_err(out, torch_ref(q, k, v, mask)) <= TOL[torch.float16]
@@ -205,7 +205,7 @@ def test_llama8b_prefill_full(views):
 
 
 def test_long_context_prefill_full():
-    """BASELINE config 4: B=1, Hq=32, Hkv=8, S=32768, D=128, bf16, causal, 0.5*N(0,1)."""
+    """benchmark configuration 4: B=1, Hq=32, Hkv=8, S=32768, D=128, bf16, causal, 0.5*N(0,1)."""
     L = 32768
     q, k, v, mask = workloads.long_context_prefill(seed=0, device=DEV, L=L)
     out = run_prefill(q, k, v, mask)
@@ -217,7 +217,7 @@ def test_long_context_prefill_full():
 
 
 def test_decode_full():
-    """BASELINE config 3: B=64, Hq=32, Hkv=8, D=128, fp16, ctx in [512, 8192], cache [B,Hkv,8192,128]."""
+    """benchmark configuration 3: B=64, Hq=32, Hkv=8, D=128, fp16, ctx in [512, 8192], cache [B,Hkv,8192,128]."""
     q, kc, vc, ctx = workloads.decode_cache(seed=0, device=DEV)
     # rows beyond ctx are garbage that must not reach the result
     for b in range(0, 64, 7):
@@ -232,7 +232,7 @@ def test_decode_full():
 
 
 def test_ragged_prefill_full():
-    """BASELINE config 5: 16 sequences, lengths in [128, 2048], Hq=64, Hkv=8, D=128, fp16, N(0,1)."""
+    """benchmark configuration 5: 16 sequences, lengths in [128, 2048], Hq=64, Hkv=8, D=128, fp16, N(0,1)."""
     q, k, v, cu = workloads.ragged_prefill(seed=0, device=DEV)
     lens = (cu[1:] - cu[:-1]).tolist()
     out = torch.full(q.shape, float("nan"), dtype=q.dtype, device=DEV)

@@ -70,7 +70,7 @@ def test_oracle_matches_sdpa_and_numpy(B, Hq, Hkv, L, D, kind):
 
 
 def test_cpu_plumbing_config():
-    """BASELINE config 1: B=1, Hq=8, Hkv=2, S=256, D=64, fp32, causal, scale 1/sqrt(64)."""
+    """benchmark configuration 1: B=1, Hq=8, Hkv=2, S=256, D=64, fp32, causal, scale 1/sqrt(64)."""
     import workloads
     q, k, v, mask = workloads.cpu_plumbing(seed=0)
     got = oracle.flash_attn(q, k, v, mask)
