@@ -198,6 +198,7 @@ def test_qkv_op_and_reference_checks(kerns):
     (256, 2048, 1024, 0.5, 1.0),     # two tile rows
     (40, 512, 1984, 1.0, 0.0),       # K steps (31) not a multiple of the slice count
     (1, 4096, 4096, 1.0, 1.0),       # one row: with [K, N] the sliced tiles, with [N, K] still the few-row kernel
+    (24, 1024, 2048, 1.0, 1.0),      # 17-32 rows: with a workspace the sliced tiles for both layouts
 ])
 def test_gemm_k_slices_against_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, seed=M + N + K)

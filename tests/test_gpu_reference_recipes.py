@@ -110,3 +110,29 @@ def test_opcheck_rmsnorm_and_rope():
     r = workloads.rope_input(seed=5, device=DEV, B=2, L=8, H=4, D=128)
     _opcheck(torch.ops.minfer.il_rope.default, (64, 3, 1e6, r))
     _opcheck(torch.ops.minfer.neox_rope.default, (64, 3, 1e6, r))
+
+
+def test_opcheck_producers_and_quantised_operands():
+    """The ops beyond the reference's set: the cache producers, the Q8_0 operands of gemm / qkv / the attention ops."""
+    q8 = GGMLQuantizationType.Q8_0
+    q8b, q8s = GGML_QUANT_SIZES[q8]
+    q, k, v, pos, kc, vc = workloads.kv_append(seed=3, device=DEV, B=2, L=5, Hq=8, Hkv=2, D=128, Lmax=16)
+    _opcheck(torch.ops.minfer.rope_kv_append.default, (1, 128, 5e5, q.clone(), k, v, pos, kc.clone(), vc.clone()))
+    w = torch.ones(128, dtype=q.dtype, device=DEV)
+    _opcheck(torch.ops.minfer.rope_kv_append_norm.default, (1, 128, 5e5, 1e-6, q.clone(), k, v, w, w, pos, kc.clone(), vc.clone()))
+    kq = torch.zeros(2, 2, 16, 136, dtype=torch.uint8, device=DEV)
+    _opcheck(torch.ops.minfer.rope_kv_append.default, (1, 128, 5e5, q.clone(), k, v, pos, kq, kq.clone()))
+    # a weight of Q8_0 blocks
+    a, wf, bias = workloads.gemm_input(8, 256, 512, seed=4, device=DEV)
+    wq = torch.empty(256, 512 // 32 * 34, dtype=torch.uint8, device=DEV)
+    torch.ops.minfer.quant.default(q8, q8b, q8s, wf.t().contiguous(), wq)
+    _opcheck(torch.ops.minfer.gemm.default, (q8, q8b, q8s, 1.0, 1.0, a, wq, bias, torch.zeros_like(bias)))
+    outs = [torch.zeros(1, 8, 256, dtype=torch.float16, device=DEV) for _ in range(3)]
+    _opcheck(torch.ops.minfer.qkv.default, (q8, q8, q8, q8b, q8b, q8b, q8s, q8s, q8s, a, wq, wq, wq, *outs))
+    # decode over Q8_0 caches
+    qd, kcf, vcf, ctx = workloads.decode_cache(seed=2, device=DEV, B=2, Hq=8, Hkv=2, Lmax=64, ctx_lo=1, ctx_hi=64)
+    kc8 = torch.empty(2, 2, 64, 136, dtype=torch.uint8, device=DEV)
+    vc8 = torch.empty_like(kc8)
+    torch.ops.minfer.quant.default(q8, q8b, q8s, kcf.reshape(-1, 128), kc8.view(-1, 136))
+    torch.ops.minfer.quant.default(q8, q8b, q8s, vcf.reshape(-1, 128), vc8.view(-1, 136))
+    _opcheck(torch.ops.minfer.flash_attn_decode.default, (q8, q8b, q8s, qd, kc8, vc8, ctx, torch.zeros_like(qd)))
