@@ -35,8 +35,12 @@ template <int MB_, int NB_, int WAVES_N_, int OCC_> struct GemmShape {
     static constexpr int A_PANEL = BM * 128, B_PANEL = BN * 128;   // bytes of one K step
     static constexpr int A_COPIES = A_PANEL / 1024 / WAVES, B_COPIES = B_PANEL / 1024 / WAVES;   // wave-wide copies per wave
 };
-// (4 waves with 128 x 128 each, GemmShape<4, 4, 2, 1>, read a third fewer LDS bytes per flop and run 3.2x slower: with
-// one wave per SIMD nothing covers a wave's waits for its fragments.)
+// (4 waves with 128 x 128 each, GemmShape<4, 4, 2, 1>, read a third fewer LDS bytes per flop.  Compiled as it stands
+// that shape spills (its 256 accumulators leave the allocator no register to move anything with) and runs 3.2x slower;
+// with 14 of the 16 accumulator blocks pinned to the accumulation registers and 2 to the vector registers by inline
+// assembly, one copy offset per panel, and the LDS reads and global->LDS copies issued one after each MFMA, since no
+// second wave covers a burst of them, it is spill-free and ends level with the 8-wave shape at 4096^3 (122.5 against
+// 124.0 us) and 4 % behind at 8192^3: the LDS bytes are not what bounds this kernel.)
 using GemmBig = GemmShape<4, 2, 4, 2>;
 using GemmSmall = GemmShape<2, 2, 2, 2>;
 constexpr int kRowTile = 8192;              // sub-tile [64 rows][64 k], 128-byte rows (A, and B as [N, K])
