@@ -260,6 +260,8 @@ def make_q8(M, N, K, seed):
     (16, 256, 14336, 2.0, 3.0),      # a long contraction split over the eight waves
     (17, 5152, 256, 1.0, 0.0),       # two column groups per workgroup, a ragged last one
     (4, 5200, 512, 1.0, 1.0),        # the same with one block of rows
+    (40, 5152, 512, 2.0, 1.0),       # three and four blocks of rows with two column groups
+    (64, 5120, 256, 1.0, 0.0),
     (64, 264, 192, 0.5, 1.0),        # its largest row count; K a multiple of 64 but not of 128: a short last step
     (37, 24, 64, 1.0, 1.0),          # one step, half-empty column group
     (65, 256, 256, 1.0, 2.0),        # above 64 rows: dequantise into the workspace, then the fp16 kernels
