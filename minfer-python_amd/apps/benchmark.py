@@ -49,6 +49,30 @@ def flash_attn(backend: str, which: str):
     Compare(results).print()
 
 
+def flash_attn_operand_data(backend: str, which: str):
+    """The prefill kernel on one shape (B=1, 32 heads over 8 KV heads, L=8192) with random and with constant operands,
+    fp16 and bf16: the instruction stream is the same in all cases, so any difference is what the values cost the
+    chip in power (the matrix units switch less on constant data) and the clock it can then hold."""
+    kerns = KernelBackend(backend)
+    B, Hq, Hkv, L, D = 1, 32, 8, 8192, 128
+    mask = workloads.causal_mask(B, L, device="cuda")
+    results = []
+    for dtype, qt in ((torch.float16, GGMLQuantizationType.F16), (torch.bfloat16, GGMLQuantizationType.BF16)):
+        qb, qs = GGML_QUANT_SIZES[qt]
+        q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, dtype, scale=0.5, device="cuda")
+        for name, (qq, kk, vv) in (("N(0, 0.5)", (q, k, v)),
+                                   ("all 0.25", (torch.full_like(q, 0.25), torch.full_like(k, 0.25), torch.full_like(v, 0.25))),
+                                   ("all 0", (torch.zeros_like(q), torch.zeros_like(k), torch.zeros_like(v)))):
+            out = torch.zeros_like(q)
+            if which == "minfer":
+                fn = lambda: kerns.flash_attn(qt, qb, qs, qq, kk, vv, mask, out)
+            else:
+                k_exp, v_exp = kk.repeat_interleave(Hq // Hkv, dim=1), vv.repeat_interleave(Hq // Hkv, dim=1)
+                fn = lambda: refs.flash_attn(qq, k_exp, v_exp, mask)
+            results.append(_measure(fn, f"L={L}, {str(dtype).split('.')[-1]}, operands {name}", which, "flash_attn"))
+    Compare(results).print()
+
+
 def flash_attn_decode(backend: str, which: str):
     kerns = KernelBackend(backend)
     results = []
@@ -182,7 +206,7 @@ def gemm(backend: str, which: str):
 
 
 if __name__ == "__main__":
-    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
+    KERNELS = {"flash_attn": flash_attn, "flash_attn_operand_data": flash_attn_operand_data, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
                "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "rmsnorm": rmsnorm, "il_rope": il_rope, "neox_rope": neox_rope,
                "rope_kv_append": rope_kv_append, "gemm": gemm}
     parser = argparse.ArgumentParser()
