@@ -39,6 +39,9 @@ DECODE_Q8_TRAFFIC_BYTES = 598453 * 1024     # decode over Q8_0 caches (split + c
 APPEND_Q8_TRAFFIC_BYTES = 737585 * 1024     # rope_kv_append into Q8_0 caches
 APPEND_NORM_TRAFFIC_BYTES = 786620 * 1024   # rope_kv_append_norm, the same shape
 QKV_TRAFFIC_BYTES = 377657 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
+LONG_TRAFFIC_BYTES = None                   # long-context prefill (classify + main), S=32768 bf16
+RAGGED_TRAFFIC_BYTES = None                 # packed ragged prefill
+GEMM_Q8_TRAFFIC_BYTES = None                # one token against a 14336 x 4096 weight of Q8_0 blocks
 
 
 class HipEvents:
@@ -88,22 +91,92 @@ class HipEvents:
         return sum(ms) / len(ms), ms_sorted[len(ms) // 2]
 
 
+def _median3(fn):
+    ts = []
+    for _ in range(3):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    return sorted(ts)[1]
+
+
 def cpu_baseline(torch, workloads, refs, L):
     """The reference's CPU attention path: refs.flash_attn = torch SDPA, fp32, K/V pre-expanded outside
     the timed region, on the same seeded inputs up-cast (reference: apps/benchmark.py:240-248)."""
     q, k, v, mask = workloads.llama8b_prefill(seed=0, L=L)
     q, k, v = q.float(), k.float().repeat_interleave(4, 1), v.float().repeat_interleave(4, 1)
     refs.flash_attn(q[:, :4], k[:, :4], v[:, :4], mask)  # warm-up on a slice
-    ts = []
-    for _ in range(3):
-        t0 = time.perf_counter()
-        refs.flash_attn(q, k, v, mask)
-        ts.append(time.perf_counter() - t0)
-    t = sorted(ts)[1]
+    t = _median3(lambda: refs.flash_attn(q, k, v, mask))
     flops = workloads.prefill_flops(32, 128, [L])
     return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
             "sample": f"refs.flash_attn (torch SDPA, fp32, dense causal mask) on the full S={L} workload, median of 3: {t * 1e3:.1f} ms",
             "host_cpus": os.cpu_count()}
+
+
+def cpu_baseline_plumbing(torch, workloads, refs):
+    """BASELINE configs[0] (B=1, Hq=8, Hkv=2, S=256, D=64, fp32): the reference's CPU path on it."""
+    q, k, v, mask = workloads.cpu_plumbing(seed=0)
+    k, v = k.repeat_interleave(4, 1), v.repeat_interleave(4, 1)
+    refs.flash_attn(q, k, v, mask)
+    t = _median3(lambda: refs.flash_attn(q, k, v, mask))
+    flops = workloads.prefill_flops(8, 64, [256])
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"refs.flash_attn (torch SDPA, fp32) on the full B=1 Hq=8 Hkv=2 S=256 D=64 workload, median of 3: {t * 1e3:.3f} ms"}
+
+
+def cpu_baseline_decode(torch, workloads, refs, n_seq=16):
+    """The reference's CPU path on the decode workload: SDPA in fp32 with Lq = 1 and the [B,1,1,Lmax] mask that ctx_lens
+    gives, K/V caches pre-expanded to the query heads outside the timed region.  A sample of `n_seq` of the 64
+    sequences (the expanded fp32 caches of all 64 would be 17 GB); same algorithmic bytes per sequence as the GPU figure."""
+    q, kc, vc, ctx = workloads.decode_cache(seed=0, B=n_seq)
+    q, kc, vc = q.float(), kc.float().repeat_interleave(4, 1), vc.float().repeat_interleave(4, 1)
+    refs.flash_attn_decode(q[:1], kc[:1], vc[:1], ctx[:1])
+    t = _median3(lambda: refs.flash_attn_decode(q, kc, vc, ctx))
+    nbytes = workloads.decode_bytes(ctx.tolist(), 32, 8, 128)
+    return {"value": nbytes / t / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"refs.flash_attn_decode (torch SDPA, fp32, mask from ctx_lens) on {n_seq} of the 64 sequences "
+                      f"(sum ctx = {int(ctx.sum())} rows, fp16-cache algorithmic bytes), median of 3: {t * 1e3:.1f} ms"}
+
+
+def cpu_baseline_ragged(torch, workloads, refs):
+    """The reference's CPU path on the packed workload: one refs.flash_attn call per sequence with its causal bool mask
+    (masks and the GQA expansion built outside the timed region), times summed over the 16 sequences."""
+    q, k, v, cu = workloads.ragged_prefill(seed=0)
+    n_rep = q.shape[1] // k.shape[1]
+    q, k, v = q.float(), k.float().repeat_interleave(n_rep, 1), v.float().repeat_interleave(n_rep, 1)
+    cu = cu.tolist()
+    parts = [(q[:, :, lo:hi], k[:, :, lo:hi], v[:, :, lo:hi], workloads.causal_mask(1, hi - lo)) for lo, hi in zip(cu[:-1], cu[1:])]
+    refs.flash_attn(*parts[0])
+
+    def run():
+        for a in parts:
+            refs.flash_attn(*a)
+    t = _median3(run)
+    lens = [hi - lo for lo, hi in zip(cu[:-1], cu[1:])]
+    flops = workloads.prefill_flops(q.shape[1], 128, lens)
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"refs.flash_attn (torch SDPA, fp32, causal bool mask) once per sequence on the full packed workload "
+                      f"(16 sequences, T={cu[-1]}), summed, median of 3: {t * 1e3:.1f} ms"}
+
+
+def cpu_baseline_long(torch, workloads, refs, L=32768, rows=1024, cap_s=60.0):
+    """The reference's CPU path on the long-context workload, bounded: the last `rows` query rows of the S=32768 problem
+    against all keys (SDPA, fp32, their rows of the dense causal mask), one timed run; the whole problem is 32 times
+    that.  Reported as capped if the run exceeds `cap_s`."""
+    g = torch.Generator().manual_seed(0)
+    q = (0.5 * torch.randn(1, 32, rows, 128, generator=g)).bfloat16().float()
+    k = (0.5 * torch.randn(1, 8, L, 128, generator=g)).bfloat16().float().repeat_interleave(4, 1)
+    v = (0.5 * torch.randn(1, 8, L, 128, generator=g)).bfloat16().float().repeat_interleave(4, 1)
+    i = torch.arange(L - rows, L)
+    mask = (torch.arange(L)[None, :] <= i[:, None])[None, None].contiguous()
+    refs.flash_attn(q[:, :1, :64], k[:, :1], v[:, :1], mask[:, :, :64])
+    t0 = time.perf_counter()
+    refs.flash_attn(q, k, v, mask)
+    t = time.perf_counter() - t0
+    flops = 4.0 * 128 * 32 * sum(range(L - rows + 1, L + 1))
+    return {"value": flops / t / 1e12, "unit": "TFLOP/s", "cores": torch.get_num_threads(), "kind": "port", "capped": t > cap_s,
+            "sample": f"refs.flash_attn (torch SDPA, fp32) on the last {rows} query rows of the S={L} workload against all keys "
+                      f"({flops:.3e} of its 8.796e12 algorithmic flop), one run: {t * 1e3:.1f} ms"}
 
 
 def rope_cpu_baseline(torch, workloads, refs):
@@ -352,6 +425,30 @@ def main():
     q8_gbs = q8bytes / (q8_avg_ms * 1e-3) / 1e9
     del wq8, xa, xo
 
+    # ---- BASELINE configs[0] (the CPU-plumbing shape: B=1, Hq=8, Hkv=2, S=256, D=64) through the GPU op; its fp32
+    # inputs are rounded to fp16, the op having no fp32 form.  Two launches of a few microseconds: launch-bound.
+    cq, ck, cv, cmask = workloads.cpu_plumbing(seed=0)
+    cq, ck, cv, cmask = cq.half().to(dev), ck.half().to(dev), cv.half().to(dev), cmask.to(dev)
+    cout = torch.empty_like(cq)
+    cstep = lambda: kerns.flash_attn(qt, qb, qs, cq, ck, cv, cmask, cout)
+    for _ in range(50):
+        cstep()
+    torch.cuda.synchronize()
+    c_avg_ms, c_med_ms = ev.time_each(cstep, stream, 50)
+    cflops = workloads.prefill_flops(8, 64, [256])
+
+    # ---- calibration: what the chip sustains on the matrix instruction alone, on operand values of the benchmarks'
+    # distribution (the nominal peak assumes 2.4 GHz, which the chip does not hold with the matrix pipes busy) ----
+    import calibration
+    sus_f16 = calibration.mfma_rate(torch.float16, "random", timed_ms=100.0, prewarm_ms=100.0)
+    sus_bf16 = calibration.mfma_rate(torch.bfloat16, "random", timed_ms=100.0, prewarm_ms=100.0)
+
+    def mfma_roofline(achieved_tf, sustained, **extra):
+        r = {"bound": "mfma", "achieved": achieved_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": achieved_tf / PEAK_MFMA_TFLOPS,
+             "sustained_mfma_only": sustained["tflops"], "frac_of_sustained": achieved_tf / sustained["tflops"]}
+        r.update(extra)
+        return r
+
     rec = {
         "metric": "prefill attn TFLOP/s + decode KV GB/s (Llama-3-8B GQA), % of roofline",
         "value": tflops, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
@@ -360,10 +457,9 @@ def main():
         "dtype": "f16", "data": "synthetic", "launch": "hipgraph replay of one op call" if args.graph else "eager",
         "config": {"workload": "prefill B=1 Hq=32 Hkv=8 S=4096 D=128 fp16 causal dense-mask (BASELINE configs[1])",
                    "global_batch": 1, "seq_len": L, "parallelism": "single-gpu"},
-        "roofline": {"bound": "mfma", "achieved": achieved, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / PEAK_MFMA_TFLOPS, "traffic": PREFILL_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE,
-                     "kernel": "classify_mask_kernel + prefill_kernel<F16,128,dense>",
-                     "algorithmic_flops": flops, "avg_ms": avg_ms, "median_ms": med_ms},
+        "roofline": mfma_roofline(achieved, sus_f16, traffic=PREFILL_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
+                                  kernel="classify_mask_kernel + prefill_kernel<F16,128,dense>",
+                                  algorithmic_flops=flops, avg_ms=avg_ms, median_ms=med_ms),
         "decode": {"value": d_gbs, "unit": "GB/s", "ms": d_avg_ms, "median_ms": d_med_ms,
                    "workload": "decode B=64 Hq=32 Hkv=8 D=128 fp16 ctx~U[512,8192] cache [64,8,8192,128] (BASELINE configs[2])",
                    "roofline": {"bound": "hbm", "achieved": d_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s",
@@ -380,12 +476,12 @@ def main():
                                        "algorithmic_bytes": d8bytes}}
     rec["long_context"] = {"value": l_tf, "unit": "TFLOP/s", "ms": l_avg_ms, "median_ms": l_med_ms,
                            "workload": "prefill B=1 Hq=32 Hkv=8 S=32768 D=128 bf16 causal dense-mask, mask 1 GiB (BASELINE configs[3])",
-                           "roofline": {"bound": "mfma", "achieved": l_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": l_tf / PEAK_MFMA_TFLOPS,
-                                        "traffic": None, "kernel": "classify_mask_kernel + prefill_kernel<BF16,128,dense>", "algorithmic_flops": lflops}}
+                           "roofline": mfma_roofline(l_tf, sus_bf16, traffic=LONG_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
+                                                     kernel="classify_mask_kernel + prefill_kernel<BF16,128,dense>", algorithmic_flops=lflops)}
     rec["ragged"] = {"value": v_tf, "unit": "TFLOP/s", "ms": v_avg_ms, "median_ms": v_med_ms,
                      "workload": f"packed prefill of 16 sequences, lengths U[128,2048] (T={sum(vlens)}), Hq=64 Hkv=8 D=128 fp16, causal within a sequence (BASELINE configs[4])",
-                     "roofline": {"bound": "mfma", "achieved": v_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": v_tf / PEAK_MFMA_TFLOPS,
-                                  "traffic": None, "kernel": "prefill_kernel<F16,128,varlen>", "algorithmic_flops": vflops}}
+                     "roofline": mfma_roofline(v_tf, sus_f16, traffic=RAGGED_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
+                                               kernel="prefill_kernel<F16,128,varlen>", algorithmic_flops=vflops)}
     rec["rope_kv_append_q8_0"] = {"value": a8_gbs, "unit": "GB/s", "ms": a8_avg_ms, "median_ms": a8_med_ms,
                                   "workload": "the rope_kv_append workload into Q8_0 caches, uint8 [8,8,4096,136]",
                                   "roofline": {"bound": "hbm", "achieved": a8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": a8_gbs / PEAK_HBM_GBS,
@@ -404,12 +500,17 @@ def main():
                                                "traffic": APPEND_NORM_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "rope_norm_append_kernel<F16,neox>", "algorithmic_bytes": abytes}}
     rec["qkv"] = {"value": p_tf, "unit": "TFLOP/s", "ms": p_avg_ms, "median_ms": p_med_ms,
                   "workload": "q,k,v = x wq^T, x wk^T, x wv^T in one launch: x [1,4096,4096], wq [4096,4096], wk and wv [1024,4096] fp16 (Llama-3-8B prefill)",
-                  "roofline": {"bound": "mfma", "achieved": p_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": p_tf / PEAK_MFMA_TFLOPS,
-                               "traffic": QKV_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_kernel<F16,[N,K],256x256,grouped>", "algorithmic_flops": pflops}}
+                  "roofline": mfma_roofline(p_tf, sus_f16, traffic=QKV_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
+                                            kernel="gemm_kernel<F16,[N,K],256x256,grouped>", algorithmic_flops=pflops)}
     rec["gemm_q8_0"] = {"value": q8_gbs, "unit": "GB/s", "ms": q8_avg_ms, "median_ms": q8_med_ms,
                         "workload": "one token against a weight of Q8_0 blocks: x [1,1,4096] fp16, W uint8 [14336, 4352] (Llama-3-8B FFN up), out fp16",
                         "roofline": {"bound": "hbm", "achieved": q8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": q8_gbs / PEAK_HBM_GBS,
-                                     "traffic": None, "kernel": "gemm_skinny_q8_kernel<1,1>", "algorithmic_bytes": q8bytes}}
+                                     "traffic": GEMM_Q8_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_skinny_q8_kernel<1,1>", "algorithmic_bytes": q8bytes}}
+    rec["cpu_plumbing"] = {"value": cflops / (c_avg_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms": c_avg_ms, "median_ms": c_med_ms,
+                           "workload": "prefill B=1 Hq=8 Hkv=2 S=256 D=64 causal dense-mask, fp32 inputs rounded to fp16 for the GPU op (BASELINE configs[0]); launch-bound"}
+    rec["calibration"] = {"mfma_only_f16_random": sus_f16, "mfma_only_bf16_random": sus_bf16,
+                          "note": "v_mfma_f32_32x32x16 alone, two waves per SIMD on every compute unit, operands 0.5*N(0,1); "
+                                  "frac_of_sustained = achieved / this, reported beside frac (= achieved / nominal peak)"}
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,
                       "workload": "rmsnorm per token, x [8,4096,6144] fp16, eps 1e-6 (reference test/kernels.py:59-74)",
                       "roofline": {"bound": "hbm", "achieved": n_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": n_gbs / PEAK_HBM_GBS,
@@ -417,10 +518,14 @@ def main():
     rec["gemm"] = {"value": g_tf, "unit": "TFLOP/s", "ms": g_avg_ms, "median_ms": g_med_ms,
                    "workload": "gemm alpha=1 beta=0, A [1,4096,4096] x W [4096,4096] fp16 (reference README HGEMM table, M=K=N=4096)",
                    "published_reference_us": 605.3,
-                   "roofline": {"bound": "mfma", "achieved": g_tf, "peak": PEAK_MFMA_TFLOPS, "unit": "TFLOP/s", "frac": g_tf / PEAK_MFMA_TFLOPS,
-                                "traffic": GEMM_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_kernel<F16,[K,N],256x256>", "algorithmic_flops": gflops}}
+                   "roofline": mfma_roofline(g_tf, sus_f16, traffic=GEMM_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
+                                             kernel="gemm_kernel<F16,[K,N],256x256>", algorithmic_flops=gflops)}
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
+        rec["decode"]["cpu_baseline"] = cpu_baseline_decode(torch, workloads, refs)
+        rec["ragged"]["cpu_baseline"] = cpu_baseline_ragged(torch, workloads, refs)
+        rec["long_context"]["cpu_baseline"] = cpu_baseline_long(torch, workloads, refs)
+        rec["cpu_plumbing"]["cpu_baseline"] = cpu_baseline_plumbing(torch, workloads, refs)
         rec["rope"]["cpu_baseline"] = rope_cpu_baseline(torch, workloads, refs)
     print(json.dumps(rec))
 

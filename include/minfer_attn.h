@@ -96,7 +96,9 @@ int minfer_flash_attn_decode(int dtype, const void* q, const void* k_cache, cons
  * MINFER_ATTN_EWORKSPACE (nothing launched).  The call allocates and frees nothing.  Its first call on a device
  * looks the array's address up (which may load the code object): make that call outside a graph capture.  All calls
  * on one GPU share the array: calls that overlap in time on one GPU (two streams, two threads) race; calls that
- * follow each other on one stream do not.  Arguments, results and errors are otherwise those of
+ * follow each other on one stream do not.  The array used is the copy on the device that owns `stream` (the
+ * current device for the null stream); that device must be the current one, a stream of another device is
+ * rejected with MINFER_ATTN_EINVAL.  Arguments, results and errors are otherwise those of
  * minfer_flash_attn_decode (16-bit caches only).
  */
 #define MINFER_DECODE_NOALLOC_SCRATCH_BYTES (64u << 20)
@@ -111,6 +113,11 @@ int minfer_flash_attn_decode_noalloc(int dtype, const void* q, const void* k_cac
  * cu_seqlens[s]..cu_seqlens[s+1]-1 form sequence s and attend causally inside it only.
  * Equals minfer_flash_attn with B = 1, L = T under the block-diagonal causal mask.  Needs no
  * workspace.  No counterpart in the reference; strides->q0, kv0, o0 are ignored.
+ * max_seqlen: an upper bound of the sequence lengths (0 = not known); it sizes the launch and selects the
+ * workgroup shape, and rows of a sequence past max_seqlen are not computed.  cu_seqlens is read on the
+ * device only and is not trusted: every sequence is cut to its part inside [0, T) and an end before its
+ * start is an empty sequence, so malformed entries (decreasing, negative, past T) cannot cause an access
+ * outside q/k/v/out; which rows such a call computes is unspecified beyond that, valid ones excepted.
  */
 int minfer_flash_attn_varlen(int dtype, const void* q, const void* k, const void* v,
                              const int32_t* cu_seqlens, int64_t n_seqs, int64_t max_seqlen,
@@ -314,6 +321,18 @@ int minfer_rope_kv_append_q8_0(int dtype, int style, void* q, const void* k, con
                                int64_t B, int64_t L, int64_t Hq, int64_t Hkv, int64_t D, int64_t Lmax,
                                int64_t cache_stride_b, int64_t cache_stride_h,
                                int64_t rotary_dim, double freq_base, void* stream);
+
+/*
+ * Calibration, not an operator (no counterpart in the reference): `workgroups` workgroups of 8 waves issue
+ * 8 * iters v_mfma_f32_32x32x16 (f16 or bf16) each, back to back on four accumulators, from 16 operand fragments
+ * (64 lanes x 16 bytes each, 16 KiB in all) that every wave reads once from `operands`; 32 768 flop per instruction,
+ * i.e. workgroups * 8 * 8 * iters * 32768 flop per launch.  Timed by the caller, it gives the matrix rate the chip
+ * sustains on the caller's operand values (random values cost more power than constant ones), the figure the
+ * attention and GEMM kernels' fractions of the nominal peak can be read against.  sink: workgroups * 512 floats.
+ */
+#define MINFER_CALIB_MFMA_OPERAND_BYTES 16384
+#define MINFER_CALIB_MFMA_FLOP_PER_ITER (8 * 8 * 32768)   /* per workgroup */
+int minfer_calib_mfma_rate(int dtype, const void* operands, int64_t iters, int64_t workgroups, float* sink, void* stream);
 
 #ifdef __cplusplus
 }

@@ -205,8 +205,28 @@ def gemm(backend: str, which: str):
            make, which)
 
 
+def mfma_rate(backend: str, which: str):
+    """Calibration, not an operator: the rate the chip sustains on v_mfma_f32_32x32x16 alone (two waves per SIMD on
+    every compute unit, nothing else in the loop), for random, constant and zero operand values, fp16 and bf16.  `ref`
+    runs torch.matmul (the vendor library) at 8192^3 for comparison.  The nominal dense peak is 2500 TFLOP/s."""
+    import calibration
+    if which == "minfer":
+        print(f"{'dtype':<10}{'operands':<12}{'TFLOP/s':>10}{'of 2500':>10}   (launches of ~5 ms back to back, 200 ms timed after 150 ms of warm-up)")
+        for dtype in (torch.float16, torch.bfloat16):
+            for kind in ("random", "constant", "zero"):
+                r = calibration.mfma_rate(dtype, kind)
+                print(f"{r['dtype']:<10}{kind:<12}{r['tflops']:>10.1f}{r['tflops'] / 2500.0:>10.3f}")
+    else:
+        results = []
+        for dtype in (torch.float16, torch.bfloat16):
+            a = (0.5 * torch.randn(8192, 8192, device="cuda")).to(dtype)
+            b = (0.5 * torch.randn(8192, 8192, device="cuda")).to(dtype)
+            results.append(_measure(lambda: torch.matmul(a, b), f"torch.matmul 8192^3 {str(dtype).split('.')[-1]} (1.0995e12 flop)", which, "mfma_rate"))
+        Compare(results).print()
+
+
 if __name__ == "__main__":
-    KERNELS = {"flash_attn": flash_attn, "flash_attn_operand_data": flash_attn_operand_data, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
+    KERNELS = {"mfma_rate": mfma_rate, "flash_attn": flash_attn, "flash_attn_operand_data": flash_attn_operand_data, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
                "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "rmsnorm": rmsnorm, "il_rope": il_rope, "neox_rope": neox_rope,
                "rope_kv_append": rope_kv_append, "gemm": gemm}
     parser = argparse.ArgumentParser()

@@ -1,0 +1,73 @@
+"""Calibration measurements next to the operator benchmarks: what the chip sustains on the matrix instruction
+alone.  Calls the library's calibration entry point (include/minfer_attn.h: minfer_calib_mfma_rate) through ctypes;
+it is not an operator and has no counterpart in the reference."""
+import ctypes
+import os
+
+import torch
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(os.path.dirname(HERE), "lib", "libminfer_attn.so")
+DTYPE_CODE = {torch.float16: 1, torch.bfloat16: 30}
+OPERAND_BYTES = 16384
+FLOP_PER_ITER = 8 * 8 * 32768     # per workgroup
+
+_lib = None
+
+
+def _load():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise RuntimeError(f"{LIB_PATH} is not built; run python minfer-python_amd/build.py")
+        _lib = ctypes.CDLL(LIB_PATH)
+        _lib.minfer_calib_mfma_rate.restype = ctypes.c_int
+        _lib.minfer_calib_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+        _lib.minfer_attn_last_error.restype = ctypes.c_char_p
+    return _lib
+
+
+def mfma_operands(dtype, kind: str, device="cuda", seed=0):
+    """16 KiB of operand fragments: 'random' = 0.5 * N(0,1) (the value distribution of the prefill benchmarks),
+    'constant' = every element 0.25, 'zero'."""
+    n = OPERAND_BYTES // 2
+    if kind == "random":
+        g = torch.Generator().manual_seed(seed)
+        return (0.5 * torch.randn(n, generator=g)).to(dtype).to(device)
+    if kind == "constant":
+        return torch.full((n,), 0.25, dtype=dtype, device=device)
+    if kind == "zero":
+        return torch.zeros(n, dtype=dtype, device=device)
+    raise ValueError(f"unknown operand kind {kind}")
+
+
+def launch_mfma_rate(operands, iters: int, workgroups: int, sink):
+    rc = _load().minfer_calib_mfma_rate(DTYPE_CODE[operands.dtype], operands.data_ptr(), iters, workgroups, sink.data_ptr(),
+                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+    if rc != 0:
+        raise RuntimeError(_load().minfer_attn_last_error().decode())
+
+
+def mfma_rate(dtype=torch.float16, kind="random", timed_ms=200.0, prewarm_ms=150.0, device="cuda"):
+    """Sustained rate of v_mfma_f32_32x32x16 on the whole chip, TFLOP/s: one workgroup of 8 waves per compute unit,
+    launches of ~5 ms run back to back for `prewarm_ms` (the clocks settle), then for `timed_ms` between two events."""
+    ops = mfma_operands(dtype, kind, device)
+    wgs = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(wgs * 512, dtype=torch.float32, device=device)
+    a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    iters = 2000
+    launch_mfma_rate(ops, iters, wgs, sink)
+    a.record(); launch_mfma_rate(ops, iters, wgs, sink); b.record(); b.synchronize()
+    iters = max(100, int(iters * 5.0 / max(a.elapsed_time(b), 1e-3)))          # ~5 ms per launch
+    per_launch_ms = 5.0
+    for _ in range(max(1, int(prewarm_ms / per_launch_ms))):
+        launch_mfma_rate(ops, iters, wgs, sink)
+    n = max(1, int(timed_ms / per_launch_ms))
+    a.record()
+    for _ in range(n):
+        launch_mfma_rate(ops, iters, wgs, sink)
+    b.record(); b.synchronize()
+    ms = a.elapsed_time(b) / n
+    flop = float(wgs) * iters * FLOP_PER_ITER
+    return {"tflops": flop / (ms * 1e-3) / 1e12, "ms_per_launch": ms, "iters": iters, "workgroups": wgs, "launches": n,
+            "operands": kind, "dtype": str(dtype).replace("torch.", "")}

@@ -224,6 +224,26 @@ def qkv(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def gemm_q8_0(backend: str, which: str, workload: str, repeat: int):
+    """A decode step's projection against a weight kept as Q8_0 blocks: one token x [1,1,4096] against W uint8
+    [14336, 4352] (Llama-3-8B FFN up; the reference routes this case to an empty launcher, gemm/op.cuh:199-210).
+    `ref` multiplies with the dequantised fp16 weight."""
+    kerns = KernelBackend(backend)
+    q8 = GGMLQuantizationType.Q8_0
+    wf = workloads.gemm_input(16, 14336, 4096, seed=3, device="cuda")[1].t().contiguous()
+    wq8 = torch.empty(14336, 4096 // 32 * 34, dtype=torch.uint8, device="cuda")
+    kerns._quant(q8, *GGML_QUANT_SIZES[q8], wf, wq8)
+    x = workloads.gemm_input(1, 16, 4096, seed=4, device="cuda")[0]
+    out = torch.zeros(1, 1, 14336, dtype=torch.float16, device="cuda")
+    if which == "minfer":
+        fn = lambda: kerns.gemm(q8, *GGML_QUANT_SIZES[q8], 1.0, 0.0, x, wq8, out, out)
+    else:
+        fn = lambda: kerns.gemm(QT, QB, QS, 1.0, 0.0, x, wf, out, out)
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def copy(backend: str, which: str, workload: str, repeat: int):
     """A plain device-to-device copy of 1 GiB: the known-size kernel that HBM byte counters
     (FETCH_SIZE / WRITE_SIZE) are calibrated against."""
@@ -234,8 +254,24 @@ def copy(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def mfma_rate(backend: str, which: str, workload: str, repeat: int):
+    """Calibration like `copy`: the library's matrix-instruction-only loop (v_mfma_f32_32x32x16_f16, two waves per SIMD
+    on every compute unit), ~5 ms per launch, on random operand values (--workload reference: constant ones).  The
+    kernel's duration in a trace, or MFMA counters over it, give the rate the matrix pipes sustain when nothing else
+    runs: 256 workgroups x 8 waves x 8 x iters instructions of 32 768 flop."""
+    import calibration
+    ops = calibration.mfma_operands(torch.float16, "constant" if workload == "reference" else "random")
+    wgs = torch.cuda.get_device_properties(0).multi_processor_count
+    sink = torch.empty(wgs * 512, dtype=torch.float32, device="cuda")
+    iters = 40000
+    print(f"mfma_rate: {wgs} workgroups x {iters} iterations = {wgs * iters * calibration.FLOP_PER_ITER:.4e} flop per launch")
+    for _ in range(repeat):
+        calibration.launch_mfma_rate(ops, iters, wgs, sink)
+    torch.cuda.synchronize()
+
+
 if __name__ == "__main__":
-    KERNELS = {"flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
+    KERNELS = {"mfma_rate": mfma_rate, "gemm_q8_0": gemm_q8_0, "flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
                "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "il_rope": il_rope, "rope_kv_append": rope_kv_append,
                "rope_kv_append_q8_0": rope_kv_append_q8_0, "rope_kv_append_norm": rope_kv_append_norm, "qkv": qkv, "quant": quant, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
     parser = argparse.ArgumentParser()

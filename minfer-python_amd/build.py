@@ -23,7 +23,7 @@ EXT_SO = os.path.join(EXT_DIR, "_C.so")
 HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibility=hidden",
              "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
              "-I" + os.path.join(ROOT, "include"), "-I" + CSRC]
-KERNEL_SOURCES = ["attn_prefill.hip", "attn_decode.hip", "rope.hip", "rmsnorm.hip", "gemm.hip", "quant.hip", "attn_api.hip"]
+KERNEL_SOURCES = ["attn_prefill.hip", "attn_decode.hip", "rope.hip", "rmsnorm.hip", "gemm.hip", "quant.hip", "calib.hip", "attn_api.hip"]
 
 
 def _run(cmd):

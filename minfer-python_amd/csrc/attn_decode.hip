@@ -823,12 +823,23 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode_q8_0(const void* q, const void* 
 namespace minfer_attn {
 static __device__ __align__(256) unsigned char scratch[MINFER_DECODE_NOALLOC_SCRATCH_BYTES];
 
-static int decode_scratch(void** ptr_out) {
+// The kernels run on the device that owns the caller's stream, so that device's copy of the array is the one to
+// hand them.  The address is looked up once per device, with that device current (hipGetSymbolAddress answers for
+// the current device); a stream that belongs to another device than the current one is refused, as a launch on it
+// would be.
+static int decode_scratch(hipStream_t stream, void** ptr_out) {
     static std::mutex mu;
     static void* ptrs[64] = {nullptr};
-    int dev = 0;
-    if (hipGetDevice(&dev) != hipSuccess) return fail(MINFER_ATTN_ELAUNCH, "flash_attn_decode_noalloc: hipGetDevice failed");
+    int cur = 0, dev = 0;
+    if (hipGetDevice(&cur) != hipSuccess) return fail(MINFER_ATTN_ELAUNCH, "flash_attn_decode_noalloc: hipGetDevice failed");
+    dev = cur;
+    if (stream) {   // the null stream belongs to the current device
+        hipDevice_t sd = 0;
+        if (hipStreamGetDevice(stream, &sd) != hipSuccess) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: hipStreamGetDevice failed for the given stream");
+        dev = (int)sd;
+    }
     if (dev < 0 || dev >= 64) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: device index above 63 unsupported");
+    if (dev != cur) return fail(MINFER_ATTN_EINVAL, "flash_attn_decode_noalloc: the stream belongs to another device than the current one (hipSetDevice to the stream's device before the call)");
     std::lock_guard<std::mutex> lock(mu);
     if (!ptrs[dev]) {
         void* ptr = nullptr;
@@ -862,7 +873,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_decode_noalloc(int dtype, const void* q
         return MINFER_ATTN_EWORKSPACE;
     }
     void* ws = nullptr;
-    if (int rc = decode_scratch(&ws)) return rc;
+    if (int rc = decode_scratch((hipStream_t)stream_v, &ws)) return rc;
     DecodeParams p{};
     if (int rc = fill_decode(p, q, k_cache, v_cache, ctx_lens, B, Hq, Hkv, Lmax, D, st, ws,
                              (size_t)MINFER_DECODE_NOALLOC_SCRATCH_BYTES, kGroupRows)) return rc;

@@ -156,6 +156,7 @@ struct PrefillParams {
     int NQT, NKT;          // dense: 64-row query / key tile counts of the mask classification
     int NQ;                // workgroup-level query tiles (dense: exact; varlen: upper bound)
     int n_seqs;
+    int max_len;           // varlen: rows of a sequence past this many are not computed (>= every length for a valid call)
     int mask_vec;          // dense: mask rows may be read as aligned 32-bit words
     float scale_log2;      // softmax scale * log2(e)
 };
@@ -226,8 +227,14 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         bool found = false;
         for (int base = 0; base < p.n_seqs && !found; base += 64) {
             const int sq = base + lane;
-            const int lo = sq < p.n_seqs ? p.cu[sq] : 0;
-            const int len = sq < p.n_seqs ? p.cu[sq + 1] - lo : 0;
+            // cu_seqlens is device data nobody has checked: every sequence is cut to the part of it that lies
+            // inside the packed tensors ([0, L) rows) and to max_seqlen rows, and an end before its start is an
+            // empty sequence, so no entry can produce an address outside q/k/v/out or a negative tile count.
+            int lo = 0, len = 0;
+            if (sq < p.n_seqs) {
+                lo = min(max(p.cu[sq], 0), p.L);
+                len = min(min(max(p.cu[sq + 1], lo), p.L) - lo, p.max_len);
+            }
             const int n = (len + 32 * QBW - 1) / (32 * QBW);
             const int incl = wave_inclusive_scan(n, lane);
             const int total = __builtin_amdgcn_readfirstlane(__shfl(incl, 63));
@@ -720,8 +727,16 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const 
     p.L = (int)T; p.B = 1;
     p.NQT = p.NKT = 0;
     const int rows_per_wg = 32 * (kWaves >> p.hpw_log2);
-    p.NQ = (int)((T + rows_per_wg - 1) / rows_per_wg + n_seqs);  // >= sum over sequences of ceil(len / rows_per_wg)
+    // max_seqlen 0 means "not known".  Rows of a sequence past max_seqlen are not computed, so a caller's bound
+    // must be at least the longest sequence (as in every varlen attention interface).
+    const int64_t max_len = (max_seqlen > 0 && max_seqlen < T) ? max_seqlen : T;
+    // query tiles: sum over sequences of ceil(len / rows_per_wg) <= both bounds below (cu_seqlens lives on the device,
+    // so the exact count is not known here; workgroups past it exit at once)
+    const int64_t nq_packed = (T + rows_per_wg - 1) / rows_per_wg + n_seqs;
+    const int64_t nq_each = n_seqs * ((max_len + rows_per_wg - 1) / rows_per_wg);
+    p.NQ = (int)(nq_each < nq_packed ? nq_each : nq_packed);
     p.n_seqs = (int)n_seqs;
+    p.max_len = (int)max_len;
     const int64_t grid = (int64_t)p.NQ * Hkv * p.n_hg;
     if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: problem too large for one launch");
     return dispatch_prefill<MODE_VARLEN>(dtype, D, p, (int)grid, stream);

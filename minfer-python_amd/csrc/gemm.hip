@@ -428,9 +428,11 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_q8_kernel(const
         uint32_t wq[NR][9];
 #pragma unroll
         for (int nr = 0; nr < NR; ++nr) {
+            // four words per load, at addresses that are only word-aligned: the vector type says so
+            typedef uint32_t u32x4_w __attribute__((ext_vector_type(4), aligned(4)));
             const uint32_t* src = reinterpret_cast<const uint32_t*>(wrow[nr] + (int64_t)bc * 34 - (odd ? 2 : 0));
-            const u32x4 a = *reinterpret_cast<const u32x4*>(src);
-            const u32x4 b = *reinterpret_cast<const u32x4*>(src + 4);
+            const u32x4_w a = *reinterpret_cast<const u32x4_w*>(src);
+            const u32x4_w b = *reinterpret_cast<const u32x4_w*>(src + 4);
             wq[nr][0] = a[0]; wq[nr][1] = a[1]; wq[nr][2] = a[2]; wq[nr][3] = a[3];
             wq[nr][4] = b[0]; wq[nr][5] = b[1]; wq[nr][6] = b[2]; wq[nr][7] = b[3];
             wq[nr][8] = src[8];
@@ -439,7 +441,8 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_q8_kernel(const
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
-            for (int j = 0; j < 4; ++j) x[mb][j] = *reinterpret_cast<const s16x8*>(xrow[mb] + 32 * bc + 8 * j);
+            for (int j = 0; j < 4; ++j)   // a lane past the last block contributes exact zeros, whatever block 0 or 1 holds
+                x[mb][j] = real ? *reinterpret_cast<const s16x8*>(xrow[mb] + 32 * bc + 8 * j) : s16x8{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int nr = 0; nr < NR; ++nr) {
             const uint16_t bits = (uint16_t)(odd ? wq[nr][0] >> 16 : wq[nr][0]);
@@ -716,12 +719,18 @@ constexpr int64_t kQ8SkinnyRows = 64;    // up to here the kernel that streams t
 
 static size_t q8_dequant_bytes(int64_t N, int64_t K) { return ((size_t)N * (size_t)K * 2 + 255) & ~(size_t)255; }
 
-// the streaming kernel takes up to 64 rows and needs weight rows that are multiples of 4 bytes (an even number of blocks)
-static bool q8_streams(int64_t M, int64_t K) { return M <= kQ8SkinnyRows && (K / 32) % 2 == 0; }
+// the streaming kernel takes up to 64 rows, needs weight rows that are multiples of 4 bytes (an even number of blocks)
+// and stores 8-byte pieces of D (N a multiple of 4); every other shape goes through the dequantised weight
+static bool q8_streams(int64_t M, int64_t N, int64_t K) { return M <= kQ8SkinnyRows && (K / 32) % 2 == 0 && N % 4 == 0; }
+// ... and it reads 16-byte pieces of A and aligned 8-byte pieces of C (only when beta != 0) and D
+static bool q8_stream_operands(const void* A, const void* C, const void* D, int64_t lda, int64_t ldc, int64_t ldd, double beta) {
+    return aligned16(A) && lda % 8 == 0 && ldd % 4 == 0 && ((uintptr_t)D & 7u) == 0 &&
+           (beta == 0.0 || (ldc % 4 == 0 && ((uintptr_t)C & 7u) == 0));
+}
 
 MINFER_ATTN_EXPORT size_t minfer_gemm_q8_0_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
-    if (q8_streams(M, K)) return 0;
+    if (q8_streams(M, N, K)) return 0;
     return q8_dequant_bytes(N, K) + minfer_gemm_workspace_bytes(M, N, K);
 }
 
@@ -739,19 +748,18 @@ MINFER_ATTN_EXPORT int minfer_gemm_q8_0(const void* A, const void* Bq, const voi
     hipStream_t stream = (hipStream_t)stream_v;
     const int64_t row_bytes = K / 32 * 34;
     if (((uintptr_t)Bq & 3u) != 0) return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: the weight must be 4-byte aligned");
-    if (q8_streams(M, K)) {
-        // the streaming kernel reads aligned words of the weight, 16-byte pieces of A, and stores 8-byte pieces of D
-        if (!aligned16(A) || lda % 8 != 0 || ldc % 4 != 0 || ldd % 4 != 0 || ((uintptr_t)D & 7u) != 0 || ((uintptr_t)C & 7u) != 0 || N % 4 != 0)
-            return fail(MINFER_ATTN_EINVAL, "gemm_q8_0: A must be 16-byte aligned with lda a multiple of 8; C, D 8-byte aligned with strides and N multiples of 4");
+    if (q8_streams(M, N, K) && q8_stream_operands(A, C, D, lda, ldc, ldd, beta)) {
         GemmParams p{};
-        p.A = A; p.B = Bq; p.C = C; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
+        p.A = A; p.B = Bq; p.C = beta != 0.0 ? C : nullptr; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
         p.lda = lda; p.ldb = row_bytes; p.ldc = ldc; p.ldd = ldd; p.alpha = (float)alpha; p.beta = (float)beta;
         return launch_skinny_q8(p, stream);
     }
     // otherwise: the weight as fp16 in the workspace, then the fp16 kernels on it
     const size_t deq = q8_dequant_bytes(N, K);
     if (!workspace || !aligned16(workspace) || workspace_bytes < deq)
-        return fail(MINFER_ATTN_EWORKSPACE, "gemm_q8_0: this shape needs a workspace of N*K*2 bytes (rounded up to 256) for the dequantised weight");
+        return fail(MINFER_ATTN_EWORKSPACE, "gemm_q8_0: this call needs a workspace of N*K*2 bytes (rounded up to 256) for the dequantised weight "
+                                            "(more than 64 rows, an odd number of blocks per row, N not a multiple of 4, or A/C/D not aligned for the streaming kernel: "
+                                            "A 16 bytes with lda a multiple of 8, C and D 8 bytes with strides multiples of 4)");
     if (int rc = minfer_dequant_q8_0(MINFER_ATTN_F16, Bq, workspace, N, K, stream_v)) return rc;
     return gemm_impl(MINFER_ATTN_F16, MINFER_GEMM_B_NK, A, workspace, C, D, M, N, K, lda, K, ldc, ldd, alpha, beta,
                      (char*)workspace + deq, workspace_bytes - deq, stream_v);

@@ -453,7 +453,12 @@ void gemm_hip(int64_t qtype_int, int64_t qblock_size, int64_t qtype_size, double
         STD_TORCH_CHECK(A.size(0) * A.size(1) == C.size(0) * C.size(1) && C.size(-1) == N, "gemm: C does not have the shape of A B^T");
         STD_TORCH_CHECK(C.sizes().equals(D.sizes()), "gemm: C and D shapes differ");
         STD_TORCH_CHECK(alpha != 0.0, "gemm: alpha must not be 0");
-        const size_t ws_bytes = minfer_gemm_q8_0_workspace_bytes(M, N, K);
+        size_t ws_bytes = minfer_gemm_q8_0_workspace_bytes(M, N, K);
+        // a view that starts off a 16-byte boundary cannot feed the kernel that streams the blocks: such a call goes
+        // through the dequantised weight like the shapes that kernel does not take
+        const auto misaligned = [](const void* ptr) { return (reinterpret_cast<uintptr_t>(ptr) & 15u) != 0; };
+        if (ws_bytes == 0 && (misaligned(A.const_data_ptr()) || misaligned(D.const_data_ptr()) || (beta != 0.0 && misaligned(C.const_data_ptr()))))
+            ws_bytes = ((static_cast<size_t>(N) * static_cast<size_t>(K) * 2 + 255) & ~static_cast<size_t>(255)) + minfer_gemm_workspace_bytes(M, N, K);
         Tensor ws = byte_workspace(A, ws_bytes);
         check_rc(minfer_gemm_q8_0(A.const_data_ptr(), B.const_data_ptr(), C.const_data_ptr(), D.mutable_data_ptr(), M, N, K, K, N, N,
                                   alpha, beta, ws_bytes ? ws.mutable_data_ptr() : nullptr, ws_bytes, current_stream()),

@@ -16,11 +16,12 @@ class GGMLQuantizationType(IntEnum):
     BF16 = 30
 
 
-# (elements per block, bytes per block); reference: src/minfer/const.py:39-41.  The reference
-# lists BF16 as (256, 512) at const.py:67, the same bytes per element.
+# (elements per block, bytes per block); reference: src/minfer/const.py:39-41.  BF16 is (256, 512) as in
+# the reference's table (const.py:67): the same two bytes per element; the operators ignore the pair for
+# 16-bit types.
 GGML_QUANT_SIZES: dict[GGMLQuantizationType, tuple[int, int]] = {
     GGMLQuantizationType.F32: (1, 4),
     GGMLQuantizationType.F16: (1, 2),
     GGMLQuantizationType.Q8_0: (32, 2 + 32),   # reference: src/minfer/const.py:46
-    GGMLQuantizationType.BF16: (1, 2),
+    GGMLQuantizationType.BF16: (256, 512),
 }

@@ -267,6 +267,8 @@ def make_q8(M, N, K, seed):
     (65, 256, 256, 1.0, 2.0),        # above 64 rows: dequantise into the workspace, then the fp16 kernels
     (300, 1032, 512, 2.0, 0.0),
     (5, 64, 96, 1.0, 1.0),           # an odd number of blocks per row: workspace path at any row count
+    (3, 18, 256, 1.0, 1.0),          # out_dim not a multiple of 4 with few rows: workspace path as well
+    (64, 1030, 128, 2.0, 0.0),
 ])
 def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
     a, wq, c, w_deq = make_q8(M, N, K, seed=M * 7 + N + K)
@@ -274,7 +276,7 @@ def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
     da, dwq, dc = a.to(DEV), wq.to(DEV), c.to(DEV)
     d = torch.zeros(M, N, dtype=torch.float16, device=DEV)
     need = capi.lib().minfer_gemm_q8_0_workspace_bytes(M, N, K)
-    assert (need == 0) == (M <= 64 and (K // 32) % 2 == 0)
+    assert (need == 0) == (M <= 64 and (K // 32) % 2 == 0 and N % 4 == 0)
     ws = torch.full((max(need, 16),), 0xFF, dtype=torch.uint8, device=DEV)
     assert capi.gemm_q8_0(da, dwq, dc, d, alpha, beta, ws if need else None) == capi.OK, capi.last_error()
     assert_close(d, exact, torch.float16, "q8_0 weight")

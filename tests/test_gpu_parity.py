@@ -352,6 +352,46 @@ def test_varlen_matches_oracle_and_dense(dtype, Hq, Hkv, D, lens):
     assert max_err(out, dense) <= TOL[dtype] / 2 + one_ulp
 
 
+def test_varlen_malformed_cu_seqlens_stay_in_bounds():
+    """cu_seqlens lives on the device and is never checked by the host: a decreasing entry, a negative one and one
+    past T must not move any access outside q/k/v/out.  The tensors are views with guard rows on both sides of every
+    head (NaN in q/k/v, which would poison any result that read them; a sentinel in out); sequences that are valid
+    and overlap no other come out as the oracle computes them."""
+    Hq, Hkv, D, T, G = 8, 2, 128, 600, 96
+    g = torch.Generator().manual_seed(77)
+
+    def guarded(H, fill, scale=1.0):
+        buf = torch.full((1, H, T + 2 * G, D), fill, dtype=torch.float16)
+        buf[:, :, G:G + T] = (scale * torch.randn(1, H, T, D, generator=g)).to(torch.float16)
+        buf = buf.to(DEV)
+        return buf, buf[:, :, G:G + T]
+
+    qb, q = guarded(Hq, float("nan"))
+    kb, k = guarded(Hkv, float("nan"))
+    vb, v = guarded(Hkv, float("nan"), 0.5)
+    ob = torch.full((1, Hq, T + 2 * G, D), 7.0, dtype=torch.float16, device=DEV)
+    out = ob[:, :, G:G + T]
+    # sequence 0 = rows [0,200); 1 ends before it starts (empty); 2 = [150,400) overlaps the end of 0; 3 starts at 400
+    # and claims rows far past T (cut to [400,600)); 4 starts past T (empty); 5 has a negative start and end (empty)
+    cu = torch.tensor([0, 200, 150, 400, 2_000_000_000, -5, -3], dtype=torch.int32, device=DEV)
+    assert capi.flash_attn_varlen(q, k, v, cu, 0, out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert torch.all(ob[:, :, :G] == 7.0) and torch.all(ob[:, :, G + T:] == 7.0)     # guard rows of out untouched
+    assert not torch.isnan(out).any()                                                 # no guard row of q/k/v was read
+    qc, kc, vc = q.cpu(), k.cpu(), v.cpu()
+    for lo, hi, rows in [(0, 200, slice(0, 150)), (150, 400, slice(50, 250)), (400, 600, slice(0, 200))]:
+        want = oracle.flash_attn(qc[:, :, lo:hi], kc[:, :, lo:hi], vc[:, :, lo:hi], workloads.causal_mask(1, hi - lo))
+        assert max_err(out[:, :, lo:hi][:, :, rows], want[:, :, rows]) <= TOL[torch.float16]
+    # the same with max_seqlen given: rows of a sequence past it are left alone, the others are as before
+    ob.fill_(7.0)
+    assert capi.flash_attn_varlen(q, k, v, cu, 100, out) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert torch.all(ob[:, :, :G] == 7.0) and torch.all(ob[:, :, G + T:] == 7.0)
+    assert torch.all(out[:, :, 500:] == 7.0)                                          # rows 100.. of the last sequence
+    want = oracle.flash_attn(qc[:, :, 400:500], kc[:, :, 400:500], vc[:, :, 400:500], workloads.causal_mask(1, 100))
+    assert max_err(out[:, :, 400:500], want) <= TOL[torch.float16]
+
+
 # ------------------------------------------------------------------------------------------------
 # the registered torch ops (the reference's call path) give the same bits and the same errors
 # ------------------------------------------------------------------------------------------------

@@ -164,7 +164,10 @@ def test_gemm_q8_0_validation_rejects_before_launch():
     assert g(beta=1.0) == capi.EINVAL                                  # beta != 0 needs C
     assert g(lda=128) == capi.EINVAL and "leading" in capi.last_error()
     assert g(b=0x2002) == capi.EINVAL and "4-byte" in capi.last_error()
-    assert g(a=0x1008) == capi.EINVAL and "16-byte" in capi.last_error()   # the streaming kernel's alignment
+    # operands the streaming kernel cannot take (A off a 16-byte boundary, N not a multiple of 4) go through the
+    # dequantised weight, i.e. ask for the workspace instead of being refused
+    assert g(a=0x1008) == capi.EWORKSPACE and "not aligned" in capi.last_error()
+    assert g(N=18, ldc=18, ldd=18) == capi.EWORKSPACE
     assert g(M=100) == capi.EWORKSPACE and "workspace" in capi.last_error()   # more than 64 rows: needs the dequantised weight
     assert g(K=96, lda=96) == capi.EWORKSPACE                               # an odd number of blocks per row as well
     assert g(M=0) == capi.OK and g(N=0) == capi.OK and capi.last_error() == ""
@@ -172,6 +175,7 @@ def test_gemm_q8_0_validation_rejects_before_launch():
     assert ws(1, 4096, 4096) == 0 and ws(64, 14336, 4096) == 0
     assert ws(65, 4096, 4096) == 4096 * 4096 * 2 + L.minfer_gemm_workspace_bytes(65, 4096, 4096)
     assert ws(4, 64, 96) == (64 * 96 * 2 + 255) // 256 * 256 and ws(4, 64, 100) == 0 and ws(0, 64, 128) == 0
+    assert ws(4, 18, 256) == (18 * 256 * 2 + 255) // 256 * 256      # N not a multiple of 4: the query and the call agree
 
 
 def test_gemm_workspace_sizes():
@@ -233,6 +237,8 @@ def test_python_surface_matches_reference_names(kerns):
     import oracle
 
     assert GGMLQuantizationType.F16 == 1 and GGML_QUANT_SIZES[GGMLQuantizationType.F16] == (1, 2)
+    # the reference's table value for BF16 (reference: src/minfer/const.py:67), kept for callers that compare tables
+    assert GGMLQuantizationType.BF16 == 30 and GGML_QUANT_SIZES[GGMLQuantizationType.BF16] == (256, 512)
     assert list(inspect.signature(te.flash_attn).parameters) == [
         "qtype_int", "qblock_size", "qtype_size", "q", "k", "v", "mask", "out"]
     assert callable(kerns.flash_attn) and callable(kerns.flash_attn_decode) and callable(kerns.flash_attn_varlen)
