@@ -162,14 +162,17 @@ struct PrefillParams {
 };
 
 enum { MODE_DENSE = 0, MODE_VARLEN = 1 };
-constexpr int kWaves = 8;   // waves per workgroup
-constexpr int kThreads = kWaves * 64;
+// Waves per workgroup, a template argument of the kernel: 8 (one workgroup per compute unit: 256 query rows share every
+// K/V tile staged in LDS) or 4 (two workgroups per compute unit, 128 rows per tile: twice the tile copies per flop, but
+// one workgroup's prologue, epilogue and hand-over run under the other's tiles, which is what counts when sequences
+// are short).
+constexpr int kWavesBig = 8, kWavesSmall = 4;
 
-template <int D> struct TileGeom {
+template <int D, int NW> struct TileGeom {
     static constexpr int RB = D * 2;          // bytes per K/V row
     static constexpr int G = RB / 16;         // 16-byte granules per row
     static constexpr int RPI = 1024 / RB;     // rows one wave-wide copy instruction covers
-    static constexpr int NLD = 64 / (kWaves * RPI);  // copy instructions per wave, per tile, per tensor
+    static constexpr int NLD = 64 / (NW * RPI);  // copy instructions per wave, per tile, per tensor
     static constexpr int RPW = 256 / RB;      // rows per 256-byte bank window
     static constexpr int TILE_BYTES = 64 * RB;
     // XOR swizzles applied to the granule index of a row.  K is read 16 rows x one granule at a
@@ -179,24 +182,32 @@ template <int D> struct TileGeom {
     static MA_DEV int swz_v(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
 };
 
-template <class T, int D, int MODE>
-__global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParams p) {
-    using GEO = TileGeom<D>;
+template <class T, int D, int MODE, int NW>
+__global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams p) {
+    using GEO = TileGeom<D, NW>;
     constexpr int RB = GEO::RB, G = GEO::G, RPI = GEO::RPI, NLD = GEO::NLD;
     constexpr int KC = D / 16;   // 16-wide contraction chunks of Q K^T
     constexpr int DB = D / 32;   // 32-row blocks of O^T
+    constexpr int kWaves = NW;
+    constexpr int STAGE_BYTES = 2 * GEO::TILE_BYTES;   // a stage = the K tile followed by the V tile
+    constexpr int ROWS_BYTES = 32 * RB;                // a wave's 32 query (or output) rows
 
-    __shared__ __attribute__((aligned(1024))) char k_lds[2][GEO::TILE_BYTES];
-    __shared__ __attribute__((aligned(1024))) char v_lds[2][GEO::TILE_BYTES];
+    __shared__ __attribute__((aligned(1024))) char kv_lds[2][STAGE_BYTES];
     __shared__ uint32_t tile_list[MODE == MODE_DENSE ? kMaxKeyTiles : 1];
     __shared__ int n_active_s;
     // A wave's own 32 query rows on their way in (whole rows, copied global->LDS) and its 32 output rows on their way
-    // out (so that a store instruction writes whole rows): no other wave touches a wave's area, so it needs no barrier.
-    __shared__ __attribute__((aligned(1024))) char q_lds[kWaves][32 * GEO::RB];
+    // out (so that a store instruction writes whole rows).  With 8 waves the area is separate memory, the wave's own, so
+    // neither step needs a barrier.  With 4 waves (4 x ROWS_BYTES = one stage) it lies inside the K/V stages, which is
+    // what lets two workgroups fit a compute unit: the query rows in stage 1, which no tile copy touches before the
+    // barrier that opens tile 0 (by then every wave has its fragments in registers); the output rows in the stage the
+    // last tile did not use, which every wave finished reading before the barrier that opened the last tile.
+    constexpr bool kAliasRows = NW * ROWS_BYTES <= STAGE_BYTES;
+    __shared__ __attribute__((aligned(1024))) char q_lds_own[kAliasRows ? 1 : NW][kAliasRows ? 16 : ROWS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
     const int h = lane >> 5, l32 = lane & 31;
     const int HPW = 1 << p.hpw_log2, QBW = kWaves >> p.hpw_log2;  // heads, 32-row query blocks per workgroup
+    char* const q_stage = kAliasRows ? &kv_lds[1][w * ROWS_BYTES] : &q_lds_own[kAliasRows ? 0 : w][0];
 
     // ---- which (batch, KV head, head group, query tile) is this workgroup -------------------
     const int BG = p.B * p.Hkv;
@@ -274,7 +285,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     for (int j = 0; j < 32 / RPI; ++j) {
         const int row = j * RPI + lane / G, pg = lane % G;
         const short* src = Qh + (int64_t)min(q_row0 + row, last_row) * p.q2 + 8 * (pg ^ GEO::swz_k(row));
-        copy16_global_to_lds(src, &q_lds[w][j * RPI * RB]);
+        copy16_global_to_lds(src, q_stage + j * RPI * RB);
     }
 
     // ---- list of key tiles this workgroup visits ---------------------------------------------
@@ -309,30 +320,20 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
         n_active = (top_row >> 6) + 1;
     }
 
-    // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
-    // Q is multiplied by scale*log2(e) once, here, so that the MFMA accumulator of Q K^T is directly
-    // the base-2 exponent of the softmax weight (minus the running reference it is initialised with).
-    // (The rows were requested before the tile list was built.)
     const float c2 = p.scale_log2;
-    s16x8 qf[KC];
-    wait_vmcnt<0>();   // the wave's own rows have landed (nobody else reads them)
-    {
-        const uint32_t qa = lds_addr(&q_lds[w][0]) + l32 * RB;
-        const int sw = GEO::swz_k(l32);
-#pragma unroll
-        for (int c = 0; c < KC; ++c) qf[c] = T::scale8(lds_read_b128(qa + 16 * ((2 * c + h) ^ sw), 0), c2);
-    }
+    s16x8 qf[KC];   // the wave's query rows as B-operand fragments; filled once the first K/V tile has been requested
 
     // ---- global -> LDS tile copy ----------------------------------------------------------
-    // Instruction j of this wave fills rows (j*kWaves + w)*RPI .. +RPI-1 of the tile; the lane's byte
-    // offset from the tile's first key row is a constant (row and swizzled granule), so a full tile
-    // costs no vector ALU work: scalar base + constant per-lane offset.
-    uint32_t k_off[NLD], v_off[NLD];
-#pragma unroll
-    for (int j = 0; j < NLD; ++j) {
-        const int row = (j * kWaves + w) * RPI + lane / G, pg = lane % G;
-        k_off[j] = (uint32_t)((int64_t)row * p.kv2 + 8 * (pg ^ GEO::swz_k(row))) * 2u;
-        v_off[j] = (uint32_t)((int64_t)row * p.kv2 + 8 * (pg ^ GEO::swz_v(row))) * 2u;
+    // Instruction j of this wave fills rows (j*kWaves + w)*RPI .. +RPI-1 of the tile.  The lane's byte offset from the
+    // first of the instruction's rows is a constant (row and swizzled granule; kWaves*RPI is a multiple of every
+    // swizzle period, so it is the same for every j), and the instruction's first row goes into the scalar base: a
+    // full tile costs no vector ALU work.
+    static_assert((kWaves * RPI) % 16 == 0, "the swizzles repeat every 16 rows at most");
+    uint32_t k_off0, v_off0;
+    {
+        const int row = w * RPI + lane / G, pg = lane % G;
+        k_off0 = (uint32_t)((int64_t)(lane / G) * p.kv2 + 8 * (pg ^ GEO::swz_k(row))) * 2u;
+        v_off0 = (uint32_t)((int64_t)(lane / G) * p.kv2 + 8 * (pg ^ GEO::swz_v(row))) * 2u;
     }
     auto issue_tile = [&](int kt, int stage) {
         const int key0 = kt * 64;
@@ -342,8 +343,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
 #pragma unroll
             for (int j = 0; j < NLD; ++j) {
                 const int row0 = (j * kWaves + w) * RPI;
-                copy16_global_to_lds(kbase, k_off[j], &k_lds[stage][row0 * RB]);
-                copy16_global_to_lds(vbase, v_off[j], &v_lds[stage][row0 * RB]);
+                copy16_global_to_lds(kbase + (int64_t)row0 * p.kv2, k_off0, &kv_lds[stage][row0 * RB]);
+                copy16_global_to_lds(vbase + (int64_t)row0 * p.kv2, v_off0, &kv_lds[stage][GEO::TILE_BYTES + row0 * RB]);
             }
         } else {   // tile crossing the end of the sequence: rows past it re-read the last row
 #pragma unroll
@@ -351,8 +352,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
                 const int row0 = (j * kWaves + w) * RPI;
                 const int row = row0 + lane / G, pg = lane % G;
                 const int64_t grow = (int64_t)(min(key0 + row, last_row) - key0) * p.kv2;
-                copy16_global_to_lds(kbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_k(row))) * 2u, &k_lds[stage][row0 * RB]);
-                copy16_global_to_lds(vbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_v(row))) * 2u, &v_lds[stage][row0 * RB]);
+                copy16_global_to_lds(kbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_k(row))) * 2u, &kv_lds[stage][row0 * RB]);
+                copy16_global_to_lds(vbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_v(row))) * 2u, &kv_lds[stage][GEO::TILE_BYTES + row0 * RB]);
             }
         }
     };
@@ -366,13 +367,13 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     {
         const int sw = GEO::swz_k(l32);
 #pragma unroll
-        for (int c = 0; c < KC; ++c) k_rd[c] = lds_addr(&k_lds[0][0]) + l32 * RB + 16 * ((2 * c + h) ^ sw);
+        for (int c = 0; c < KC; ++c) k_rd[c] = lds_addr(&kv_lds[0][0]) + l32 * RB + 16 * ((2 * c + h) ^ sw);
         const int vrow = 4 * h + (li >> 2);
         const int swv = GEO::swz_v(vrow);
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
             const int dcol = 32 * db + 16 * (blk & 1) + 4 * (li & 3);
-            v_rd[db] = lds_addr(&v_lds[0][0]) + vrow * RB + 16 * ((dcol >> 3) ^ swv) + 2 * (dcol & 7);
+            v_rd[db] = lds_addr(&kv_lds[0][GEO::TILE_BYTES]) + vrow * RB + 16 * ((dcol >> 3) ^ swv) + 2 * (dcol & 7);
         }
     }
 
@@ -431,7 +432,7 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     // ---- one key tile, K/V in LDS stage STAGE (compile-time, so every LDS address is base + immediate) ----
     auto process_tile = [&](auto stage_tag, int kt, uint32_t cls_w) {
         constexpr int STAGE = decltype(stage_tag)::value;
-        constexpr int SOFF = STAGE * GEO::TILE_BYTES;
+        constexpr int SOFF = STAGE * STAGE_BYTES;
         const int key0 = kt * 64;
 
         // S^T = K Q^T, accumulated on top of -reference: register r of block kb is key 32kb + 8(r/4) + 4h + r%4.
@@ -561,12 +562,24 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     // ---- main loop: one barrier per tile; the copy of tile t+1 is issued right after the barrier that
     // opens tile t, into the stage tile t-1 has just vacated ---------------------------------------
     uint32_t e_cur = list_entry(0), e_next = list_entry(1);
+    int kt_first = 0; uint32_t cls_first = TILE_NONE;
     if (n_active > 0) {
-        int kt0; uint32_t c0;
-        tile_of(e_cur, 0, kt0, c0);
-        issue_tile(kt0, 0);
-        if (MODE == MODE_DENSE && c0 == TILE_MIXED) fetch_mask(kt0);
+        tile_of(e_cur, 0, kt_first, cls_first);
+        issue_tile(kt_first, 0);
     }
+    // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
+    // Q is multiplied by scale*log2(e) once, here, so that the MFMA accumulator of Q K^T is directly
+    // the base-2 exponent of the softmax weight (minus the running reference it is initialised with).
+    // The rows were requested before the tile list was built, and the first K/V tile after them: copies retire in
+    // order, so the rows have landed once no more than that tile's copies are outstanding.
+    if (n_active > 0) wait_vmcnt<2 * NLD>(); else wait_vmcnt<0>();
+    {
+        const uint32_t qa = lds_addr(q_stage) + l32 * RB;
+        const int sw = GEO::swz_k(l32);
+#pragma unroll
+        for (int c = 0; c < KC; ++c) qf[c] = T::scale8(lds_read_b128(qa + 16 * ((2 * c + h) ^ sw), 0), c2);
+    }
+    if (MODE == MODE_DENSE && n_active > 0 && cls_first == TILE_MIXED) fetch_mask(kt_first);
     auto iteration = [&](auto stage_tag, int it) {
         constexpr int STAGE = decltype(stage_tag)::value;
         int kt, ktn; uint32_t cls_w, cn;
@@ -594,7 +607,8 @@ __global__ __launch_bounds__(kThreads, 2) void prefill_kernel(const PrefillParam
     const float l = sum_across_halves(l_sum);
     const float inv = l > 0.f ? 1.f / l : 0.f;
     {
-        const uint32_t so = lds_addr(&q_lds[w][0]);
+        const int free_stage = (n_active & 1);   // the last tile sat in stage (n_active - 1) & 1
+        const uint32_t so = kAliasRows ? lds_addr(&kv_lds[0][0]) + free_stage * STAGE_BYTES + w * ROWS_BYTES : lds_addr(q_stage);
         typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
         typedef __attribute__((address_space(3))) u32x2 lds_u32x2;
 #pragma unroll
@@ -625,18 +639,39 @@ static size_t cls_bytes(int64_t B, int64_t L) {
     return (size_t)(B * nt * nt + 255) / 256 * 256;
 }
 
-template <class T, int D, int MODE>
+template <class T, int D, int MODE, int NW>
 static int launch_prefill(const PrefillParams& p, int grid, hipStream_t stream) {
-    hipLaunchKernelGGL((prefill_kernel<T, D, MODE>), dim3(grid), dim3(kThreads), 0, stream, p);
+    hipLaunchKernelGGL((prefill_kernel<T, D, MODE, NW>), dim3(grid), dim3(NW * 64), 0, stream, p);
     return check_launch("prefill_kernel");
 }
 
-template <int MODE>
-static int dispatch_prefill(int dtype, int64_t D, const PrefillParams& p, int grid, hipStream_t stream) {
+template <int MODE, int NW>
+static int dispatch_prefill_nw(int dtype, int64_t D, const PrefillParams& p, int grid, hipStream_t stream) {
     if (dtype == MINFER_ATTN_F16) {
-        return D == 128 ? launch_prefill<F16, 128, MODE>(p, grid, stream) : launch_prefill<F16, 64, MODE>(p, grid, stream);
+        return D == 128 ? launch_prefill<F16, 128, MODE, NW>(p, grid, stream) : launch_prefill<F16, 64, MODE, NW>(p, grid, stream);
     }
-    return D == 128 ? launch_prefill<BF16, 128, MODE>(p, grid, stream) : launch_prefill<BF16, 64, MODE>(p, grid, stream);
+    return D == 128 ? launch_prefill<BF16, 128, MODE, NW>(p, grid, stream) : launch_prefill<BF16, 64, MODE, NW>(p, grid, stream);
+}
+
+template <int MODE>
+static int dispatch_prefill(int dtype, int64_t D, const PrefillParams& p, int waves, int grid, hipStream_t stream) {
+    return waves == kWavesSmall ? dispatch_prefill_nw<MODE, kWavesSmall>(dtype, D, p, grid, stream)
+                                : dispatch_prefill_nw<MODE, kWavesBig>(dtype, D, p, grid, stream);
+}
+
+// Waves per workgroup for a launch whose sequences have at most `longest` rows.  Short sequences mean few key tiles per
+// workgroup, so the cost a workgroup pays once (query rows in, first tile, output rows out, hand-over of the compute
+// unit) is a large share: two small workgroups per compute unit hide it under each other's tiles.  Long sequences
+// amortise it and gain more from sharing every staged K/V tile among 256 rows.
+#ifndef MINFER_PREFILL_FORCE_WAVES
+#define MINFER_PREFILL_FORCE_WAVES 0
+#endif
+// Measured, 4 against 8 waves, 32 query heads over 8 KV heads: 128 packed sequences of 128 rows 87 / 98 us, 64 of 512
+// rows 256 / 263 us, dense B=16 L=512 68 / 73 us, B=8 L=1024 95.5 / 97.8 us, B=4 L=2048 159 / 156 us, L=4096 157 / 146 us.
+constexpr int64_t kSmallWorkgroupMaxRows = 1024;
+static int prefill_waves(int64_t longest) {
+    if (MINFER_PREFILL_FORCE_WAVES) return MINFER_PREFILL_FORCE_WAVES;
+    return longest <= kSmallWorkgroupMaxRows ? kWavesSmall : kWavesBig;
 }
 
 // The global->LDS tile copies address a tile's rows with a 32-bit unsigned per-lane byte offset from the tile's first
@@ -650,7 +685,7 @@ static int check_row_stride(const minfer_attn_strides* st, const char* op) {
 }
 
 static void fill_common(PrefillParams& p, const void* q, const void* k, const void* v, void* out,
-                        int64_t Hq, int64_t Hkv, int64_t D, const minfer_attn_strides* st) {
+                        int64_t Hq, int64_t Hkv, int64_t D, const minfer_attn_strides* st, int kWaves) {
     p.q = q; p.k = k; p.v = v; p.out = out;
     p.q0 = st->q0; p.q1 = st->q1; p.q2 = st->q2;
     p.kv0 = st->kv0; p.kv1 = st->kv1; p.kv2 = st->kv2;
@@ -687,7 +722,8 @@ MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k
     hipStream_t stream = (hipStream_t)stream_v;
 
     PrefillParams p{};
-    fill_common(p, q, k, v, out, Hq, Hkv, D, st);
+    const int kWaves = prefill_waves(L);
+    fill_common(p, q, k, v, out, Hq, Hkv, D, st, kWaves);
     p.mask = mask; p.cls = (const uint8_t*)workspace; p.cu = nullptr;
     p.L = (int)L; p.B = (int)B;
     p.NQT = p.NKT = (int)((L + 63) / 64);
@@ -705,7 +741,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k
         hipLaunchKernelGGL(classify_mask_kernel, dim3((p.NKT + 15) / 16, p.NQT, (unsigned)B), dim3(256), 0, stream,
                            mask, (uint8_t*)workspace, p.L, p.NQT, p.NKT, p.mask_vec);
     if (int rc = check_launch("classify_mask_kernel")) return rc;
-    return dispatch_prefill<MODE_DENSE>(dtype, D, p, (int)grid, stream);
+    return dispatch_prefill<MODE_DENSE>(dtype, D, p, kWaves, (int)grid, stream);
 }
 
 MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const void* k, const void* v,
@@ -721,15 +757,16 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const 
     if (T > 0x7fffffffLL / 2) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: T too large");
     hipStream_t stream = (hipStream_t)stream_v;
 
+    // max_seqlen 0 means "not known".  Rows of a sequence past max_seqlen are not computed, so a caller's bound
+    // must be at least the longest sequence (as in every varlen attention interface).
+    const int64_t max_len = (max_seqlen > 0 && max_seqlen < T) ? max_seqlen : T;
     PrefillParams p{};
-    fill_common(p, q, k, v, out, Hq, Hkv, D, st);
+    const int kWaves = prefill_waves(max_len);
+    fill_common(p, q, k, v, out, Hq, Hkv, D, st, kWaves);
     p.mask = nullptr; p.cls = nullptr; p.cu = cu_seqlens;
     p.L = (int)T; p.B = 1;
     p.NQT = p.NKT = 0;
     const int rows_per_wg = 32 * (kWaves >> p.hpw_log2);
-    // max_seqlen 0 means "not known".  Rows of a sequence past max_seqlen are not computed, so a caller's bound
-    // must be at least the longest sequence (as in every varlen attention interface).
-    const int64_t max_len = (max_seqlen > 0 && max_seqlen < T) ? max_seqlen : T;
     // query tiles: sum over sequences of ceil(len / rows_per_wg) <= both bounds below (cu_seqlens lives on the device,
     // so the exact count is not known here; workgroups past it exit at once)
     const int64_t nq_packed = (T + rows_per_wg - 1) / rows_per_wg + n_seqs;
@@ -739,7 +776,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const 
     p.max_len = (int)max_len;
     const int64_t grid = (int64_t)p.NQ * Hkv * p.n_hg;
     if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn_varlen: problem too large for one launch");
-    return dispatch_prefill<MODE_VARLEN>(dtype, D, p, (int)grid, stream);
+    return dispatch_prefill<MODE_VARLEN>(dtype, D, p, kWaves, (int)grid, stream);
 }
 
 // ------------------------------------------------------------------------------------------------

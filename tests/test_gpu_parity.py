@@ -112,6 +112,10 @@ def test_golden_decode_and_varlen():
     (1, 4, 2, 63, 64, "causal", False),
     (3, 4, 1, 65, 128, "full", False),
     (1, 4, 1, 1040, 128, "blocky", False),
+    # above 1024 rows the launch uses 8-wave workgroups (4-wave ones below): the same kinds of edges there
+    (1, 6, 2, 1093, 128, "random", False),   # n_rep = 3, byte-wise mask path
+    (1, 8, 1, 1100, 64, "window", True),     # n_rep = 8, D = 64, transposed views
+    (2, 4, 4, 1029, 128, "causal", False),   # n_rep = 1, a last tile of 5 rows
 ])
 def test_dense_matches_oracle(dtype, B, Hq, Hkv, L, D, kind, views):
     gen = torch.Generator().manual_seed(1000 * L + D + Hq)
@@ -330,6 +334,7 @@ def test_decode_equals_last_prefill_row():
     (6, 2, 128, [1, 1, 1]),
     (4, 4, 64, [300]),
     (8, 2, 128, [(7 * i) % 41 for i in range(150)]),      # more sequences than a wave has lanes, some empty
+    (8, 2, 64, [700, 333, 0, 20, 64, 1]),
 ])
 def test_varlen_matches_oracle_and_dense(dtype, Hq, Hkv, D, lens):
     g = torch.Generator().manual_seed(sum(lens))
@@ -342,6 +347,13 @@ def test_varlen_matches_oracle_and_dense(dtype, Hq, Hkv, D, lens):
     assert capi.flash_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), max(lens), out) == capi.OK, capi.last_error()
     torch.cuda.synchronize()
     assert max_err(out, oracle.flash_attn_varlen(q, k, v, cu)) <= TOL[dtype]
+    # max_seqlen chooses the workgroup shape (4 waves up to 1024 rows, 8 above; 0 = not known = T): the same bits either way
+    out0 = torch.full(q.shape, float("nan"), dtype=dtype, device=DEV)
+    assert capi.flash_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), 0, out0) == capi.OK, capi.last_error()
+    out_big = torch.full(q.shape, float("nan"), dtype=dtype, device=DEV)
+    assert capi.flash_attn_varlen(q.to(DEV), k.to(DEV), v.to(DEV), cu.to(DEV), 5000, out_big) == capi.OK, capi.last_error()
+    torch.cuda.synchronize()
+    assert torch.equal(out0, out) and torch.equal(out_big, out)
     # same result as the reference-signature op under the block-diagonal causal mask
     blk = torch.zeros(T, T, dtype=torch.bool)
     for lo, hi in zip(cu[:-1].tolist(), cu[1:].tolist()):
