@@ -334,6 +334,18 @@ int minfer_rope_kv_append_q8_0(int dtype, int style, void* q, const void* k, con
 #define MINFER_CALIB_MFMA_FLOP_PER_ITER (8 * 8 * 32768)   /* per workgroup */
 int minfer_calib_mfma_rate(int dtype, const void* operands, int64_t iters, int64_t workgroups, float* sink, void* stream);
 
+/*
+ * Calibration as well: the prefill kernel's per-tile instruction mix at head_dim 128 (32 MFMAs, 16 + 32 LDS fragment
+ * reads, the softmax's maximum / exponential / pack / denominator instructions) on one K and one V tile that stay in
+ * LDS, with no global memory traffic, barrier, mask or bookkeeping in the loop; `iters` tiles per wave, 32 * 32768
+ * flop each, workgroups * 8 waves.  lds_reads = 0 keeps the fragments in registers, softmax = 0 feeds the second GEMM
+ * from registers.  With both set this is the rate an attention kernel free of every fixed cost would reach on the
+ * caller's operand values.  operands and sink as for minfer_calib_mfma_rate.  No counterpart in the reference.
+ */
+#define MINFER_CALIB_ATTN_MIX_FLOP_PER_ITER (8 * 32 * 32768)   /* per workgroup */
+int minfer_calib_attn_mix(int dtype, const void* operands, int64_t iters, int64_t workgroups, int lds_reads, int softmax,
+                          float* sink, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

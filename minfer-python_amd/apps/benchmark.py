@@ -216,6 +216,14 @@ def mfma_rate(backend: str, which: str):
             for kind in ("random", "constant", "zero"):
                 r = calibration.mfma_rate(dtype, kind)
                 print(f"{r['dtype']:<10}{kind:<12}{r['tflops']:>10.1f}{r['tflops'] / 2500.0:>10.3f}")
+        # the prefill kernel's per-tile instruction mix without any memory traffic, barrier or bookkeeping: what each kind
+        # of co-running work costs the matrix rate, and what a kernel with no fixed cost at all would reach
+        print(f"{'dtype':<10}{'operands':<12}{'fragments':<12}{'softmax':<10}{'TFLOP/s':>10}{'of 2500':>10}   (32 MFMAs per wave and 64-key tile, head_dim 128)")
+        for dtype in (torch.float16, torch.bfloat16):
+            for kind in ("random", "zero"):
+                for lds_reads, softmax in ((False, False), (True, False), (False, True), (True, True)):
+                    r = calibration.attn_mix_rate(dtype, kind, lds_reads, softmax)
+                    print(f"{r['dtype']:<10}{kind:<12}{'from LDS' if lds_reads else 'registers':<12}{'yes' if softmax else 'no':<10}{r['tflops']:>10.1f}{r['tflops'] / 2500.0:>10.3f}")
     else:
         results = []
         for dtype in (torch.float16, torch.bfloat16):

@@ -52,7 +52,7 @@ struct F16 {
         const h16x8 v = __builtin_bit_cast(h16x8, x);
         h16x8 r;
 #pragma unroll
-        for (int i = 0; i < 8; ++i) r[i] = (_Float16)((float)v[i] * f);
+        for (int i = 0; i < 8; ++i) r[i] = (_Float16)__builtin_fmaf((float)v[i], f, 0.f);   // one mixed-precision fma each
         return __builtin_bit_cast(s16x8, r);
     }
     // acc + lo + hi of a packed pair, in fp32: sums exactly the rounded values the MFMA consumes

@@ -280,12 +280,25 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     // The wave's Q rows are requested now and used after the tile list is built, so that the two latencies overlap.
     // They are copied global->LDS as whole rows (RPI rows per instruction, with the K tile's swizzle) and read back as
     // fragments: fetched straight into fragment registers every instruction would touch 32 rows for 32 bytes each.
-    // Rows past the end of the sequence re-read its last row.
+    // A block that lies wholly inside its sequence (all but a sequence's last one) takes the short way: a wave-uniform
+    // base per instruction plus one 32-bit lane offset (swz_k of the instruction's first row and of the lane's row
+    // within it occupy different bits, so the instruction's share of the swizzle is a constant).  Otherwise rows past
+    // the end of the sequence re-read its last row.
+    if (q_row0 + 32 <= seq_len) {
+        const int row_in = lane / G, pg = lane % G;
+        const uint32_t lane_row = (uint32_t)((int64_t)row_in * p.q2) * 2u;
+        const int g0 = pg ^ GEO::swz_k(row_in);
+        const short* qbase = Qh + (int64_t)q_row0 * p.q2;
 #pragma unroll
-    for (int j = 0; j < 32 / RPI; ++j) {
-        const int row = j * RPI + lane / G, pg = lane % G;
-        const short* src = Qh + (int64_t)min(q_row0 + row, last_row) * p.q2 + 8 * (pg ^ GEO::swz_k(row));
-        copy16_global_to_lds(src, q_stage + j * RPI * RB);
+        for (int j = 0; j < 32 / RPI; ++j)
+            copy16_global_to_lds(qbase + (int64_t)(j * RPI) * p.q2, lane_row + 16u * (uint32_t)(g0 ^ GEO::swz_k(j * RPI)), q_stage + j * RPI * RB);
+    } else {
+#pragma unroll
+        for (int j = 0; j < 32 / RPI; ++j) {
+            const int row = j * RPI + lane / G, pg = lane % G;
+            const short* src = Qh + (int64_t)min(q_row0 + row, last_row) * p.q2 + 8 * (pg ^ GEO::swz_k(row));
+            copy16_global_to_lds(src, q_stage + j * RPI * RB);
+        }
     }
 
     // ---- list of key tiles this workgroup visits ---------------------------------------------
@@ -622,11 +635,23 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
                 *(lds_u32x2*)(uintptr_t)(so + l32 * RB + 16 * (gi ^ (l32 & (G - 1))) + 8 * h) = pk;
             }
         }
+        if (q_row0 + 32 <= seq_len) {   // every row exists: a wave-uniform base per store plus one 32-bit lane offset
+            const int row_in = lane / G, gi = lane % G;
+            const uint32_t lane_off = (uint32_t)((int64_t)row_in * p.o2 + 8 * gi) * 2u;
+            char* obase = reinterpret_cast<char*>(Oh + (int64_t)q_row0 * p.o2);
 #pragma unroll
-        for (int i = 0; i < 32 / RPI; ++i) {
-            const int r = i * RPI + lane / G, gi = lane % G;
-            const s16x8 val = lds_read_b128(so + r * RB + 16 * (gi ^ (r & (G - 1))), 0);
-            if (q_row0 + r < seq_len) *reinterpret_cast<s16x8*>(Oh + (int64_t)(q_row0 + r) * p.o2 + 8 * gi) = val;
+            for (int i = 0; i < 32 / RPI; ++i) {
+                const int r = i * RPI + row_in;
+                const s16x8 val = lds_read_b128(so + r * RB + 16 * (gi ^ (r & (G - 1))), 0);
+                *reinterpret_cast<s16x8*>(obase + (int64_t)(i * RPI) * p.o2 * 2 + lane_off) = val;
+            }
+        } else {
+#pragma unroll
+            for (int i = 0; i < 32 / RPI; ++i) {
+                const int r = i * RPI + lane / G, gi = lane % G;
+                const s16x8 val = lds_read_b128(so + r * RB + 16 * (gi ^ (r & (G - 1))), 0);
+                if (q_row0 + r < seq_len) *reinterpret_cast<s16x8*>(Oh + (int64_t)(q_row0 + r) * p.o2 + 8 * gi) = val;
+            }
         }
     }
 }
@@ -674,11 +699,12 @@ static int prefill_waves(int64_t longest) {
     return longest <= kSmallWorkgroupMaxRows ? kWavesSmall : kWavesBig;
 }
 
-// The global->LDS tile copies address a tile's rows with a 32-bit unsigned per-lane byte offset from the tile's first
-// row (rows 0..63 of it, plus a granule inside the row): the K/V row stride must keep that below 2^32.
+// The global->LDS copies of K/V tiles and query rows and the output stores address a block's rows with a 32-bit unsigned
+// per-lane byte offset from the block's first row (a few rows of it, plus a granule inside the row): the row strides
+// must keep that below 2^32.
 static int check_row_stride(const minfer_attn_strides* st, const char* op) {
-    if (st->kv2 >= (INT64_C(1) << 25)) {
-        snprintf(error_buf(), 512, "%s: k/v row stride (dim 2) must be below 2^25 elements", op);
+    if (st->kv2 >= (INT64_C(1) << 25) || st->q2 >= (INT64_C(1) << 25) || st->o2 >= (INT64_C(1) << 25)) {
+        snprintf(error_buf(), 512, "%s: row strides (dim 2) of q, k/v and out must be below 2^25 elements", op);
         return MINFER_ATTN_EINVAL;
     }
     return MINFER_ATTN_OK;
