@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
 # These are figures from those earlier counter runs, not measured in the run that prints them.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels_pmc.md (rocprofv3 --pmc runs of the same workloads; not re-measured by this run)"
-PREFILL_TRAFFIC_BYTES = 107531 * 1024
+PREFILL_TRAFFIC_BYTES = 107400 * 1024
 DECODE_TRAFFIC_BYTES = 1092838 * 1024
 ROPE_TRAFFIC_BYTES = 393312 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
@@ -39,9 +39,9 @@ DECODE_Q8_TRAFFIC_BYTES = 598453 * 1024     # decode over Q8_0 caches (split + c
 APPEND_Q8_TRAFFIC_BYTES = 737585 * 1024     # rope_kv_append into Q8_0 caches
 APPEND_NORM_TRAFFIC_BYTES = 786620 * 1024   # rope_kv_append_norm, the same shape
 QKV_TRAFFIC_BYTES = 377657 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
-LONG_TRAFFIC_BYTES = None                   # long-context prefill (classify + main), S=32768 bf16
-RAGGED_TRAFFIC_BYTES = None                 # packed ragged prefill
-GEMM_Q8_TRAFFIC_BYTES = None                # one token against a 14336 x 4096 weight of Q8_0 blocks
+LONG_TRAFFIC_BYTES = 2721654 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
+RAGGED_TRAFFIC_BYTES = 748670 * 1024        # packed ragged prefill (T=20514, Hq=64)
+GEMM_Q8_TRAFFIC_BYTES = 67126 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
 
 
 class HipEvents:

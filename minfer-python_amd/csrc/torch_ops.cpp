@@ -515,6 +515,16 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
         // weights as rows of Q8_0 blocks, uint8 [out_dim, hidden_dim / 32 * 34] (each may also be 16-bit): one projection per weight
         STD_TORCH_CHECK(t == ScalarType::Half, "qkv: x must be float16 with a Q8_0 weight");
         STD_TORCH_CHECK(K % 32 == 0, "qkv: hidden_dim must be a multiple of the block size");
+        // one workspace, sized for the projection that needs most, serves the three calls one after the other (they run
+        // in stream order): the dequantised weight of a Q8_0 projection with many rows, the K slices of a 16-bit one
+        size_t ws_max = 0;
+        for (int i = 0; i < 3; ++i) {
+            const int64_t N = outs[i]->dim() == 3 ? outs[i]->size(-1) : 0;
+            const size_t need = qtypes[i] == MINFER_Q8_0 ? minfer_gemm_q8_0_workspace_bytes(M, N, K) : minfer_gemm_workspace_bytes(M, N, K);
+            ws_max = need > ws_max ? need : ws_max;
+        }
+        Tensor wsp = byte_workspace(x, ws_max);
+        void* wsp_ptr = ws_max ? wsp.mutable_data_ptr() : nullptr;
         for (int i = 0; i < 3; ++i) {
             const Tensor& w = *ws[i];
             Tensor& o = *outs[i];
@@ -526,16 +536,14 @@ void qkv_hip(int64_t q_qtype_int, int64_t k_qtype_int, int64_t v_qtype_int, int6
                 STD_TORCH_CHECK(qblocks[i] == MINFER_Q8_0_BLOCK && qsizes[i] == MINFER_Q8_0_BLOCK_BYTES, names[i], ": Q8_0 is (qblock_size, qtype_size) = (32, 34)");
                 STD_TORCH_CHECK(w.scalar_type() == ScalarType::Byte && w.size(0) == N && w.size(1) == K / 32 * 34, names[i],
                                 ": a Q8_0 weight is uint8 [out_dim, hidden_dim / 32 * 34]");
-                const size_t ws_bytes = minfer_gemm_q8_0_workspace_bytes(M, N, K);
-                Tensor wsp = byte_workspace(x, ws_bytes);
                 check_rc(minfer_gemm_q8_0(x.const_data_ptr(), w.const_data_ptr(), nullptr, o.mutable_data_ptr(), M, N, K, K, N, N, 1.0, 0.0,
-                                          ws_bytes ? wsp.mutable_data_ptr() : nullptr, ws_bytes, stream),
+                                          wsp_ptr, ws_max, stream),
                          names[i]);
             } else {
                 STD_TORCH_CHECK(qtypes[i] == 1 && w.scalar_type() == t && w.size(0) == N && w.size(1) == K, names[i],
                                 ": next to a Q8_0 weight, a 16-bit weight must be float16 [out_dim, hidden_dim]");
-                check_rc(minfer_gemm(dtype, MINFER_GEMM_B_NK, x.const_data_ptr(), w.const_data_ptr(), nullptr, o.mutable_data_ptr(), M, N, K, K, K, N, N,
-                                     1.0, 0.0, stream),
+                check_rc(minfer_gemm_ws(dtype, MINFER_GEMM_B_NK, x.const_data_ptr(), w.const_data_ptr(), nullptr, o.mutable_data_ptr(), M, N, K, K, K, N, N,
+                                        1.0, 0.0, wsp_ptr, ws_max, stream),
                          names[i]);
             }
         }
