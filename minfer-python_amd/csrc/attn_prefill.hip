@@ -496,22 +496,23 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- masking ----------------------------------------------------------------------
+        // Register 4j + e of block kb is key key0 + 32kb + 8j + 4h + e.  The test by position (keys past the end of the
+        // sequence; in a packed batch also keys after the lane's query row) is one compare of a constant with a per-lane
+        // limit; dense MIXED tiles test their mask bytes as well.
         if (cls_w == TILE_MIXED || key0 + 64 > seq_len) {
             const bool use_bytes = MODE == MODE_DENSE && cls_w == TILE_MIXED;
+            int lim = last_row - key0 - 4 * h;                              // largest kept 32kb + 8j + e
+            if (MODE == MODE_VARLEN) lim = min(lim, qrow - key0 - 4 * h);
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb) {
+            for (int kb = 0; kb < 2; ++kb)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int kbase = key0 + 32 * kb + 8 * j + 4 * h;
+                for (int j = 0; j < 4; ++j)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        bool keep = kbase + e < seq_len;
+                        bool keep = 32 * kb + 8 * j + e <= lim;
                         if (MODE == MODE_DENSE) keep = keep && (!use_bytes || ((mw[kb][j] >> (8 * e)) & 0xffu) != 0u);
-                        else keep = keep && (kbase + e <= qrow);
                         e_acc[kb][4 * j + e] = keep ? e_acc[kb][4 * j + e] : -INFINITY;
                     }
-                }
-            }
         }
         // ---- reference update (rare after the first tiles) --------------------------------------
         {
