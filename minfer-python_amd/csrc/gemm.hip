@@ -18,6 +18,7 @@
 // conflicts.  Workgroup ids are dealt so that one XCD works on consecutive tiles of a tile row (they share the
 // A panel in that XCD's L2).
 #include <algorithm>
+#include <atomic>
 
 #include "attn_common.h"
 #include "attn_host.h"
@@ -29,8 +30,8 @@ namespace minfer_attn {
 constexpr int kBK = 64;
 // Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
 // 128 x 128 otherwise.  A wave owns 32*MB rows x 32*NB columns; OCC waves per SIMD.
-template <int MB_, int NB_, int WAVES_N_, int OCC_> struct GemmShape {
-    static constexpr int MB = MB_, NB = NB_, WAVES_M = 2, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N, OCC = OCC_;
+template <int MB_, int NB_, int WAVES_N_, int OCC_, int WAVES_M_ = 2> struct GemmShape {
+    static constexpr int MB = MB_, NB = NB_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N, OCC = OCC_;
     static constexpr int BM = 32 * MB * WAVES_M, BN = 32 * NB * WAVES_N;
     static constexpr int A_PANEL = BM * 128, B_PANEL = BN * 128;   // bytes of one K step
     static constexpr int A_COPIES = A_PANEL / 1024 / WAVES, B_COPIES = B_PANEL / 1024 / WAVES;   // wave-wide copies per wave
@@ -43,6 +44,11 @@ template <int MB_, int NB_, int WAVES_N_, int OCC_> struct GemmShape {
 // 124.0 us) and 4 % behind at 8192^3: the LDS bytes are not what bounds this kernel.)
 using GemmBig = GemmShape<4, 2, 4, 2>;
 using GemmSmall = GemmShape<2, 2, 2, 2>;
+// 256 x 192 (8 waves as 4 x 2, a wave owns 64 x 96): for widths that are multiples of 192 whose 256 x 256 tiles would
+// leave half the chip idle in their last round (4096 x 6144 is 384 large tiles, one and a half rounds on 256 compute
+// units, but 512 of these, two full rounds of three quarters the work each).  [N, K] weights only: its 192 columns are
+// three 64-row sub-tiles of such a weight, but one and a half of the 128-column sub-tiles of a [K, N] one.
+using GemmWide = GemmShape<2, 3, 2, 2, 4>;
 constexpr int kRowTile = 8192;              // sub-tile [64 rows][64 k], 128-byte rows (A, and B as [N, K])
 constexpr int kColTile = 16384;             // sub-tile [64 k][128 n], 256-byte rows (B as [K, N])
 
@@ -75,15 +81,21 @@ MA_DEV int group_of_unit(const GemmGroup& g, int c, int& local) {
 MA_DEV int swz_row_tile(int row) { return (row >> 1) & 7; }        // 128-byte rows, read 32 rows x 16 bytes
 MA_DEV int swz_col_tile(int row) { return (row & 3) << 2; }        // 256-byte rows, read 4 rows x 64 bytes (transposing)
 
-template <class T, bool NT, class SH, bool GROUPED = false, bool SPLIT = false>
+// CONCAT (with GROUPED, [N, K] weights whose widths are multiples of 64): the weights' columns are numbered through as
+// one wide matrix and tiled without regard to where one weight ends, so a tile may hold columns of two weights; every
+// 64-column sub-tile of the B panel and every 32-column block of a wave lies inside one weight, which is looked up
+// per copy instruction and per block (grp.end = cumulative column counts).
+template <class T, bool NT, class SH, bool GROUPED = false, bool SPLIT = false, bool CONCAT = false>
 __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const GemmParams p) {
+    static_assert(!CONCAT || (GROUPED && NT && !SPLIT && SH::WAVES == 8), "CONCAT: grouped [N, K] weights, one sub-tile per copy index");
     constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB, NB = SH::NB, CA = SH::A_COPIES, CB = SH::B_COPIES;
     __shared__ __attribute__((aligned(1024))) char a_lds[2][SH::A_PANEL];
     __shared__ __attribute__((aligned(1024))) char b_lds[2][SH::B_PANEL];
 
     const int lane = threadIdx.x & 63, w = wave_id();
     const int h = lane >> 5, l32 = lane & 31;
-    const int wm = w & 1, wn = w >> 1;   // wave's place in the tile: rows 32*MB*wm .., columns 64*wn ..
+    const int wm = w % SH::WAVES_M, wn = w / SH::WAVES_M;   // wave's place in the tile: rows 32*MB*wm .., columns 32*NB*wn ..
+    static_assert(NT || SH::BN % 128 == 0, "a [K, N] weight is staged in sub-tiles of 128 columns");
 
     // ---- which tile ----------------------------------------------------------------------------------
     // (SPLIT: consecutive workgroup ids are the K slices of one tile, so the slices of a tile run on different XCDs)
@@ -104,7 +116,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     short* Dg = (short*)p.D;
     int N = p.N;
     int64_t ldb = p.ldb, ldd = p.ldd;
-    if (GROUPED) {   // the tile column's weight, output and place inside them (all wave-uniform)
+    if (GROUPED && !CONCAT) {   // the tile column's weight, output and place inside them (all wave-uniform)
         int local;
         const int sg = group_of_unit(p.grp, in_band / gm, local);
         n0 = local * kBN;
@@ -121,6 +133,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     //   B as [K, N]:         k rows 4*(q%16) .. +3 of sub-tile q/16 (64 k rows of 256 bytes, 128 columns).
     uint32_t a_off[CA], b_off[CB];
     int a_dst[CA], b_dst[CB];
+    const short* b_src[CONCAT ? CB : 1];   // CONCAT: first weight row of copy j's sub-tile (wave-uniform)
 #pragma unroll
     for (int j = 0; j < CA; ++j) {
         const int q = j * NW + w;
@@ -132,7 +145,15 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 #pragma unroll
     for (int j = 0; j < CB; ++j) {
         const int q = j * NW + w;
-        if (NT) {
+        if (CONCAT) {   // copy j of every wave lies in sub-tile j, whose 64 weight rows belong to one weight
+            const int row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
+            int local;
+            const int sg = group_of_unit(p.grp, n0 + 64 * j, local);
+            const int64_t ldj = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
+            b_src[j] = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]) + (int64_t)local * ldj;
+            b_off[j] = (uint32_t)((int64_t)row * ldj + 8 * (pg ^ swz_row_tile(row))) * 2u;
+            b_dst[j] = j * kRowTile + 8 * (q & 7) * 128;
+        } else if (NT) {
             const int sub = q >> 3, row = 8 * (q & 7) + (lane >> 3), pg = lane & 7;
             const int n = min(n0 + 64 * sub + row, N - 1) - n0;
             b_off[j] = (uint32_t)((int64_t)n * ldb + 8 * (pg ^ swz_row_tile(row))) * 2u;
@@ -155,7 +176,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 #pragma unroll
         for (int j = 0; j < CA; ++j) copy16_global_to_lds(abase, a_off[j], &a_lds[stage][a_dst[j]]);
 #pragma unroll
-        for (int j = 0; j < CB; ++j) copy16_global_to_lds(bbase, b_off[j], &b_lds[stage][b_dst[j]]);
+        for (int j = 0; j < CB; ++j) copy16_global_to_lds(CONCAT ? b_src[CONCAT ? j : 0] + (int64_t)kt * kBK : bbase, b_off[j], &b_lds[stage][b_dst[j]]);
     };
 
     // ---- per-lane LDS read addresses (stage 0; stage, sub-tile and block offsets are immediates) ---------
@@ -167,8 +188,9 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 #pragma unroll
         for (int kk = 0; kk < 4; ++kk) {
             const uint32_t o = l32 * 128 + 16 * ((2 * kk + h) ^ sw);
-            m_rd[kk] = lds_addr(&a_lds[0][0]) + (MB / 2) * wm * kRowTile + o;
-            if (NT) n_rd[kk] = lds_addr(&b_lds[0][0]) + (NB / 2) * wn * kRowTile + o;    // n fragments: as the m fragments
+            // (a 32-row block is half a 64-row sub-tile: block g of a panel starts g * kRowTile / 2 bytes into it)
+            m_rd[kk] = lds_addr(&a_lds[0][0]) + MB * wm * (kRowTile / 2) + o;
+            if (NT) n_rd[kk] = lds_addr(&b_lds[0][0]) + NB * wn * (kRowTile / 2) + o;    // n fragments: as the m fragments
         }
         if (!NT) {
             // n fragments through transpose reads of the [k][n] sub-tile wn>>1: per 16-lane group 4 k rows x 16 columns
@@ -196,7 +218,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
             if (NT) {
-                nf[nb] = lds_read_b128(n_rd[kk], BOFF + (nb >> 1) * kRowTile + 32 * (nb & 1) * 128);
+                nf[nb] = lds_read_b128(n_rd[kk], BOFF + nb * (kRowTile / 2));
             } else {
                 const s16x4 t0 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk) * 256);
                 const s16x4 t1 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk + 4) * 256);
@@ -204,7 +226,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
             }
         }
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) mf[mb] = lds_read_b128(m_rd[kk], AOFF + (mb >> 1) * kRowTile + 32 * (mb & 1) * 128);
+        for (int mb = 0; mb < MB; ++mb) mf[mb] = lds_read_b128(m_rd[kk], AOFF + mb * (kRowTile / 2));
     };
     // ---- main loop ---------------------------------------------------------------------------------------
     // Fragments are double-buffered in registers: while the 8 (4) MFMAs of one 16-wide k slice run, the fragments
@@ -253,10 +275,18 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
         if (m >= p.M) continue;
 #pragma unroll
         for (int nb = 0; nb < NB; ++nb) {
+            int nb0 = n0 + 32 * NB * wn + 32 * nb;   // first column of the block
+            if (CONCAT) {                             // ... inside the weight that holds the block
+                int local;
+                const int sg = group_of_unit(p.grp, nb0, local);
+                nb0 = local;
+                Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
+                ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
+            }
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const int n = n0 + 32 * NB * wn + 32 * nb + 8 * j + 4 * h;
-                if (n >= N) continue;
+                const int n = nb0 + 8 * j + 4 * h;
+                if (!CONCAT && n >= N) continue;
                 if (SPLIT) {   // the slice's raw sums; gemm_reduce_kernel adds the slices up and applies alpha, beta and C
                     const f32x4 raw = {acc[nb][mb][4 * j], acc[nb][mb][4 * j + 1], acc[nb][mb][4 * j + 2], acc[nb][mb][4 * j + 3]};
                     *reinterpret_cast<f32x4*>(p.part + ((int64_t)slice * p.M + m) * N + n) = raw;
@@ -569,11 +599,36 @@ static int launch_tiled(GemmParams& p, hipStream_t stream) {
     return check_launch("gemm_kernel");
 }
 
+// Rounds of the chip a launch of `tiles` workgroups (one per compute unit at a time) costs: full rounds count 1; a last
+// round that fills only part of the chip counts 0.55 + 0.45 x that part (its compute units run faster, the chip being
+// less loaded: 4096 x 6144 x 4096 as 384 large tiles takes 1.76 rounds' time, 2048 x 6144 x 4096 as 192 takes 0.87).
+static double rounds_cost(int64_t tiles) {
+    static std::atomic<int> cached[64];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) dev = 0;
+    int cus = cached[dev].load(std::memory_order_relaxed);
+    if (cus == 0) {
+        if (hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus <= 0) cus = 256;
+        cached[dev].store(cus, std::memory_order_relaxed);
+    }
+    const int64_t full = tiles / cus, rest = tiles % cus;
+    return (double)full + (rest ? 0.55 + 0.45 * (double)rest / cus : 0.0);
+}
+// A 256 x 192 tile is 0.75 of a 256 x 256 one and runs 5 % below its rate per flop (8192 x 6144 x 4096: 366 against 347 us).
+static bool wide_shape_pays(int64_t big_tiles, int64_t wide_tiles) {
+    return 0.75 * 1.05 * rounds_cost(wide_tiles) < 0.97 * rounds_cost(big_tiles);
+}
+
 template <class T, bool NT>
 static int launch_gemm(GemmParams& p, bool fast, hipStream_t stream) {
     if (fast) {
         // large tiles halve the LDS and L2 traffic per flop; they are worth it once they fill most of the chip
         const int64_t big_tiles = (int64_t)((p.M + GemmBig::BM - 1) / GemmBig::BM) * ((p.N + GemmBig::BN - 1) / GemmBig::BN);
+        if constexpr (NT) {
+            if (big_tiles >= 160 && p.N % GemmWide::BN == 0 &&
+                wide_shape_pays(big_tiles, (int64_t)((p.M + GemmWide::BM - 1) / GemmWide::BM) * (p.N / GemmWide::BN)))
+                return launch_tiled<T, NT, GemmWide>(p, stream);
+        }
         return big_tiles >= 160 ? launch_tiled<T, NT, GemmBig>(p, stream) : launch_tiled<T, NT, GemmSmall>(p, stream);
     }
     const int grid = (int)std::min<int64_t>(((int64_t)p.M * p.N + 255) / 256, 256 * 16);
@@ -606,8 +661,27 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
 #undef MINFER_SKINNY
         return check_launch("gemm_skinny_kernel (grouped)");
     }
-    const int64_t big_tiles = (int64_t)((p.M + GemmBig::BM - 1) / GemmBig::BM) * ((n_sum + GemmBig::BN - 1) / GemmBig::BN);
+    int64_t big_tiles = 0;
+    for (int s = 0; s < n_w; ++s) big_tiles += (int64_t)((p.M + GemmBig::BM - 1) / GemmBig::BM) * ((p.grp.N[s] + GemmBig::BN - 1) / GemmBig::BN);
     const bool big = big_tiles >= 160;
+    // 256 x 192 tiles over the weights' columns numbered through, when that fills the chip's rounds better (the Llama-3-8B
+    // QKV projection of 4096 tokens: 384 large tiles, one and a half rounds, or 512 of these, two rounds of 3/4 the work)
+    bool concat = big && n_sum % GemmWide::BN == 0 && n_sum < (INT64_C(1) << 31);
+    for (int s = 0; s < n_w; ++s) concat = concat && p.grp.N[s] % 64 == 0;
+    if (concat) {
+        const int64_t wide_tiles = (int64_t)((p.M + GemmWide::BM - 1) / GemmWide::BM) * (n_sum / GemmWide::BN);
+        concat = wide_shape_pays(big_tiles, wide_tiles);
+    }
+    if (concat) {
+        int acc = 0;
+        for (int s = 0; s < kMaxGroup; ++s) { if (s < n_w) acc += p.grp.N[s]; p.grp.end[s] = acc; }
+        p.N = (int)n_sum;
+        p.tiles_m = (p.M + GemmWide::BM - 1) / GemmWide::BM;
+        p.tiles_n = (int)(n_sum / GemmWide::BN);
+        p.per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
+        hipLaunchKernelGGL((gemm_kernel<T, true, GemmWide, true, false, true>), dim3(p.per_xcd * 8), dim3(GemmWide::WAVES * 64), 0, stream, p);
+        return check_launch("gemm_kernel (grouped, columns numbered through)");
+    }
     const int bm = big ? GemmBig::BM : GemmSmall::BM, bn = big ? GemmBig::BN : GemmSmall::BN;
     p.tiles_m = (p.M + bm - 1) / bm;
     p.tiles_n = fill_ends(bn);

@@ -56,6 +56,8 @@ def make(M, N, K, layout, dtype, seed):
     (8, 4096, 4096, 1.0, 0.0),       # a decode step's tokens: with an [N, K] weight, the kernel that streams it once
     (64, 1024, 1792, 2.0, 3.0),      # its largest row count; K steps not a multiple of the eight waves
     (48, 8192, 8192, 1.0, 0.0),      # more than 32 rows against a large weight: the tiled kernel again
+    (2048, 6144, 128, 1.0, 1.0),     # [N, K]: 256 x 192 tiles (one full round instead of three quarters of one)
+    (1800, 6144, 64, 2.0, 3.0),      # the same with a ragged last tile row
     (30, 5200, 128, 2.0, 1.0),       # wide enough for two column groups per workgroup, the last one ragged
     (37, 24, 192, 0.5, 1.0),         # ragged rows, a last group of 16 columns that is half empty
     (17, 4104, 64, 1.0, 1.0),        # one K step: seven of the eight waves have nothing to add
@@ -124,7 +126,9 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
 
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("M,K,Nq,Nk,Nv", [
-    (4096, 4096, 4096, 1024, 1024),    # Llama-3-8B prefill: 256 x 256 tiles, 24 tile columns over three weights
+    (4096, 4096, 4096, 1024, 1024),    # Llama-3-8B prefill: 256 x 192 tiles over the weights' columns numbered through (two full rounds)
+    (2000, 128, 4096, 1024, 1024),     # the same tiling with a ragged last tile row; tiles that hold columns of q and k, of k and v
+    (4096, 128, 4096, 2048, 2048),     # 8192 columns: no multiple of 192, 256 x 256 tiles per weight
     (512, 6144, 6144, 1024, 1024),     # the reference test's head shape at a smaller batch: 128 x 128 tiles
     (300, 256, 200, 72, 136),          # ragged rows, widths that end inside a tile
     (1, 4096, 4096, 1024, 1024),       # a decode step: the few-row kernel over the three weights' column groups
