@@ -34,11 +34,11 @@ DECODE_TRAFFIC_BYTES = 1092838 * 1024
 ROPE_TRAFFIC_BYTES = 393312 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
 NORM_TRAFFIC_BYTES = 786659 * 1024          # rmsnorm on [8,4096,6144]
-GEMM_TRAFFIC_BYTES = 230579 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
+GEMM_TRAFFIC_BYTES = 230260 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
 DECODE_Q8_TRAFFIC_BYTES = 598453 * 1024     # decode over Q8_0 caches (split + combine)
 APPEND_Q8_TRAFFIC_BYTES = 737585 * 1024     # rope_kv_append into Q8_0 caches
 APPEND_NORM_TRAFFIC_BYTES = 786620 * 1024   # rope_kv_append_norm, the same shape
-QKV_TRAFFIC_BYTES = 377657 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
+QKV_TRAFFIC_BYTES = 378663 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
 LONG_TRAFFIC_BYTES = 2721654 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
 RAGGED_TRAFFIC_BYTES = 748670 * 1024        # packed ragged prefill (T=20514, Hq=64)
 GEMM_Q8_TRAFFIC_BYTES = 67126 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
@@ -508,7 +508,7 @@ def main():
     rec["qkv"] = {"value": p_tf, "unit": "TFLOP/s", "ms": p_avg_ms, "median_ms": p_med_ms,
                   "workload": "q,k,v = x wq^T, x wk^T, x wv^T in one launch: x [1,4096,4096], wq [4096,4096], wk and wv [1024,4096] fp16 (Llama-3-8B prefill)",
                   "roofline": mfma_roofline(p_tf, sus_f16, traffic=QKV_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
-                                            kernel="gemm_kernel<F16,[N,K],256x256,grouped>", algorithmic_flops=pflops)}
+                                            kernel="gemm_kernel<F16,[N,K],256x192,grouped,columns numbered through>", algorithmic_flops=pflops)}
     rec["gemm_q8_0"] = {"value": q8_gbs, "unit": "GB/s", "ms": q8_avg_ms, "median_ms": q8_med_ms,
                         "workload": "one token against a weight of Q8_0 blocks: x [1,1,4096] fp16, W uint8 [14336, 4352] (Llama-3-8B FFN up), out fp16",
                         "roofline": {"bound": "hbm", "achieved": q8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": q8_gbs / PEAK_HBM_GBS,
