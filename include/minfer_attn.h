@@ -101,7 +101,9 @@ int minfer_flash_attn_decode(int dtype, const void* q, const void* k_cache, cons
  * rejected with MINFER_ATTN_EINVAL.  Arguments, results and errors are otherwise those of
  * minfer_flash_attn_decode (16-bit caches only).
  */
+#ifndef MINFER_DECODE_NOALLOC_SCRATCH_BYTES   /* a build that never calls the entry point may shrink the array (define it when compiling the library) */
 #define MINFER_DECODE_NOALLOC_SCRATCH_BYTES (64u << 20)
+#endif
 int minfer_flash_attn_decode_noalloc(int dtype, const void* q, const void* k_cache, const void* v_cache,
                                      const int32_t* ctx_lens, void* out,
                                      int64_t B, int64_t Hq, int64_t Hkv, int64_t Lmax, int64_t D,
