@@ -161,7 +161,12 @@ struct PrefillParams {
     float scale_log2;      // softmax scale * log2(e)
 };
 
-enum { MODE_DENSE = 0, MODE_VARLEN = 1 };
+// MODE_DENSE: dense bool mask, tile classes from the pre-pass.  MODE_VARLEN: packed sequences, causal by index.
+// MODE_DENSE_SELF: dense bool mask of a short problem (L <= 1024, rows readable in 16-byte pieces): every workgroup
+// classifies its own rows of the mask in its prologue, one wave-wide load per row, and no pre-pass is launched.
+enum { MODE_DENSE = 0, MODE_VARLEN = 1, MODE_DENSE_SELF = 2 };
+constexpr int kSelfClassifyMaxGrid = 512;
+constexpr int kSelfClassifyMaxL = 1024;   // 16 key tiles: lane l of a wave-wide load holds columns 16l .. 16l+15 of one row
 // Waves per workgroup, a template argument of the kernel: 8 (one workgroup per compute unit: 256 query rows share every
 // K/V tile staged in LDS) or 4 (two workgroups per compute unit, 128 rows per tile: twice the tile copies per flop, but
 // one workgroup's prologue, epilogue and hand-over run under the other's tiles, which is what counts when sequences
@@ -193,7 +198,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     constexpr int ROWS_BYTES = 32 * RB;                // a wave's 32 query (or output) rows
 
     __shared__ __attribute__((aligned(1024))) char kv_lds[2][STAGE_BYTES];
-    __shared__ uint32_t tile_list[MODE == MODE_DENSE ? kMaxKeyTiles : 1];
+    constexpr bool kDense = MODE != MODE_VARLEN;
+    __shared__ uint32_t tile_list[MODE == MODE_DENSE ? kMaxKeyTiles : (MODE == MODE_DENSE_SELF ? kSelfClassifyMaxL / 64 : 1)];
     __shared__ int n_active_s;
     // A wave's own 32 query rows on their way in (whole rows, copied global->LDS) and its 32 output rows on their way
     // out (so that a store instruction writes whole rows).  With 8 waves the area is separate memory, the wave's own, so
@@ -229,7 +235,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
 
     int seq_lo = 0, seq_len = p.L;  // token rows of the attended sequence
     int qtile;                      // workgroup-level query tile (32*QBW rows) inside the sequence
-    if (MODE == MODE_DENSE) {
+    if (kDense) {
         qtile = p.NQ - 1 - rank;    // longest rows of a causal mask first
     } else {
         // the sequence that holds query tile `rank` of the packed batch: 64 sequences per step, a prefix sum of their
@@ -271,11 +277,11 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     const int last_row = seq_len - 1;
     const int qrow = q_row0 + l32;                               // this lane's query row
 
-    const short* Qh = (const short*)p.q + (MODE == MODE_DENSE ? (int64_t)b * p.q0 : 0) + (int64_t)head * p.q1 + (int64_t)seq_lo * p.q2;
-    const short* Kh = (const short*)p.k + (MODE == MODE_DENSE ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
-    const short* Vh = (const short*)p.v + (MODE == MODE_DENSE ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
-    short* Oh = (short*)p.out + (MODE == MODE_DENSE ? (int64_t)b * p.o0 : 0) + (int64_t)head * p.o1 + (int64_t)seq_lo * p.o2;
-    const uint8_t* mrow = MODE == MODE_DENSE ? p.mask + ((size_t)b * p.L + min(qrow, last_row)) * p.L : nullptr;
+    const short* Qh = (const short*)p.q + (kDense ? (int64_t)b * p.q0 : 0) + (int64_t)head * p.q1 + (int64_t)seq_lo * p.q2;
+    const short* Kh = (const short*)p.k + (kDense ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
+    const short* Vh = (const short*)p.v + (kDense ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
+    short* Oh = (short*)p.out + (kDense ? (int64_t)b * p.o0 : 0) + (int64_t)head * p.o1 + (int64_t)seq_lo * p.o2;
+    const uint8_t* mrow = kDense ? p.mask + ((size_t)b * p.L + min(qrow, last_row)) * p.L : nullptr;
 
     // The wave's Q rows are requested now and used after the tile list is built, so that the two latencies overlap.
     // They are copied global->LDS as whole rows (RPI rows per instruction, with the K tile's swizzle) and read back as
@@ -305,9 +311,51 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     // entry = key tile | (2-bit class for each 64-row query tile the workgroup overlaps) << 16
     const int qt64_first = (qtile * QBW * 32) >> 6;
     const int n_qt64 = QBW >= 2 ? QBW / 2 : 1;
-    const int my_qt64_slot = (q_row0 >> 6) - qt64_first;
+    // (a workgroup that classifies its own rows does so per 32-row query block: slot = the wave's block)
+    const int my_qt64_slot = MODE == MODE_DENSE_SELF ? (w >> p.hpw_log2) : (q_row0 >> 6) - qt64_first;
     int n_active;
-    if (MODE == MODE_DENSE) {
+    if (MODE == MODE_DENSE_SELF) {
+        // Every wave reads 32/HPW rows of its own query block (the HPW waves of a block share its rows), 8 rows in flight:
+        // lane l holds the 16 mask bytes of key columns 16l .. 16l+15, so lanes 4t .. 4t+3 cover key tile t.  Rows past the
+        // end re-read the last row, which changes neither the OR nor the AND.
+        __shared__ uint32_t any_s[NW][kSelfClassifyMaxL / 64], all_s[NW][kSelfClassifyMaxL / 64];
+        const int rpw = 32 >> p.hpw_log2;
+        const int row_first = q_row0 + (w & (HPW - 1)) * rpw;
+        uint32_t any_acc = 0u, all_acc = 0x01010101u;
+        if (16 * lane < p.L) {
+            const uint8_t* mb = p.mask + (size_t)b * p.L * p.L + 16 * lane;
+            for (int r0 = 0; r0 < rpw; r0 += 8) {
+                uint4 x[8];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = *reinterpret_cast<const uint4*>(mb + (size_t)min(row_first + r0 + i, last_row) * p.L);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    any_acc |= x[i].x | x[i].y | x[i].z | x[i].w;
+                    all_acc &= x[i].x & x[i].y & x[i].z & x[i].w;
+                }
+            }
+        }
+        any_acc |= __shfl_xor(any_acc, 1); any_acc |= __shfl_xor(any_acc, 2);
+        all_acc &= __shfl_xor(all_acc, 1); all_acc &= __shfl_xor(all_acc, 2);
+        if ((lane & 3) == 0) { any_s[w][lane >> 2] = any_acc; all_s[w][lane >> 2] = all_acc; }
+        __syncthreads();
+        if (w == 0) {
+            const int kt = lane;
+            uint32_t c = 0;
+            if (kt < p.NKT) {
+                for (int sb = 0; sb < QBW; ++sb) {
+                    uint32_t a = 0u, l = 0x01010101u;
+                    for (int ww = sb * HPW; ww < (sb + 1) * HPW; ++ww) { a |= any_s[ww][kt]; l &= all_s[ww][kt]; }
+                    c |= (a == 0u ? TILE_NONE : (l == 0x01010101u ? TILE_ALL : TILE_MIXED)) << (2 * sb);
+                }
+            }
+            const uint64_t bal = __ballot(c != 0);
+            if (c) tile_list[__popcll(bal & ((1ull << lane) - 1ull))] = (uint32_t)kt | (c << 16);
+            if (lane == 0) n_active_s = __popcll(bal);
+        }
+        __syncthreads();
+        n_active = n_active_s;
+    } else if (MODE == MODE_DENSE) {
         if (w == 0) {
             int cnt = 0;
             for (int base = 0; base < p.NKT; base += 64) {
@@ -405,7 +453,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     for (int r = 0; r < 16; ++r) neg_ref[r] = 0.f;
 
     auto tile_of = [&](uint32_t e, int it, int& kt, uint32_t& cls_w) {
-        if (MODE == MODE_DENSE) {
+        if (kDense) {
             kt = (int)(e & 0xffffu);
             cls_w = (e >> (16 + 2 * my_qt64_slot)) & 3u;
         } else {
@@ -415,7 +463,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         if (!wave_on) cls_w = TILE_NONE;
     };
     auto list_entry = [&](int it) -> uint32_t {   // wave-uniform
-        if (MODE != MODE_DENSE || n_active <= 0) return 0u;
+        if (!kDense || n_active <= 0) return 0u;
         return __builtin_amdgcn_readfirstlane(tile_list[min(it, n_active - 1)]);
     };
     // mask words of a MIXED dense tile: word [kb][j] covers keys key0 + 32kb + 8j + 4h + 0..3
@@ -500,7 +548,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         // sequence; in a packed batch also keys after the lane's query row) is one compare of a constant with a per-lane
         // limit; dense MIXED tiles test their mask bytes as well.
         if (cls_w == TILE_MIXED || key0 + 64 > seq_len) {
-            const bool use_bytes = MODE == MODE_DENSE && cls_w == TILE_MIXED;
+            const bool use_bytes = kDense && cls_w == TILE_MIXED;
             int lim = last_row - key0 - 4 * h;                              // largest kept 32kb + 8j + e
             if (MODE == MODE_VARLEN) lim = min(lim, qrow - key0 - 4 * h);
 #pragma unroll
@@ -510,7 +558,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
                         bool keep = 32 * kb + 8 * j + e <= lim;
-                        if (MODE == MODE_DENSE) keep = keep && (!use_bytes || ((mw[kb][j] >> (8 * e)) & 0xffu) != 0u);
+                        if (kDense) keep = keep && (!use_bytes || ((mw[kb][j] >> (8 * e)) & 0xffu) != 0u);
                         e_acc[kb][4 * j + e] = keep ? e_acc[kb][4 * j + e] : -INFINITY;
                     }
         }
@@ -593,7 +641,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
 #pragma unroll
         for (int c = 0; c < KC; ++c) qf[c] = T::scale8(lds_read_b128(qa + 16 * ((2 * c + h) ^ sw), 0), c2);
     }
-    if (MODE == MODE_DENSE && n_active > 0 && cls_first == TILE_MIXED) fetch_mask(kt_first);
+    if (kDense && n_active > 0 && cls_first == TILE_MIXED) fetch_mask(kt_first);
     auto iteration = [&](auto stage_tag, int it) {
         constexpr int STAGE = decltype(stage_tag)::value;
         int kt, ktn; uint32_t cls_w, cn;
@@ -604,7 +652,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         __syncthreads();       // everyone's has; stage STAGE^1 is no longer being read
         if (it + 1 < n_active) issue_tile(ktn, STAGE ^ 1);
         if (cls_w != TILE_NONE) process_tile(stage_tag, kt, cls_w);
-        if (MODE == MODE_DENSE && it + 1 < n_active && cn == TILE_MIXED) fetch_mask(ktn);   // after this tile's words were used
+        if (kDense && it + 1 < n_active && cn == TILE_MIXED) fetch_mask(ktn);   // after this tile's words were used
         e_cur = e_next; e_next = e_after;
     };
     for (int it = 0; it < n_active; it += 2) {
@@ -761,6 +809,13 @@ MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k
     const int64_t grid = (int64_t)p.NQ * B * Hkv * p.n_hg;
     if (grid > 0x7fffffffLL) return fail(MINFER_ATTN_EINVAL, "flash_attn: problem too large for one launch");
 
+    // A short problem whose mask rows can be read in 16-byte pieces and whose workgroups all fit on the chip at once
+    // (2 per CU, 256 CUs) needs no pre-pass: its workgroups classify their own rows, which takes 2-3 us off a call of
+    // 9-28 us.  With more workgroups than that the pre-pass is cheaper than every head re-reading the mask rows.
+    if (p.mask_vec && L <= kSelfClassifyMaxL && kWaves == kWavesSmall && grid <= kSelfClassifyMaxGrid) {
+        p.cls = nullptr;
+        return dispatch_prefill_nw<MODE_DENSE_SELF, kWavesSmall>(dtype, D, p, (int)grid, stream);
+    }
     if (p.mask_vec)
         hipLaunchKernelGGL(classify_mask_kernel_256, dim3((p.NKT + 3) / 4, p.NQT, (unsigned)B), dim3(256), 0, stream,
                            mask, (uint8_t*)workspace, p.L, p.NQT, p.NKT);

@@ -128,6 +128,34 @@ def test_dense_matches_oracle(dtype, B, Hq, Hkv, L, D, kind, views):
     assert max_err(out, want) <= TOL[dtype]
 
 
+@pytest.mark.parametrize("B,Hq,Hkv,L,D,kind", [
+    (1, 4, 4, 16, 128, "random"),      # n_rep = 1: four query blocks per workgroup, of which one has rows
+    (2, 4, 2, 48, 64, "full"),         # n_rep = 2
+    (1, 6, 2, 208, 128, "window"),     # n_rep = 3
+    (2, 8, 2, 320, 128, "blocky"),     # n_rep = 4, key tiles that no row of a query block attends
+    (1, 16, 2, 512, 64, "random"),     # n_rep = 8: two head groups
+    (1, 16, 1, 1008, 128, "blocky"),   # n_rep = 16, a last key tile of 48 columns
+    (1, 8, 2, 1024, 128, "random"),    # the longest mask whose rows one wave-wide load covers
+    (3, 32, 8, 512, 128, "blocky"),    # more workgroups than fit on the chip at once: the pre-pass classifies
+])
+def test_short_dense_masks_classified_inside_the_kernel(B, Hq, Hkv, L, D, kind):
+    """A short dense problem with 16-byte readable mask rows launches no classification pre-pass: each workgroup
+    classifies its own mask rows.  Checked against the oracle, and bit for bit against the same call with the mask at an
+    odd address, which takes the pre-pass and the byte-wise mask reads."""
+    dtype = torch.float16
+    gen = torch.Generator().manual_seed(77 * L + Hq)
+    q, k, v = workloads.dense_prefill(B, Hq, Hkv, L, D, dtype, seed=L + Hq + 1, scale=0.5, device=DEV)
+    mask = make_mask(kind, B, L, gen)
+    md = mask.to(DEV)
+    out = run_prefill(q, k, v, md)
+    assert not torch.isnan(out).any()
+    assert max_err(out, oracle.flash_attn(q, k, v, mask)) <= TOL[dtype]
+    shifted = torch.zeros(md.numel() + 1, dtype=torch.bool, device=DEV)[1:].view(md.shape)
+    shifted.copy_(md)
+    assert shifted.data_ptr() % 16 == 1
+    assert torch.equal(run_prefill(q, k, v, shifted), out)
+
+
 def test_cpu_plumbing_config_on_gpu():
     """benchmark configuration 1 (fp32 N(0,1) inputs, S=256, D=64): the same seeded inputs rounded to fp16."""
     q, k, v, mask = workloads.cpu_plumbing(seed=0)
