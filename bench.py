@@ -42,6 +42,34 @@ QKV_TRAFFIC_BYTES = 378663 * 1024           # qkv in one launch, M=K=4096, N=409
 LONG_TRAFFIC_BYTES = 2721654 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
 RAGGED_TRAFFIC_BYTES = 748670 * 1024        # packed ragged prefill (T=20514, Hq=64)
 GEMM_Q8_TRAFFIC_BYTES = 67126 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
+# The kernel sources the counter runs were made against (first 12 hex digits of each file's sha1).  A row one of whose
+# sources has changed since carries "traffic_stale": true, so a constant that describes an earlier kernel says so.
+TRAFFIC_MEASURED_AGAINST = {
+    "attn_common.h": "", "attn_prefill.hip": "", "attn_decode.hip": "", "quant_q8.h": "", "rope.hip": "", "rmsnorm.hip": "", "gemm.hip": "",
+}
+TRAFFIC_ROW_SOURCES = {
+    "": ("attn_common.h", "attn_prefill.hip"), "long_context": ("attn_common.h", "attn_prefill.hip"), "ragged": ("attn_common.h", "attn_prefill.hip"),
+    "decode": ("attn_common.h", "attn_decode.hip"), "decode_q8_0": ("attn_common.h", "attn_decode.hip", "quant_q8.h"),
+    "rope": ("attn_common.h", "rope.hip"), "rope_kv_append": ("attn_common.h", "rope.hip"),
+    "rope_kv_append_q8_0": ("attn_common.h", "rope.hip", "quant_q8.h"), "rope_kv_append_norm": ("attn_common.h", "rope.hip"),
+    "rmsnorm": ("attn_common.h", "rmsnorm.hip"), "gemm": ("attn_common.h", "gemm.hip"), "qkv": ("attn_common.h", "gemm.hip"),
+    "gemm_q8_0": ("attn_common.h", "gemm.hip", "quant_q8.h"),
+}
+
+
+def source_digest(name):
+    import hashlib
+    with open(os.path.join(PKG, "csrc", name), "rb") as f:
+        return hashlib.sha1(f.read()).hexdigest()[:12]
+
+
+def mark_stale_traffic(rec):
+    """Adds "traffic_stale" to every roofline that quotes a traffic constant."""
+    changed = {n for n, d in TRAFFIC_MEASURED_AGAINST.items() if source_digest(n) != d}
+    for row, sources in TRAFFIC_ROW_SOURCES.items():
+        roof = (rec if row == "" else rec[row]).get("roofline", {})
+        if roof.get("traffic") is not None:
+            roof["traffic_stale"] = bool(changed.intersection(sources))
 
 
 class HipEvents:
@@ -530,6 +558,7 @@ def main():
                    "published_reference_us": 605.3,
                    "roofline": mfma_roofline(g_tf, sus_f16, traffic=GEMM_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
                                              kernel="gemm_kernel<F16,[K,N],256x256>", algorithmic_flops=gflops)}
+    mark_stale_traffic(rec)
     if not args.no_cpu_baseline:
         rec["cpu_baseline"] = cpu_baseline(torch, workloads, refs, L)
         rec["decode"]["cpu_baseline"] = cpu_baseline_decode(torch, workloads, refs)

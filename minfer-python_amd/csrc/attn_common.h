@@ -111,6 +111,14 @@ MA_DEV void copy16_global_to_lds(const void* src, void* lds_base) {
 }
 // Same, with the source given as a wave-uniform base plus a 32-bit unsigned per-lane byte offset, which
 // costs no vector ALU work when the offset is loop-invariant.
+//
+// A vector-memory instruction must not read a scalar register earlier than five instructions after a vector
+// instruction (readfirstlane) wrote it.  The compiler keeps that distance for the instructions it emits but cannot see
+// into an asm statement, which itself puts two instructions between.  BASE_FRESH = false is for bases that are scalar
+// values long before the call (a tile loop's row base); BASE_FRESH = true (three more idle issue slots) is for a base
+// computed from per-wave values right before the call.  build.py scans the generated code of every kernel for a copy
+// that reads a scalar register written by a vector instruction fewer than five instructions earlier and fails on one.
+template <bool BASE_FRESH = false>
 MA_DEV void copy16_global_to_lds(const void* uniform_base, uint32_t lane_byte_offset, void* lds_base) {
     const uint32_t dst = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)(lds_void*)lds_base);
     const uint64_t b = (uint64_t)(uintptr_t)uniform_base;
@@ -118,10 +126,16 @@ MA_DEV void copy16_global_to_lds(const void* uniform_base, uint32_t lane_byte_of
     // sign-extended into the high word of the address
     const uint64_t sb = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b >> 32)) << 32) |
                         (uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 :
-                 : "s"(dst), "v"(lane_byte_offset), "s"(sb)
-                 : "memory", "m0");
+    if (BASE_FRESH)
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(dst), "v"(lane_byte_offset), "s"(sb)
+                     : "memory", "m0");
+    else
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                     :
+                     : "s"(dst), "v"(lane_byte_offset), "s"(sb)
+                     : "memory", "m0");
 }
 
 // 32-bit LDS address of a __shared__ object, and reads at such an address plus a compile-time offset

@@ -297,7 +297,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         const short* qbase = Qh + (int64_t)q_row0 * p.q2;
 #pragma unroll
         for (int j = 0; j < 32 / RPI; ++j)
-            copy16_global_to_lds(qbase + (int64_t)(j * RPI) * p.q2, lane_row + 16u * (uint32_t)(g0 ^ GEO::swz_k(j * RPI)), q_stage + j * RPI * RB);
+            copy16_global_to_lds<true>(qbase + (int64_t)(j * RPI) * p.q2, lane_row + 16u * (uint32_t)(g0 ^ GEO::swz_k(j * RPI)), q_stage + j * RPI * RB);
     } else {
 #pragma unroll
         for (int j = 0; j < 32 / RPI; ++j) {
@@ -396,6 +396,10 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         k_off0 = (uint32_t)((int64_t)(lane / G) * p.kv2 + 8 * (pg ^ GEO::swz_k(row))) * 2u;
         v_off0 = (uint32_t)((int64_t)(lane / G) * p.kv2 + 8 * (pg ^ GEO::swz_v(row))) * 2u;
     }
+    // In this one instantiation the compiler (out of scalar registers) keeps the row bases in vector registers and moves
+    // them to scalar ones right in front of every copy, closer than a copy may follow such a move (copy16_global_to_lds);
+    // the build's scan of the generated code is what says which instantiations need this.
+    constexpr bool kFreshBases = MODE == MODE_VARLEN && NW == 4 && D == 128;
     auto issue_tile = [&](int kt, int stage) {
         const int key0 = kt * 64;
         const short* kbase = Kh + (int64_t)key0 * p.kv2;
@@ -404,8 +408,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
 #pragma unroll
             for (int j = 0; j < NLD; ++j) {
                 const int row0 = (j * kWaves + w) * RPI;
-                copy16_global_to_lds(kbase + (int64_t)row0 * p.kv2, k_off0, &kv_lds[stage][row0 * RB]);
-                copy16_global_to_lds(vbase + (int64_t)row0 * p.kv2, v_off0, &kv_lds[stage][GEO::TILE_BYTES + row0 * RB]);
+                copy16_global_to_lds<kFreshBases>(kbase + (int64_t)row0 * p.kv2, k_off0, &kv_lds[stage][row0 * RB]);
+                copy16_global_to_lds<kFreshBases>(vbase + (int64_t)row0 * p.kv2, v_off0, &kv_lds[stage][GEO::TILE_BYTES + row0 * RB]);
             }
         } else {   // tile crossing the end of the sequence: rows past it re-read the last row
 #pragma unroll
@@ -413,8 +417,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
                 const int row0 = (j * kWaves + w) * RPI;
                 const int row = row0 + lane / G, pg = lane % G;
                 const int64_t grow = (int64_t)(min(key0 + row, last_row) - key0) * p.kv2;
-                copy16_global_to_lds(kbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_k(row))) * 2u, &kv_lds[stage][row0 * RB]);
-                copy16_global_to_lds(vbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_v(row))) * 2u, &kv_lds[stage][GEO::TILE_BYTES + row0 * RB]);
+                copy16_global_to_lds<kFreshBases>(kbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_k(row))) * 2u, &kv_lds[stage][row0 * RB]);
+                copy16_global_to_lds<kFreshBases>(vbase, (uint32_t)(grow + 8 * (pg ^ GEO::swz_v(row))) * 2u, &kv_lds[stage][GEO::TILE_BYTES + row0 * RB]);
             }
         }
     };

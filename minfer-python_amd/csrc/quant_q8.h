@@ -12,6 +12,9 @@ struct Q8Block { uint4 lo, hi; uint32_t d; };
 // The four int8 of a word as fp16, exactly: sub-dword addressing lets the int16 -> fp16 conversion take one byte,
 // sign-extended, as its source and one half of the destination as its target, so a value costs one instruction
 // (building q + 1152 under the exponent byte of 1024 with a byte permute and an exclusive or, then subtracting, costs 1.5).
+// The results must pass through an instruction the compiler emits (the multiply by the scale, here) before a matrix
+// instruction reads them: a matrix instruction may read a register two instructions after a vector instruction wrote
+// it at the earliest, and the compiler cannot keep that distance for a write it does not see (measured: stale operands).
 MA_DEV void int8x4_to_f16(uint32_t w, uint32_t& out_lo, uint32_t& out_hi) {
     asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_0 dst_unused:UNUSED_PAD src0_sel:BYTE_0" : "=v"(out_lo) : "v"(w));
     asm("v_cvt_f16_i16_sdwa %0, sext(%1) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_1" : "+v"(out_lo) : "v"(w));

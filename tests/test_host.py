@@ -346,3 +346,24 @@ def test_workload_generators_are_seeded():
     assert workloads.kv_append_bytes(1, 16, 32, 8, 128, 128) == (2 * 16 * 32 * 128 + 4 * 16 * 8 * 128) * 2
     assert workloads.kv_append_bytes_q8_0(1, 16, 32, 8, 128, 128) == 16 * (2 * 32 * 128 * 2 + 2 * 8 * 128 * 2 + 2 * 8 * 136)
     assert workloads.decode_bytes_q8_0([10, 20], 32, 8, 128) == 30 * 8 * 136 * 2 + 2 * 2 * 32 * 128 * 2
+
+
+def test_build_scan_finds_dependences_too_close_to_an_asm_statement():
+    """build.py scans the generated device code for the two distances the compiler cannot keep when one end lies inside
+    an asm statement; the scan itself is checked here on small pieces of assembly text."""
+    import importlib.util
+    spec = importlib.util.spec_from_file_location("minfer_build", f"{capi.ROOT}/minfer-python_amd/build.py")
+    build = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(build)
+    copy = lambda nop: f"\t;;#ASMSTART\n\ts_mov_b32 m0, s2\n\ts_nop {nop}\n\tglobal_load_lds_dwordx4 v16, s[24:25]\n\t;;#ASMEND\n"
+    head = "kernel_a:\n\tv_readfirstlane_b32 s25, v11\n\tv_readfirstlane_b32 s24, v10\n"
+    assert len(build.asm_hazards(head + copy(0))) == 2                       # two issue slots between: too close
+    assert build.asm_hazards(head + copy(3)) == []                          # s_mov + s_nop 3 = five slots
+    assert build.asm_hazards(head + "\tv_add_u32_e32 v1, v2, v3\n" * 3 + copy(0)) == []
+    assert build.asm_hazards(head.replace("s24", "s30").replace("s25", "s31") + copy(0)) == []   # other registers
+    assert build.asm_hazards(head + ".LBB0_1:\n" + copy(0)) != []           # a branch target does not reset the distance
+    cvt = "\t;;#ASMSTART\n\tv_cvt_f16_i16_sdwa v51, sext(v68) dst_sel:WORD_1 dst_unused:UNUSED_PRESERVE src0_sel:BYTE_3\n\t;;#ASMEND\n"
+    mfma = "\tv_mfma_f32_16x16x32_f16 v[26:29], v[50:53], v[58:61], v[26:29]\n"
+    assert len(build.asm_hazards("kernel_b:\n" + cvt + "\tv_pk_mul_f16 v63, v63, v136\n" + mfma)) == 1
+    assert build.asm_hazards("kernel_b:\n" + cvt + "\tv_pk_mul_f16 v63, v63, v136\n" * 2 + mfma) == []
+    assert build.asm_hazards("kernel_b:\n" + cvt.replace("v51", "v70") + mfma) == []
