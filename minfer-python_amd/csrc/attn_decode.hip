@@ -439,7 +439,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
     int inner_off[NL];
 #pragma unroll
     for (int j = 0; j < NL; ++j) inner_off[j] = min(16 * (64 * j + lane), 16 * (NG - 1));
-    auto load_group = [&](auto inner_tag, int t, Stage& st) __attribute__((always_inline)) {
+    // K's and V's pieces of a group are requested separately: each as soon as the registers that receive them have
+    // handed the group before over to LDS (at the start and in the middle of that group's turn, not after it), so that
+    // a request has the better part of two turns to come back.
+    auto load_k = [&](auto inner_tag, int t, Stage& st) __attribute__((always_inline)) {
         constexpr bool INNER = decltype(inner_tag)::value;
         const int64_t inner_goff = (int64_t)(row_lo + t * GR) * ROWB;
 #pragma unroll
@@ -448,6 +451,10 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
             const int off = INNER ? inner_off[j] : piece_offset(t, j, last_k, goff);
             st.k[j] = stream_load(reinterpret_cast<const u32x4*>(kb16 + goff + off));
         }
+    };
+    auto load_v = [&](auto inner_tag, int t, Stage& st) __attribute__((always_inline)) {
+        constexpr bool INNER = decltype(inner_tag)::value;
+        const int64_t inner_goff = (int64_t)(row_lo + t * GR) * ROWB;
 #pragma unroll
         for (int j = 0; j < NL; ++j) {
             int64_t goff = inner_goff;
@@ -458,7 +465,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
     const std::false_type general_tag{};
     const std::true_type inner_group_tag{};
 #pragma unroll
-    for (int s = 0; s < NS; ++s) load_group(general_tag, s, ring[s]);
+    for (int s = 0; s < NS; ++s) { load_k(general_tag, s, ring[s]); load_v(general_tag, s, ring[s]); }
 
     f32x4 o_acc[DB];
 #pragma unroll
@@ -480,7 +487,8 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
         return h16x2{dh, dh};
     };
 
-    auto consume = [&](auto inner_tag, int t, const Stage& st) __attribute__((always_inline)) {
+    // (next_tag: whether group t + NS, requested during this turn, is an inner one)
+    auto consume = [&](auto inner_tag, auto next_tag, int t, Stage& st) __attribute__((always_inline)) {
         constexpr bool INNER = decltype(inner_tag)::value;
         const int r0 = row_lo + t * GR;
         int64_t goff;
@@ -490,6 +498,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
             const int off = INNER ? inner_off[j] : piece_offset(t, j, last_k, goff);
             *reinterpret_cast<u32x4*>(raw_k + off) = st.k[j];
         }
+        load_k(next_tag, t + NS, st);
         // ---- S^T = K Q^T for the two 16-key halves: lane gets head l16, keys 16h + 4*quad + r ---------------
         f32x4 s[2];
 #pragma unroll
@@ -520,6 +529,7 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
             const int off = INNER ? inner_off[j] : piece_offset(t, j, last_v, goff);
             *reinterpret_cast<u32x4*>(raw_v + off) = st.v[j];
         }
+        load_v(next_tag, t + NS, st);
 #pragma unroll
         for (int i = 0; i < GR * BPR / 64; ++i) {
             const int idx = 64 * i + lane, row = idx / BPR, c = idx % BPR;
@@ -583,17 +593,12 @@ __global__ __launch_bounds__(kDecodeWaves * 64, kDecodeWavesPerSimd) void decode
     // rounds in which every group consumed and every group requested is an inner one
     for (; t0 + 2 * NS < n_groups; t0 += NS) {
 #pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            consume(inner_group_tag, t0 + s, ring[s]);
-            load_group(inner_group_tag, t0 + s + NS, ring[s]);
-        }
+        for (int s = 0; s < NS; ++s) consume(inner_group_tag, inner_group_tag, t0 + s, ring[s]);
     }
     for (; t0 < n_groups; t0 += NS) {
 #pragma unroll
-        for (int s = 0; s < NS; ++s) {
-            if (t0 + s < n_groups) consume(general_tag, t0 + s, ring[s]);
-            load_group(general_tag, t0 + s + NS, ring[s]);
-        }
+        for (int s = 0; s < NS; ++s)
+            if (t0 + s < n_groups) consume(general_tag, general_tag, t0 + s, ring[s]);
     }
 
     // ---- the segment's partial result: un-normalised O, reference max and sum of every head -------------
