@@ -30,22 +30,28 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # These are figures from those earlier counter runs, not measured in the run that prints them.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels_pmc.md (rocprofv3 --pmc runs of the same workloads; not re-measured by this run)"
 PREFILL_TRAFFIC_BYTES = 107400 * 1024
-DECODE_TRAFFIC_BYTES = 1092838 * 1024
-ROPE_TRAFFIC_BYTES = 393312 * 1024          # il_rope on [8,4096,48,128], rotary 64
+DECODE_TRAFFIC_BYTES = 1092850 * 1024
+ROPE_TRAFFIC_BYTES = 393314 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
-NORM_TRAFFIC_BYTES = 786659 * 1024          # rmsnorm on [8,4096,6144]
-GEMM_TRAFFIC_BYTES = 230260 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
-DECODE_Q8_TRAFFIC_BYTES = 598453 * 1024     # decode over Q8_0 caches (split + combine)
-APPEND_Q8_TRAFFIC_BYTES = 737585 * 1024     # rope_kv_append into Q8_0 caches
-APPEND_NORM_TRAFFIC_BYTES = 786620 * 1024   # rope_kv_append_norm, the same shape
-QKV_TRAFFIC_BYTES = 378663 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
-LONG_TRAFFIC_BYTES = 2721654 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
-RAGGED_TRAFFIC_BYTES = 748670 * 1024        # packed ragged prefill (T=20514, Hq=64)
-GEMM_Q8_TRAFFIC_BYTES = 67126 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
+NORM_TRAFFIC_BYTES = 786691 * 1024          # rmsnorm on [8,4096,6144]
+GEMM_TRAFFIC_BYTES = 230270 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
+DECODE_Q8_TRAFFIC_BYTES = 598274 * 1024     # decode over Q8_0 caches (split + combine)
+APPEND_Q8_TRAFFIC_BYTES = 737591 * 1024     # rope_kv_append into Q8_0 caches
+APPEND_NORM_TRAFFIC_BYTES = 786609 * 1024   # rope_kv_append_norm, the same shape
+QKV_TRAFFIC_BYTES = 379200 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
+LONG_TRAFFIC_BYTES = 2721732 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
+RAGGED_TRAFFIC_BYTES = 748602 * 1024        # packed ragged prefill (T=20514, Hq=64)
+GEMM_Q8_TRAFFIC_BYTES = 67806 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
 # The kernel sources the counter runs were made against (first 12 hex digits of each file's sha1).  A row one of whose
 # sources has changed since carries "traffic_stale": true, so a constant that describes an earlier kernel says so.
 TRAFFIC_MEASURED_AGAINST = {
-    "attn_common.h": "", "attn_prefill.hip": "", "attn_decode.hip": "", "quant_q8.h": "", "rope.hip": "", "rmsnorm.hip": "", "gemm.hip": "",
+    "attn_common.h": "4188ced83d04",
+    "attn_prefill.hip": "9a7e568fd938",
+    "attn_decode.hip": "af41b9ac94d8",
+    "quant_q8.h": "4fea6a94e300",
+    "rope.hip": "b4fd0618b44e",
+    "rmsnorm.hip": "f6c4e575f461",
+    "gemm.hip": "79aa2eb1378f",
 }
 TRAFFIC_ROW_SOURCES = {
     "": ("attn_common.h", "attn_prefill.hip"), "long_context": ("attn_common.h", "attn_prefill.hip"), "ragged": ("attn_common.h", "attn_prefill.hip"),
