@@ -546,7 +546,7 @@ def main():
     rec["gemm_q8_0"] = {"value": q8_gbs, "unit": "GB/s", "ms": q8_avg_ms, "median_ms": q8_med_ms,
                         "workload": "one token against a weight of Q8_0 blocks: x [1,1,4096] fp16, W uint8 [14336, 4352] (Llama-3-8B FFN up), out fp16",
                         "roofline": {"bound": "hbm", "achieved": q8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": q8_gbs / PEAK_HBM_GBS,
-                                     "traffic": GEMM_Q8_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_skinny_q8_kernel<1,1>", "algorithmic_bytes": q8bytes}}
+                                     "traffic": GEMM_Q8_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemv_q8_kernel<activations in registers>", "algorithmic_bytes": q8bytes}}
     rec["cpu_plumbing"] = {"value": cflops / (c_avg_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms": c_avg_ms, "median_ms": c_med_ms,
                            "workload": "prefill B=1 Hq=8 Hkv=2 S=256 D=64 causal dense-mask, fp32 inputs rounded to fp16 for the GPU op (BASELINE configs[0]); launch-bound"}
     rec["calibration"] = {"mfma_only_f16_random": sus_f16, "mfma_only_bf16_random": sus_bf16,

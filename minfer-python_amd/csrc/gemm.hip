@@ -406,6 +406,122 @@ static void launch_skinny_nr(const GemmParams& p, hipStream_t stream) {
     else if (mb == 3) hipLaunchKernelGGL((gemm_skinny_kernel<T, 3, NR>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((gemm_skinny_kernel<T, 4, NR>), grid, block, 0, stream, p);
 }
+// One row against an [N, K] weight (a decode step's projection): a wave streams whole weight rows as consecutive 16-byte
+// pieces (1 KiB per instruction, where the MFMA kernel above takes 128 bytes of each of 16 rows) and multiplies in the
+// vector ALU, which one activation row leaves mostly idle; one fp32 sum per lane, added up over the lanes at the end of
+// a row.  A row is cut into segments of 4096 values (8 pieces per lane); when it is a single segment the lane keeps the
+// activations it needs in registers (XREG), otherwise the workgroup keeps the activation row in LDS.  A wave owns a run
+// of consecutive rows and has the next two segments in flight.
+constexpr int kGemvSegHalfs = 4096;
+constexpr int kGemvSegPieces = kGemvSegHalfs / 8 / 64;     // 16-byte pieces per lane and segment
+template <class T> MA_DEV float dot8(uint4 a, uint4 b, float acc);
+template <> MA_DEV float dot8<F16>(uint4 a, uint4 b, float acc) {
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, a.x), __builtin_bit_cast(h16x2, b.x), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, a.y), __builtin_bit_cast(h16x2, b.y), acc, false);
+    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, a.z), __builtin_bit_cast(h16x2, b.z), acc, false);
+    return __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, a.w), __builtin_bit_cast(h16x2, b.w), acc, false);
+}
+template <> MA_DEV float dot8<BF16>(uint4 a, uint4 b, float acc) {   // a bf16 is the upper half of the fp32 of the same value
+    const uint32_t aw[4] = {a.x, a.y, a.z, a.w}, bw[4] = {b.x, b.y, b.z, b.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc = __builtin_fmaf(__builtin_bit_cast(float, aw[i] << 16), __builtin_bit_cast(float, bw[i] << 16), acc);
+        acc = __builtin_fmaf(__builtin_bit_cast(float, aw[i] & 0xffff0000u), __builtin_bit_cast(float, bw[i] & 0xffff0000u), acc);
+    }
+    return acc;
+}
+constexpr int kGemvMaxKHalfs = 16384;                      // activation row kept in LDS: 32 KiB
+// GROUPED: the rows of up to three weights numbered through (p.grp.end[s] = rows of weights 0 .. s), every weight with
+// its own output; alpha = 1, no C.
+template <class T, bool XREG, bool GROUPED>
+__global__ __launch_bounds__(4 * 64) void gemv_kernel(const GemmParams p, int rows_per_wave) {
+    __shared__ __attribute__((aligned(16))) short x_lds[XREG ? 8 : kGemvMaxKHalfs];
+    const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
+    const int npiece = p.K / 8, nseg = XREG ? 1 : (p.K + kGemvSegHalfs - 1) / kGemvSegHalfs;
+    const int wave = (int)blockIdx.x * 4 + w;
+    const int n_rows = GROUPED ? p.grp.end[kMaxGroup - 1] : p.N;
+    const int r0 = min(wave * rows_per_wave, n_rows - 1), r1 = min(n_rows, wave * rows_per_wave + rows_per_wave);
+    const int units = max(r1 - r0, 0) * nseg;              // (row, segment) pairs of this wave (none for a wave past the rows)
+    // where row number `row` lives: its weight row and its output element (wave-uniform)
+    auto locate = [&](int row, const short*& wrow, short*& out) {
+        if (GROUPED) {
+            const int sg = (row >= p.grp.end[0]) + (row >= p.grp.end[1]);
+            const int local = row - (sg == 0 ? 0 : sg == 1 ? p.grp.end[0] : p.grp.end[1]);
+            wrow = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]) +
+                   (int64_t)local * (sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2]);
+            out = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]) + local;
+        } else {
+            wrow = (const short*)p.B + (int64_t)row * p.ldb;
+            out = (short*)p.D + row;
+        }
+    };
+    struct Unit { uint4 piece[kGemvSegPieces]; };
+    auto request = [&](int u, Unit& un) {
+        u = max(min(u, units - 1), 0);                     // past the end: the last unit again, never used
+        const int row = r0 + u / nseg, seg = u % nseg;
+        const short* base; short* unused;
+        locate(row, base, unused);
+#pragma unroll
+        for (int j = 0; j < kGemvSegPieces; ++j)
+            un.piece[j] = __builtin_bit_cast(uint4, stream_load(reinterpret_cast<const u32x4*>(base + 8 * min(seg * (kGemvSegHalfs / 8) + 64 * j + lane, npiece - 1))));
+    };
+    Unit ring[2];
+    request(0, ring[0]);
+    request(1, ring[1]);
+    uint4 xr[kGemvSegPieces];
+    if (XREG) {
+#pragma unroll
+        for (int j = 0; j < kGemvSegPieces; ++j)
+            xr[j] = *reinterpret_cast<const uint4*>((const short*)p.A + 8 * min(64 * j + lane, npiece - 1));
+    } else {
+        for (int i = tid; i < npiece; i += 4 * 64)
+            *reinterpret_cast<uint4*>(x_lds + 8 * i) = *reinterpret_cast<const uint4*>((const short*)p.A + 8 * i);
+        __syncthreads();
+    }
+    float acc = 0.f;
+    auto consume = [&](int u, Unit& un) {
+        const int row = r0 + u / nseg, seg = u % nseg;
+        uint4 wv[kGemvSegPieces];
+#pragma unroll
+        for (int j = 0; j < kGemvSegPieces; ++j) wv[j] = un.piece[j];
+        request(u + 2, un);
+#pragma unroll
+        for (int j = 0; j < kGemvSegPieces; ++j) {
+            const int piece = seg * (kGemvSegHalfs / 8) + 64 * j + lane;
+            if (piece < npiece) acc = dot8<T>(wv[j], XREG ? xr[j] : *reinterpret_cast<const uint4*>(x_lds + 8 * piece), acc);
+        }
+        if (seg == nseg - 1) {
+            float v = acc;
+            acc = 0.f;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+            if (lane == 0) {
+                const short* unused; short* out;
+                locate(row, unused, out);
+                if (!GROUPED) {
+                    v *= p.alpha;
+                    if (p.beta != 0.f) v += p.beta * T::to_float(((const short*)p.C)[row]);
+                }
+                *out = (short)(T::pack2(v, 0.f) & 0xffffu);
+            }
+        }
+    };
+    for (int u = 0; u < units; u += 2) {
+        consume(u, ring[0]);
+        if (u + 1 < units) consume(u + 1, ring[1]);
+    }
+}
+template <class T, bool GROUPED = false>
+static int launch_gemv(const GemmParams& p, int n_rows, hipStream_t stream) {
+    const int max_waves = 256 * 2 * 4;   // two workgroups of four waves per compute unit
+    const int rows_per_wave = (n_rows + max_waves - 1) / max_waves;
+    const int waves = (n_rows + rows_per_wave - 1) / rows_per_wave;
+    const dim3 grid((waves + 3) / 4), block(4 * 64);
+    if (p.K <= kGemvSegHalfs) hipLaunchKernelGGL((gemv_kernel<T, true, GROUPED>), grid, block, 0, stream, p, rows_per_wave);
+    else hipLaunchKernelGGL((gemv_kernel<T, false, GROUPED>), grid, block, 0, stream, p, rows_per_wave);
+    return check_launch("gemv_kernel");
+}
+
 template <class T>
 static int launch_skinny(const GemmParams& p, hipStream_t stream) {
     // two column groups per workgroup once that still leaves 160 workgroups and there is more than one block of rows
@@ -511,6 +627,128 @@ __global__ __launch_bounds__(kSkinnyWaves * 64) void gemm_skinny_q8_kernel(const
     pk.x = T::pack2(v[0], v[1]);
     pk.y = T::pack2(v[2], v[3]);
     *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+}
+
+// One row against Q8_0 weights (a decode step's projections): the MFMA kernel above reads 136 bytes of each of 16 weight
+// rows per instruction, which this chip's memory system serves at about half its rate.  Here a wave streams whole weight
+// rows instead, as consecutive aligned 16-byte pieces (1 KiB per instruction), and does the arithmetic in the vector
+// ALU, of which one activation row needs little: a weight row is cut into segments of 128 blocks (4352 bytes, a multiple
+// of 16, which is why K must be a multiple of 256 and the rows 16-byte aligned); a segment's pieces go through the wave's
+// LDS area, from which lane l takes blocks l and l + 64 as the nine aligned words that cover each (as
+// gemm_skinny_q8_kernel does), dequantises them exactly as minfer_dequant_q8_0 does and multiplies them with the
+// activations of the same positions into one fp32 sum per lane; after a row's last segment the 64 sums are added up.
+// The activations a lane needs are the same for every weight row when a row is one segment (K <= 4096, XREG): it keeps
+// them in registers; otherwise the workgroup keeps the activation row in LDS.  A wave owns a run of consecutive weight
+// rows and always has the next two segments' pieces in flight.  (Two rows this way cost as much as the MFMA kernel, four
+// half as much again: the dot products fill the vector ALU.)
+constexpr int kGemvWaves = 4;
+constexpr int kGemvSegBlocks = 128;                       // blocks per segment: two per lane
+constexpr int kGemvSegBytes = kGemvSegBlocks * 34;        // 4352
+constexpr int kGemvPieces = (kGemvSegBytes + 1023) / 1024;   // 16-byte pieces per lane and segment (5, the last one partly)
+constexpr int kGemvMaxK = 16384;                          // activation row kept in LDS: 32 KiB
+template <bool XREG>
+__global__ __launch_bounds__(kGemvWaves * 64) void gemv_q8_kernel(const GemmParams p, int rows_per_wave) {
+    using T = F16;
+    __shared__ __attribute__((aligned(16))) char raw[kGemvWaves][kGemvSegBytes + 48];   // + the words a last block's read runs over
+    __shared__ __attribute__((aligned(16))) short x_lds[XREG ? 8 : kGemvMaxK];
+    const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
+    const int nblk = p.K / 32, nseg = XREG ? 1 : (nblk + kGemvSegBlocks - 1) / kGemvSegBlocks;
+    const int wave = (int)blockIdx.x * kGemvWaves + w;
+    const int r0 = min(wave * rows_per_wave, p.N - 1), r1 = min(p.N, wave * rows_per_wave + rows_per_wave);
+    const int units = max(r1 - r0, 0) * nseg;              // (row, segment) pairs of this wave, row-major (none for a wave past the rows)
+    const bool odd = (lane & 1) != 0;                      // blocks l and l + 64 start 2 bytes past a word boundary
+    const uint32_t sel = odd ? kQ8SelOdd : kQ8SelEven;
+    char* my_raw = raw[w];
+
+    struct Unit { u32x4 piece[kGemvPieces]; };
+    auto request = [&](int u, Unit& un) {
+        u = max(min(u, units - 1), 0);                     // past the end: the last unit again (one cache line, never used)
+        const int row = r0 + u / nseg, seg = u % nseg;
+        const int pieces = min(kGemvSegBlocks, nblk - seg * kGemvSegBlocks) * 34 / 16;   // a multiple of 8 blocks: whole pieces
+        const char* base = (const char*)p.B + (int64_t)row * p.ldb + (int64_t)seg * kGemvSegBytes;
+#pragma unroll
+        for (int j = 0; j < kGemvPieces; ++j)
+            un.piece[j] = *reinterpret_cast<const u32x4*>(base + 16 * min(64 * j + lane, pieces - 1));
+    };
+    Unit ring[2];
+    request(0, ring[0]);
+    request(1, ring[1]);
+    // ---- the activations, while the first weight pieces are on their way ---------------------------------
+    uint4 xr[2][4];
+    if (XREG) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                xr[i][j] = *reinterpret_cast<const uint4*>((const short*)p.A + 32 * min(lane + 64 * i, nblk - 1) + 8 * j);
+    } else {
+        for (int i = tid; i < p.K / 8; i += kGemvWaves * 64)
+            *reinterpret_cast<s16x8*>(x_lds + 8 * i) = *reinterpret_cast<const s16x8*>((const short*)p.A + 8 * i);
+        __syncthreads();
+    }
+    float acc = 0.f;
+    auto consume = [&](int u, Unit& un) {
+        const int row = r0 + u / nseg, seg = u % nseg;
+        const int seg_blocks = min(kGemvSegBlocks, nblk - seg * kGemvSegBlocks);
+        const int pieces = seg_blocks * 34 / 16;
+#pragma unroll
+        for (int j = 0; j < kGemvPieces; ++j)
+            *reinterpret_cast<u32x4*>(my_raw + 16 * min(64 * j + lane, pieces - 1)) = un.piece[j];
+        request(u + 2, un);                                // the registers are free again: two units ahead
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int b = lane + 64 * i;
+            if (b < seg_blocks) {
+                const uint32_t* wp = reinterpret_cast<const uint32_t*>(my_raw + ((34 * b) & ~3));
+                uint32_t wq[9];
+#pragma unroll
+                for (int j = 0; j < 9; ++j) wq[j] = wp[j];
+                const uint16_t bits = (uint16_t)(odd ? wq[0] >> 16 : wq[0]);
+                const _Float16 dh = __builtin_bit_cast(_Float16, bits);
+                const h16x2 d2 = {dh, dh};
+                const short* xb = x_lds + (XREG ? 0 : 32 * (seg * kGemvSegBlocks + b));
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const uint4 wf = __builtin_bit_cast(uint4, dequant8_shifted(wq[2 * j], wq[2 * j + 1], wq[2 * j + 2], sel, d2));
+                    const uint4 xv = XREG ? xr[i][j] : *reinterpret_cast<const uint4*>(xb + 8 * j);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, wf.x), __builtin_bit_cast(h16x2, xv.x), acc, false);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, wf.y), __builtin_bit_cast(h16x2, xv.y), acc, false);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, wf.z), __builtin_bit_cast(h16x2, xv.z), acc, false);
+                    acc = __builtin_amdgcn_fdot2(__builtin_bit_cast(h16x2, wf.w), __builtin_bit_cast(h16x2, xv.w), acc, false);
+                }
+            }
+        }
+        if (seg == nseg - 1) {                             // the row is complete: add the lanes' sums up and store
+            float v = acc;
+            acc = 0.f;
+#pragma unroll
+            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+            if (lane == 0) {
+                v *= p.alpha;
+                if (p.beta != 0.f) v += p.beta * T::to_float(((const short*)p.C)[row]);
+                ((short*)p.D)[row] = (short)(T::pack2(v, 0.f) & 0xffffu);
+            }
+        }
+    };
+    for (int u = 0; u < units; u += 2) {
+        consume(u, ring[0]);
+        if (u + 1 < units) consume(u + 1, ring[1]);
+    }
+}
+
+// which calls the row-streaming kernel takes: one row, whole segments of 16-byte pieces, an activation row that fits its LDS area
+static bool q8_gemv_ok(int64_t M, int64_t K, const void* Bq, int64_t row_bytes) {
+    return M == 1 && K % 256 == 0 && K <= kGemvMaxK && aligned16(Bq) && row_bytes % 16 == 0;
+}
+static int launch_gemv_q8(const GemmParams& p, hipStream_t stream) {
+    // as many waves as the chip holds at a time when there are rows enough for them: two workgroups per compute unit
+    const int max_waves = 256 * 2 * kGemvWaves;
+    const int rows_per_wave = (p.N + max_waves - 1) / max_waves;
+    const int waves = (p.N + rows_per_wave - 1) / rows_per_wave;
+    const dim3 grid((waves + kGemvWaves - 1) / kGemvWaves), block(kGemvWaves * 64);
+    if (p.K <= 32 * kGemvSegBlocks) hipLaunchKernelGGL((gemv_q8_kernel<true>), grid, block, 0, stream, p, rows_per_wave);
+    else hipLaunchKernelGGL((gemv_q8_kernel<false>), grid, block, 0, stream, p, rows_per_wave);
+    return check_launch("gemv_q8_kernel");
 }
 
 static int launch_skinny_q8(const GemmParams& p, hipStream_t stream) {
@@ -650,6 +888,11 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
         }
         return acc;
     };
+    if (p.M == 1 && p.K <= kGemvMaxKHalfs && n_sum <= 0x7fffffffLL) {   // one row: whole weight rows per wave, numbered through
+        int acc = 0;
+        for (int s = 0; s < kMaxGroup; ++s) { if (s < n_w) acc += p.grp.N[s]; p.grp.end[s] = acc; }
+        return launch_gemv<T, true>(p, (int)n_sum, stream);
+    }
     if (p.M <= 32 || (p.M <= 64 && n_sum * p.K <= (INT64_C(1) << 25))) {
         const int nr = (p.M > 16 && n_sum >= 160 * 32) ? 2 : 1;
         const int groups = fill_ends(16 * nr);
@@ -759,6 +1002,8 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     const int splits = fast && workspace && aligned16(workspace) ? gemm_splits(M, N, K) : 1;
     const bool can_split = splits > 1 && workspace_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
     // (with a workspace, K slices of the tiled kernel overtake it from 17 rows on: 32 rows against 4096 x 14336, 28 us against 52)
+    if (fast && nt && M == 1 && K <= kGemvMaxKHalfs)
+        return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
     if (fast && nt && (M <= 16 || (!can_split && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))))
         return dtype == MINFER_ATTN_F16 ? launch_skinny<F16>(p, stream) : launch_skinny<BF16>(p, stream);
     if (can_split) {
@@ -826,6 +1071,7 @@ MINFER_ATTN_EXPORT int minfer_gemm_q8_0(const void* A, const void* Bq, const voi
         GemmParams p{};
         p.A = A; p.B = Bq; p.C = beta != 0.0 ? C : nullptr; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
         p.lda = lda; p.ldb = row_bytes; p.ldc = ldc; p.ldd = ldd; p.alpha = (float)alpha; p.beta = (float)beta;
+        if (q8_gemv_ok(M, K, Bq, row_bytes)) return launch_gemv_q8(p, stream);
         return launch_skinny_q8(p, stream);
     }
     // otherwise: the weight as fp16 in the workspace, then the fp16 kernels on it

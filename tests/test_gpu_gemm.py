@@ -63,6 +63,13 @@ def make(M, N, K, layout, dtype, seed):
     (17, 4104, 64, 1.0, 1.0),        # one K step: seven of the eight waves have nothing to add
     (64, 6144, 4096, 2.0, 3.0),      # 64 rows, two column groups per workgroup: the few-row kernel's largest instantiation
     (40, 5128, 1024, 1.0, 1.0),      # 40 rows (three row blocks), two column groups, the last one ragged
+    # one row against an [N, K] weight: whole weight rows per wave (segments of 4096 values)
+    (1, 4096, 4096, 1.0, 0.0),       # one segment, the activations in registers; two rows per wave
+    (1, 1000, 4160, 2.0, 3.0),       # a second segment of 64 values, the activations in LDS
+    (1, 20000, 64, 2.0, 3.0),        # ten short rows per wave
+    (1, 264, 16384, 1.0, 1.0),       # the longest activation row its LDS area holds
+    (1, 264, 16448, 1.0, 0.0),       # longer: the 16-rows-per-instruction kernel
+    (1, 8, 192, 1.0, 1.0),           # two waves with rows, the others none
 ])
 def test_gemm_matches_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, M + N + K)
@@ -131,7 +138,9 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
     (4096, 128, 4096, 2048, 2048),     # 8192 columns: no multiple of 192, 256 x 256 tiles per weight
     (512, 6144, 6144, 1024, 1024),     # the reference test's head shape at a smaller batch: 128 x 128 tiles
     (300, 256, 200, 72, 136),          # ragged rows, widths that end inside a tile
-    (1, 4096, 4096, 1024, 1024),       # a decode step: the few-row kernel over the three weights' column groups
+    (1, 4096, 4096, 1024, 1024),       # a decode step: whole weight rows per wave, the three weights' rows numbered through
+    (1, 8192, 1032, 8, 520),           # the same with the activations in LDS and runs of rows that cross from one weight to the next
+    (2, 4096, 4096, 1024, 1024),       # two rows: the few-row kernel over the three weights' column groups
     (24, 1024, 5120, 1280, 1288),      # few rows, two column groups per workgroup, a ragged last group
     (64, 512, 768, 256, 256),          # few-row kernel at its largest row count
     (33, 50, 17, 17, 9),               # nothing tileable: three plain launches
@@ -273,6 +282,15 @@ def make_q8(M, N, K, seed):
     (5, 64, 96, 1.0, 1.0),           # an odd number of blocks per row: workspace path at any row count
     (3, 18, 256, 1.0, 1.0),          # out_dim not a multiple of 4 with few rows: workspace path as well
     (64, 1030, 128, 2.0, 0.0),
+    # one row with K a multiple of 256: the kernel that streams whole weight rows (segments of 128 blocks)
+    (1, 264, 14336, 2.0, 1.0),       # three whole segments and one of 64 blocks, the activations in LDS
+    (1, 520, 4352, 1.0, 0.0),        # a last segment of 8 blocks
+    (1, 2052, 768, 0.5, 1.0),        # a single segment of 24 blocks, the activations in registers
+    (1, 20000, 256, 1.0, 1.0),       # ten weight rows per wave
+    (1, 4, 256, 1.0, 0.0),           # one wave with four rows, the others none
+    (1, 4096, 16384, 1.0, 0.0),      # the longest activation row its LDS area holds
+    (1, 512, 16640, 1.0, 0.0),       # longer: back to the 16-rows-per-instruction kernel
+    (2, 2052, 768, 0.5, 1.0),        # two rows: that kernel as well
 ])
 def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
     a, wq, c, w_deq = make_q8(M, N, K, seed=M * 7 + N + K)
