@@ -406,6 +406,107 @@ static void launch_skinny_nr(const GemmParams& p, hipStream_t stream) {
     else if (mb == 3) hipLaunchKernelGGL((gemm_skinny_kernel<T, 3, NR>), grid, block, 0, stream, p);
     else hipLaunchKernelGGL((gemm_skinny_kernel<T, 4, NR>), grid, block, 0, stream, p);
 }
+// The few-row kernel for large weights.  gemm_skinny_kernel's weight loads put 16 different weight rows into every
+// quarter of a wave, 16 cache lines touched for 256 bytes, and that, not HBM, is what it runs at (4.5 TB/s of the weight
+// at any row count).  Here the weight rows and the activation rows take the long way round: global -> LDS copies whose
+// lanes walk along the rows (a copy instruction moves 256 consecutive bytes of each of four rows, 4 lines per quarter
+// wave), and the MFMA fragments are read back from LDS.  A workgroup of four waves owns 16 columns; wave w takes every
+// fourth 128-wide K segment, each wave with its own two-stage LDS area (no barrier until the final sum): per segment
+// 4 copies for the 16 weight rows, 4 for up to 16 activation rows, 4 MFMAs.  Four rows of a copy share a 1 KiB block
+// of LDS, blocks 64 bytes apart in the banks, so that the 16 rows of a fragment read hit 16 different bank groups.
+constexpr int kRowsSeg = 128;                                  // K values per segment
+constexpr int kRowsBlock = 1024 + 64;                          // LDS bytes of four rows' segment, padded
+constexpr int kRowsStage = 4 * kRowsBlock;                     // 16 rows
+// XI: copy instructions that hold activation rows (four rows each, M <= 4 * XI); fragment columns past them multiply
+// whatever their LDS block holds into output columns that are never stored.
+// GROUPED: the 16-column groups of up to three weights numbered through (p.grp.end in groups), alpha = 1 and no C.
+template <class T, int XI, bool GROUPED>
+__global__ __launch_bounds__(4 * 64) void gemm_rows_lds_kernel(const GemmParams p) {
+    __shared__ __attribute__((aligned(16))) char wx[4][2][2][kRowsStage];   // [wave][stage][weights, activations]
+    __shared__ f32x4 part[4][64];
+    const int lane = threadIdx.x & 63, w = wave_id();
+    const int l16 = lane & 15, quad = lane >> 4;
+    int n0 = (int)blockIdx.x * 16;
+    const short* Bg = (const short*)p.B;
+    short* Dg = (short*)p.D;
+    int N = p.N;
+    int64_t ldb = p.ldb, ldd = p.ldd;
+    if (GROUPED) {   // the workgroup's weight, output and place inside them (uniform)
+        int local;
+        const int sg = group_of_unit(p.grp, (int)blockIdx.x, local);
+        n0 = local * 16;
+        Bg = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]);
+        Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
+        N = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
+        ldb = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
+        ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
+    }
+    const int nseg = p.K / kRowsSeg;                           // a multiple of 4: every wave the same number
+    const int per = nseg / 4;
+    // copy instruction i of a segment: lane L takes piece L >> 2 of row 4i + (L & 3)
+    const short* wsrc[4];
+    const short* xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        wsrc[i] = Bg + (int64_t)min(n0 + 4 * i + (lane & 3), N - 1) * ldb + 8 * (lane >> 2);
+        xsrc[i] = (const short*)p.A + (int64_t)min(4 * i + (lane & 3), p.M - 1) * p.lda + 8 * (lane >> 2);
+    }
+    auto issue = [&](int t, int stage) {                       // the wave's t-th segment
+        const int k0 = (4 * t + w) * kRowsSeg;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) copy16_global_to_lds(wsrc[i] + k0, &wx[w][stage][0][i * kRowsBlock]);
+#pragma unroll
+        for (int i = 0; i < XI; ++i) copy16_global_to_lds(xsrc[i] + k0, &wx[w][stage][1][i * kRowsBlock]);
+    };
+    // fragment of k step s (32 values) for row r = l16: piece 4s + quad of the row, inside the row's block of four
+    const int frag = (l16 >> 2) * kRowsBlock + 16 * (l16 & 3) + 64 * quad;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    issue(0, 0);
+    for (int t = 0; t < per; ++t) {
+        if (t + 1 < per) { issue(t + 1, (t + 1) & 1); wait_vmcnt<4 + XI>(); } else wait_vmcnt<0>();
+        const char* wb = &wx[w][t & 1][0][frag];
+        const char* xb = &wx[w][t & 1][1][frag];
+#pragma unroll
+        for (int s = 0; s < kRowsSeg / 32; ++s) {
+            const s16x8 a = *reinterpret_cast<const s16x8*>(wb + 256 * s);
+            const s16x8 b = *reinterpret_cast<const s16x8*>(xb + 256 * s);
+            acc = T::mfma16(a, b, acc);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // the fragments are in registers before the stage is refilled
+    }
+    part[w][lane] = acc;
+    __syncthreads();
+    if (w != 0) return;
+    f32x4 sum = part[0][lane];
+#pragma unroll
+    for (int ww = 1; ww < 4; ++ww) sum += part[ww][lane];
+    const int m = l16, n = n0 + 4 * quad;      // register r of a lane: weight row n + r, activation row m
+    if (m >= p.M || n >= N) return;
+    float v[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) v[e] = GROUPED ? sum[e] : p.alpha * sum[e];
+    if (!GROUPED && p.beta != 0.f) {
+        const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+    }
+    uint2 pk;
+    pk.x = T::pack2(v[0], v[1]);
+    pk.y = T::pack2(v[2], v[3]);
+    *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
+}
+// (16 rows at most, K a multiple of 512)
+static bool rows_lds_takes(int64_t M, int64_t K) { return M <= 16 && K % (4 * kRowsSeg) == 0; }
+template <class T, bool GROUPED = false>
+static int launch_rows_lds(const GemmParams& p, int groups, hipStream_t stream) {
+    const dim3 grid(groups), block(4 * 64);
+    if (p.M <= 4) hipLaunchKernelGGL((gemm_rows_lds_kernel<T, 1, GROUPED>), grid, block, 0, stream, p);
+    else if (p.M <= 8) hipLaunchKernelGGL((gemm_rows_lds_kernel<T, 2, GROUPED>), grid, block, 0, stream, p);
+    else if (p.M <= 12) hipLaunchKernelGGL((gemm_rows_lds_kernel<T, 3, GROUPED>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_rows_lds_kernel<T, 4, GROUPED>), grid, block, 0, stream, p);
+    return check_launch("gemm_rows_lds_kernel");
+}
+
 // One row against an [N, K] weight (a decode step's projection): a wave streams whole weight rows as consecutive 16-byte
 // pieces (1 KiB per instruction, where the MFMA kernel above takes 128 bytes of each of 16 rows) and multiplies in the
 // vector ALU, which one activation row leaves mostly idle; one fp32 sum per lane, added up over the lanes at the end of
@@ -888,11 +989,12 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
         }
         return acc;
     };
-    if (p.M == 1 && p.K <= kGemvMaxKHalfs && n_sum <= 0x7fffffffLL) {   // one row: whole weight rows per wave, numbered through
+    if (p.M == 1 && (p.K <= kGemvSegHalfs || (p.K <= kGemvMaxKHalfs && !rows_lds_takes(p.M, p.K))) && n_sum <= 0x7fffffffLL) {   // one row: whole weight rows per wave, numbered through
         int acc = 0;
         for (int s = 0; s < kMaxGroup; ++s) { if (s < n_w) acc += p.grp.N[s]; p.grp.end[s] = acc; }
         return launch_gemv<T, true>(p, (int)n_sum, stream);
     }
+    if (rows_lds_takes(p.M, p.K)) return launch_rows_lds<T, true>(p, fill_ends(16), stream);
     if (p.M <= 32 || (p.M <= 64 && n_sum * p.K <= (INT64_C(1) << 25))) {
         const int nr = (p.M > 16 && n_sum >= 160 * 32) ? 2 : 1;
         const int groups = fill_ends(16 * nr);
@@ -1002,8 +1104,12 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     const int splits = fast && workspace && aligned16(workspace) ? gemm_splits(M, N, K) : 1;
     const bool can_split = splits > 1 && workspace_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
     // (with a workspace, K slices of the tiled kernel overtake it from 17 rows on: 32 rows against 4096 x 14336, 28 us against 52)
-    if (fast && nt && M == 1 && K <= kGemvMaxKHalfs)
+    // one row: whole weight rows per wave while a row is one segment (14336 x 4096: 19.1 us against 21.9 for the LDS-staged
+    // MFMA kernel below); longer rows go to that kernel when it takes them (4096 x 14336: 18.0 against 22.1)
+    if (fast && nt && M == 1 && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
         return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
+    if (fast && nt && rows_lds_takes(M, K))
+        return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
     if (fast && nt && (M <= 16 || (!can_split && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))))
         return dtype == MINFER_ATTN_F16 ? launch_skinny<F16>(p, stream) : launch_skinny<BF16>(p, stream);
     if (can_split) {

@@ -63,9 +63,17 @@ def make(M, N, K, layout, dtype, seed):
     (17, 4104, 64, 1.0, 1.0),        # one K step: seven of the eight waves have nothing to add
     (64, 6144, 4096, 2.0, 3.0),      # 64 rows, two column groups per workgroup: the few-row kernel's largest instantiation
     (40, 5128, 1024, 1.0, 1.0),      # 40 rows (three row blocks), two column groups, the last one ragged
+    # up to 16 rows against an [N, K] weight with K a multiple of 512: weight and activation rows copied to LDS along the rows
+    (2, 4096, 4096, 1.0, 0.0),
+    (5, 264, 512, 1.0, 1.0),         # one segment per wave; rows 5..7 of the second activation copy do not exist
+    (12, 1000, 1536, 2.0, 3.0),      # three activation copies, a last group of 8 columns
+    (16, 4104, 1024, 1.0, 1.0),
+    (3, 8, 512, 1.0, 0.0),           # a single half-empty group
+    (9, 2048, 14336, 0.5, 0.0),      # 28 segments per wave
     # one row against an [N, K] weight: whole weight rows per wave (segments of 4096 values)
     (1, 4096, 4096, 1.0, 0.0),       # one segment, the activations in registers; two rows per wave
     (1, 1000, 4160, 2.0, 3.0),       # a second segment of 64 values, the activations in LDS
+    (1, 1000, 8192, 2.0, 3.0),       # longer than a segment and a multiple of 512: the LDS-staged few-row kernel instead
     (1, 20000, 64, 2.0, 3.0),        # ten short rows per wave
     (1, 264, 16384, 1.0, 1.0),       # the longest activation row its LDS area holds
     (1, 264, 16448, 1.0, 0.0),       # longer: the 16-rows-per-instruction kernel
@@ -140,7 +148,9 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
     (300, 256, 200, 72, 136),          # ragged rows, widths that end inside a tile
     (1, 4096, 4096, 1024, 1024),       # a decode step: whole weight rows per wave, the three weights' rows numbered through
     (1, 8192, 1032, 8, 520),           # the same with the activations in LDS and runs of rows that cross from one weight to the next
-    (2, 4096, 4096, 1024, 1024),       # two rows: the few-row kernel over the three weights' column groups
+    (2, 4096, 4096, 1024, 1024),       # up to 16 rows, K a multiple of 512: the LDS-staged few-row kernel over the three weights' column groups
+    (13, 1024, 520, 264, 8),           # the same with ragged last groups
+    (16, 576, 4096, 1024, 1024),       # K not a multiple of 512: the few-row kernel that loads fragments directly
     (24, 1024, 5120, 1280, 1288),      # few rows, two column groups per workgroup, a ragged last group
     (64, 512, 768, 256, 256),          # few-row kernel at its largest row count
     (33, 50, 17, 17, 9),               # nothing tileable: three plain launches
