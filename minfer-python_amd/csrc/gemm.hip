@@ -507,6 +507,115 @@ static int launch_rows_lds(const GemmParams& p, int groups, hipStream_t stream) 
     return check_launch("gemm_rows_lds_kernel");
 }
 
+// Up to 64 rows against a wide [N, K] weight (a batch of decode steps against an FFN or output-head weight): a workgroup
+// of four waves owns a stripe of 64 columns over the whole of K, wave w its columns 16w .. 16w+15; K goes by in segments
+// of 256 values, the 16 weight rows of every wave and the activation rows (shared by the four waves) copied global -> LDS
+// with instructions whose lanes walk along the rows (512 consecutive bytes of each of two rows, 2 lines per quarter
+// wave); NST stages, NST - 1 segments in flight, one workgroup per compute unit (segments of 128 values and two
+// workgroups per unit are 15-25 % slower from 24 rows on).  No K slices, so no partial sums: the activations are read once per
+// stripe (N / 64 times in all) and the weight once.  Two rows of a copy share a 1 KiB block of LDS, blocks 32 bytes apart
+// in the banks: the 16 rows of a fragment read hit 16 different bank groups.  It needs N / 64 stripes to fill the chip.
+constexpr int kStripeSeg = 256;                                // K values per segment
+constexpr int kStripeBlock = 1024 + 32;                        // LDS bytes of two rows' segment, padded
+template <int MB> struct StripeGeom {
+    static constexpr int W_BYTES = 4 * 8 * kStripeBlock;       // 4 waves x 16 weight rows
+    static constexpr int X_BYTES = MB * 8 * kStripeBlock;      // 16 * MB activation rows
+    static constexpr int STAGE = W_BYTES + X_BYTES;
+    static constexpr int NST = MB >= 4 ? 2 : 3;                // 124 / 149 / 132 KiB: one workgroup per compute unit
+    static constexpr int COPIES = 8 + 2 * MB;                  // per wave and segment
+};
+template <class T, int MB>
+__global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p) {
+    using G = StripeGeom<MB>;
+    constexpr int NST = G::NST;
+    __shared__ __attribute__((aligned(16))) char lds[NST][G::STAGE];
+    const int lane = threadIdx.x & 63, w = wave_id();
+    const int l16 = lane & 15, quad = lane >> 4;
+    const int n0 = (int)blockIdx.x * 64 + 16 * w;              // this wave's first column
+    const int nseg = p.K / kStripeSeg;
+    // copy instruction: lane L takes piece L >> 1 (16 bytes) of row 2i + (L & 1)
+    const short* wsrc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+        wsrc[i] = (const short*)p.B + (int64_t)min(n0 + 2 * i + (lane & 1), p.N - 1) * p.ldb + 8 * (lane >> 1);
+    const short* xsrc[2 * MB];                                 // this wave's share of the activation rows: row pairs w, w + 4, ...
+#pragma unroll
+    for (int j = 0; j < 2 * MB; ++j)
+        xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * (lane >> 1);
+    auto issue = [&](int t) {
+        char* st = lds[t % NST];
+        const int k0 = t * kStripeSeg;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) copy16_global_to_lds(wsrc[i] + k0, st + (w * 8 + i) * kStripeBlock);
+#pragma unroll
+        for (int j = 0; j < 2 * MB; ++j) copy16_global_to_lds(xsrc[j] + k0, st + G::W_BYTES + (w + 4 * j) * kStripeBlock);
+    };
+    // fragment of k step s (32 values) for row r = l16 of a 16-row set: piece 4s + quad, inside the pair block of the row
+    const int frag = (l16 >> 1) * kStripeBlock + 16 * (l16 & 1) + 32 * quad;
+    f32x4 acc[MB];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < NST - 1; ++t)
+        if (t < nseg) issue(t);
+    for (int t = 0; t < nseg; ++t) {
+        __syncthreads();                                       // every wave has read segment t - 1: its stage may be refilled
+        if (t + NST - 1 < nseg) issue(t + NST - 1);
+        // segment t has landed once at most the copies of the segments after it are outstanding
+        const int after = min(NST - 1, nseg - 1 - t);
+        if (after >= 2) wait_vmcnt<2 * G::COPIES>(); else if (after == 1) wait_vmcnt<G::COPIES>(); else wait_vmcnt<0>();
+        __syncthreads();                                       // ... for every wave's copies (the activation rows are shared)
+        const char* wb = lds[t % NST] + w * 8 * kStripeBlock + frag;
+        const char* xb = lds[t % NST] + G::W_BYTES + frag;
+#pragma unroll
+        for (int s = 0; s < kStripeSeg / 32; ++s) {
+            const s16x8 a = *reinterpret_cast<const s16x8*>(wb + 128 * s);
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) {
+                const s16x8 b = *reinterpret_cast<const s16x8*>(xb + mb * 8 * kStripeBlock + 128 * s);
+                acc[mb] = T::mfma16(a, b, acc[mb]);
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // fragments in registers before the barrier that frees the stage
+    }
+    const int n = n0 + 4 * quad;                               // register r of a lane: weight row n + r, activation row 16mb + l16
+    if (n >= p.N) return;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = 16 * mb + l16;
+        if (m >= p.M) continue;
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[mb][e];
+        if (p.beta != 0.f) {
+            const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+        }
+        uint2 pk;
+        pk.x = T::pack2(v[0], v[1]);
+        pk.y = T::pack2(v[2], v[3]);
+        *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+    }
+}
+// It needs stripes enough to fill the chip (192 of 256 compute units at least).  Against a very wide weight (an output
+// head: 2004 stripes, eight rounds of one workgroup per compute unit) what each workgroup pays before its first segment
+// adds up, and up to eight rows the 16-column kernel, which keeps two workgroups on a unit, is faster (128256 x 4096:
+// 166-182 against 199 us); from 33 rows on it only equals K slices of the tiled kernel at some widths (28672 columns: 47
+// against 45 us) and beats them at others (14336: 24.9 against 28.8), so it takes those only without a workspace.
+static bool stripe_takes(int64_t M, int64_t N, int64_t K, bool can_split) {
+    const int64_t stripes = (N + 63) / 64;
+    return M >= 2 && M <= 64 && K % kStripeSeg == 0 && stripes >= 192 && (M >= 9 || stripes <= 640) && (M <= 32 || !can_split || stripes <= 256);
+}
+template <class T>
+static int launch_stripe(const GemmParams& p, hipStream_t stream) {
+    const dim3 grid((p.N + 63) / 64), block(4 * 64);
+    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1>), grid, block, 0, stream, p);
+    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_stripe_kernel<T, 4>), grid, block, 0, stream, p);
+    return check_launch("gemm_stripe_kernel");
+}
+
 // One row against an [N, K] weight (a decode step's projection): a wave streams whole weight rows as consecutive 16-byte
 // pieces (1 KiB per instruction, where the MFMA kernel above takes 128 bytes of each of 16 rows) and multiplies in the
 // vector ALU, which one activation row leaves mostly idle; one fp32 sum per lane, added up over the lanes at the end of
@@ -1108,6 +1217,8 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     // MFMA kernel below); longer rows go to that kernel when it takes them (4096 x 14336: 18.0 against 22.1)
     if (fast && nt && M == 1 && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
         return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
+    if (fast && nt && stripe_takes(M, N, K, can_split))
+        return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, stream) : launch_stripe<BF16>(p, stream);
     if (fast && nt && rows_lds_takes(M, K))
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
     if (fast && nt && (M <= 16 || (!can_split && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))))

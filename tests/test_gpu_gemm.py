@@ -70,6 +70,14 @@ def make(M, N, K, layout, dtype, seed):
     (16, 4104, 1024, 1.0, 1.0),
     (3, 8, 512, 1.0, 0.0),           # a single half-empty group
     (9, 2048, 14336, 0.5, 0.0),      # 28 segments per wave
+    # 2-64 rows against a weight of 12288 columns or more, K a multiple of 256: 64-column stripes over the whole of K
+    (2, 12288, 256, 1.0, 0.0),       # one segment
+    (9, 12296, 512, 2.0, 3.0),       # a last stripe of 8 columns; two segments (fewer than the three stages)
+    (16, 14336, 1024, 1.0, 1.0),
+    (17, 12288, 768, 1.0, 0.0),      # two blocks of activation rows, the second with one row
+    (32, 12352, 1280, 0.5, 1.0),
+    (33, 12288, 512, 1.0, 1.0),      # four blocks of activation rows, two stages
+    (64, 14336, 1792, 2.0, 0.0),
     # one row against an [N, K] weight: whole weight rows per wave (segments of 4096 values)
     (1, 4096, 4096, 1.0, 0.0),       # one segment, the activations in registers; two rows per wave
     (1, 1000, 4160, 2.0, 3.0),       # a second segment of 64 values, the activations in LDS
