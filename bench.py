@@ -42,6 +42,7 @@ QKV_TRAFFIC_BYTES = 378725 * 1024           # qkv in one launch, M=K=4096, N=409
 LONG_TRAFFIC_BYTES = 2721732 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
 RAGGED_TRAFFIC_BYTES = 748602 * 1024        # packed ragged prefill (T=20514, Hq=64)
 GEMM_Q8_TRAFFIC_BYTES = 61122 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
+GEMM_DECODE_TRAFFIC_BYTES = 120667 * 1024   # 64 tokens against the same weight in fp16, [N, K]
 # The kernel sources the counter runs were made against (first 12 hex digits of each file's sha1).  A row one of whose
 # sources has changed since carries "traffic_stale": true, so a constant that describes an earlier kernel says so.
 TRAFFIC_MEASURED_AGAINST = {
@@ -51,7 +52,7 @@ TRAFFIC_MEASURED_AGAINST = {
     "quant_q8.h": "4fea6a94e300",
     "rope.hip": "b4fd0618b44e",
     "rmsnorm.hip": "f6c4e575f461",
-    "gemm.hip": "2f047d3623c9",
+    "gemm.hip": "7fa033fc1c60",
 }
 TRAFFIC_ROW_SOURCES = {
     "": ("attn_common.h", "attn_prefill.hip"), "long_context": ("attn_common.h", "attn_prefill.hip"), "ragged": ("attn_common.h", "attn_prefill.hip"),
@@ -59,7 +60,7 @@ TRAFFIC_ROW_SOURCES = {
     "rope": ("attn_common.h", "rope.hip"), "rope_kv_append": ("attn_common.h", "rope.hip"),
     "rope_kv_append_q8_0": ("attn_common.h", "rope.hip", "quant_q8.h"), "rope_kv_append_norm": ("attn_common.h", "rope.hip"),
     "rmsnorm": ("attn_common.h", "rmsnorm.hip"), "gemm": ("attn_common.h", "gemm.hip"), "qkv": ("attn_common.h", "gemm.hip"),
-    "gemm_q8_0": ("attn_common.h", "gemm.hip", "quant_q8.h"),
+    "gemm_q8_0": ("attn_common.h", "gemm.hip", "quant_q8.h"), "gemm_decode": ("attn_common.h", "gemm.hip"),
 }
 
 
@@ -459,6 +460,19 @@ def main():
     q8_gbs = q8bytes / (q8_avg_ms * 1e-3) / 1e9
     del wq8, xa, xo
 
+    # the same projection for the decode batch of BASELINE configs[2]: 64 tokens against the fp16 weight as [N, K]
+    gwn = workloads.gemm_input(16, 14336, 4096, seed=3, device=dev)[1].t().contiguous()      # [14336, 4096]
+    gxa = workloads.gemm_input(64, 16, 4096, seed=5, device=dev)[0]                            # [1, 64, 4096]
+    gxo = torch.zeros(1, 64, 14336, dtype=torch.float16, device=dev)
+    gdstep = lambda: kerns.gemm(qt, qb, qs, 1.0, 0.0, gxa, gwn, gxo, gxo)
+    for _ in range(100):
+        gdstep()
+    torch.cuda.synchronize()
+    gd_avg_ms, gd_med_ms = ev.time_each(gdstep, stream, 50)
+    gdbytes = 14336 * 4096 * 2 + 64 * 4096 * 2 + 64 * 14336 * 2
+    gd_gbs = gdbytes / (gd_avg_ms * 1e-3) / 1e9
+    del gwn, gxa, gxo
+
     # ---- BASELINE configs[0] (the CPU-plumbing shape: B=1, Hq=8, Hkv=2, S=256, D=64) through the GPU op; its fp32
     # inputs are rounded to fp16, the op having no fp32 form.  Two launches of a few microseconds: launch-bound.
     cq, ck, cv, cmask = workloads.cpu_plumbing(seed=0)
@@ -547,6 +561,10 @@ def main():
                         "workload": "one token against a weight of Q8_0 blocks: x [1,1,4096] fp16, W uint8 [14336, 4352] (Llama-3-8B FFN up), out fp16",
                         "roofline": {"bound": "hbm", "achieved": q8_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": q8_gbs / PEAK_HBM_GBS,
                                      "traffic": GEMM_Q8_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemv_q8_kernel<activations in registers>", "algorithmic_bytes": q8bytes}}
+    rec["gemm_decode"] = {"value": gd_gbs, "unit": "GB/s", "ms": gd_avg_ms, "median_ms": gd_med_ms,
+                          "workload": "64 decode tokens against an fp16 weight stored [N, K]: x [1,64,4096], W [14336,4096] (Llama-3-8B FFN up), out fp16; weight-streaming, HBM-bound",
+                          "roofline": {"bound": "hbm", "achieved": gd_gbs, "peak": PEAK_HBM_GBS, "unit": "GB/s", "frac": gd_gbs / PEAK_HBM_GBS,
+                                       "traffic": GEMM_DECODE_TRAFFIC_BYTES, "traffic_source": TRAFFIC_SOURCE, "kernel": "gemm_stripe_kernel<F16,4>", "algorithmic_bytes": gdbytes}}
     rec["cpu_plumbing"] = {"value": cflops / (c_avg_ms * 1e-3) / 1e12, "unit": "TFLOP/s", "ms": c_avg_ms, "median_ms": c_med_ms,
                            "workload": "prefill B=1 Hq=8 Hkv=2 S=256 D=64 causal dense-mask, fp32 inputs rounded to fp16 for the GPU op (BASELINE configs[0]); launch-bound"}
     rec["calibration"] = {"mfma_only_f16_random": sus_f16, "mfma_only_bf16_random": sus_bf16,

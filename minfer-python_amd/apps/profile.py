@@ -203,6 +203,18 @@ def gemm(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+def gemm_decode(backend: str, which: str, workload: str, repeat: int):
+    """64 decode tokens against an fp16 weight stored [N, K]: x [1,64,4096], W [14336,4096] (Llama-3-8B FFN up)."""
+    kerns = KernelBackend(backend)
+    w = workloads.gemm_input(16, 14336, 4096, seed=3, device="cuda")[1].t().contiguous()
+    x = workloads.gemm_input(64, 16, 4096, seed=5, device="cuda")[0]
+    out = torch.zeros(1, 64, 14336, dtype=torch.float16, device="cuda")
+    fn = (lambda: kerns.gemm(QT, QB, QS, 1.0, 0.0, x, w, out, out)) if which == "minfer" else (lambda: torch.matmul(x, w.t(), out=out))
+    for _ in range(repeat):
+        fn()
+    torch.cuda.synchronize()
+
+
 def qkv(backend: str, which: str, workload: str, repeat: int):
     """The Llama-3-8B QKV projection of a 4096-token prefill: x [1,4096,4096], wq [4096,4096], wk and wv [1024,4096];
     `ref` is three separate gemm calls."""
@@ -273,7 +285,7 @@ def mfma_rate(backend: str, which: str, workload: str, repeat: int):
 if __name__ == "__main__":
     KERNELS = {"mfma_rate": mfma_rate, "gemm_q8_0": gemm_q8_0, "flash_attn": flash_attn, "flash_attn_decode": flash_attn_decode, "flash_attn_varlen": flash_attn_varlen,
                "flash_attn_decode_q8_0": flash_attn_decode_q8_0, "il_rope": il_rope, "rope_kv_append": rope_kv_append,
-               "rope_kv_append_q8_0": rope_kv_append_q8_0, "rope_kv_append_norm": rope_kv_append_norm, "qkv": qkv, "quant": quant, "rmsnorm": rmsnorm, "gemm": gemm, "copy": copy}
+               "rope_kv_append_q8_0": rope_kv_append_q8_0, "rope_kv_append_norm": rope_kv_append_norm, "qkv": qkv, "quant": quant, "rmsnorm": rmsnorm, "gemm": gemm, "gemm_decode": gemm_decode, "copy": copy}
     parser = argparse.ArgumentParser()
     parser.add_argument("--backend", choices=["torch_ext"], default="torch_ext")
     parser.add_argument("--kernel", choices=sorted(KERNELS), required=True)
