@@ -1022,7 +1022,11 @@ static int gemm_splits(int64_t M, int64_t N, int64_t K) {
     const int64_t tiles = ((M + GemmSmall::BM - 1) / GemmSmall::BM) * ((N + GemmSmall::BN - 1) / GemmSmall::BN);
     const int64_t kt = K / kBK;
     if (tiles >= 128 || kt < 8) return 1;
-    return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, kt / 4), 32));
+    int64_t s = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, kt / 4), 32));
+    // 64-127 tiles get two or three slices that way and fill the chip once; twice as many, while a slice stays 16 steps long,
+    // keep two workgroups on a compute unit ([K,N] 4096 x 14336 at 1-16 rows: 27.5 -> 22 us; 128 rows 37 -> 32)
+    if (tiles >= 64 && tiles * s <= 256 && kt / (2 * s) >= 16) s *= 2;
+    return (int)s;
 }
 
 template <class T, bool NT>
