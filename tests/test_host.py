@@ -183,7 +183,7 @@ def test_gemm_workspace_sizes():
     ws = L.minfer_gemm_workspace_bytes
     assert ws(64, 4096, 4096) == 8 * 64 * 4096 * 4            # 32 tiles of 128 x 128: 8 slices of 8 steps
     assert ws(256, 4096, 4096) == 4 * 256 * 4096 * 4          # 64 tiles: 4 slices
-    assert ws(100, 14336, 4096) == 2 * 100 * 14336 * 4
+    assert ws(100, 14336, 4096) == 4 * 100 * 14336 * 4        # 112 tiles: 2 slices fill the chip once, 4 of 16 steps each are taken
     assert ws(4096, 4096, 4096) == 0 and ws(64, 4096, 256) == 0 and ws(64, 4096, 100) == 0 and ws(64, 4100, 4096) == 0
     assert ws(0, 4096, 4096) == 0 and ws(-1, 4096, 4096) == 0 and ws(64, 4096, 1 << 40) == 0
 
