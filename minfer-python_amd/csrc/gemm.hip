@@ -508,85 +508,133 @@ static int launch_rows_lds(const GemmParams& p, int groups, hipStream_t stream) 
 }
 
 // Up to 64 rows against a wide [N, K] weight (a batch of decode steps against an FFN or output-head weight): a workgroup
-// of four waves owns a stripe of 64 columns over the whole of K, wave w its columns 16w .. 16w+15; K goes by in segments
-// of 256 values, the 16 weight rows of every wave and the activation rows (shared by the four waves) copied global -> LDS
-// with instructions whose lanes walk along the rows (512 consecutive bytes of each of two rows, 2 lines per quarter
-// wave); NST stages, NST - 1 segments in flight, one workgroup per compute unit (segments of 128 values and two
-// workgroups per unit are 15-25 % slower from 24 rows on).  No K slices, so no partial sums: the activations are read once per
-// stripe (N / 64 times in all) and the weight once.  Two rows of a copy share a 1 KiB block of LDS, blocks 32 bytes apart
-// in the banks: the 16 rows of a fragment read hit 16 different bank groups.  It needs N / 64 stripes to fill the chip.
+// of four waves owns a stripe of 64 columns over the whole of K; K goes by in segments of 256 values, the 64 weight rows
+// and the activation rows copied global -> LDS with instructions whose lanes walk along the rows (512 consecutive bytes
+// of each of two rows, 2 lines per quarter wave); three weight stages (two segments in flight) and two or three
+// activation stages, one workgroup per compute unit (segments of 128 values and two workgroups per unit are 15-25 %
+// slower from 24 rows on).  No K slices across workgroups, so no partial sums in memory: the activations are read once
+// per stripe (N / 64 times in all) and the weight once.  Two rows of a copy share a 1 KiB block of LDS; inside block i
+// the 16-byte pieces of a row sit at piece ^ (i & 7), so the 16 rows of a fragment read hit 16 different bank groups
+// without padding (160 KiB exactly at 49-64 rows).  It needs N / 64 stripes to fill the chip.
 constexpr int kStripeSeg = 256;                                // K values per segment
-constexpr int kStripeBlock = 1024 + 32;                        // LDS bytes of two rows' segment, padded
+constexpr int kStripeBlock = 1024;                             // LDS bytes of two rows' segment
 template <int MB> struct StripeGeom {
-    static constexpr int W_BYTES = 4 * 8 * kStripeBlock;       // 4 waves x 16 weight rows
+    static constexpr int W_BYTES = 4 * 8 * kStripeBlock;       // 64 weight rows
     static constexpr int X_BYTES = MB * 8 * kStripeBlock;      // 16 * MB activation rows
-    static constexpr int STAGE = W_BYTES + X_BYTES;
-    static constexpr int NST = MB >= 4 ? 2 : 3;                // 124 / 149 / 132 KiB: one workgroup per compute unit
-    static constexpr int COPIES = 8 + 2 * MB;                  // per wave and segment
+    static constexpr int WST = MB >= 4 ? 2 : 3, XST = MB >= 3 ? 2 : 3;   // 120 / 144 / 144 / 128 KiB
+    static constexpr int CW = 8, CX = 2 * MB;                  // copies per wave and segment
 };
-template <class T, int MB>
+// SLICED: p.splits workgroups per stripe, each over its share of the segments; they leave raw fp32 sums in p.part
+// ([slice][M][N]) for gemm_reduce_kernel.
+template <class T, int MB, bool SLICED = false>
 __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p) {
     using G = StripeGeom<MB>;
-    constexpr int NST = G::NST;
-    __shared__ __attribute__((aligned(16))) char lds[NST][G::STAGE];
+    constexpr int WST = G::WST, XST = G::XST;
+    __shared__ __attribute__((aligned(16))) char w_lds[WST][G::W_BYTES];
+    __shared__ __attribute__((aligned(16))) char x_lds[XST][G::X_BYTES];
     const int lane = threadIdx.x & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    const int n0 = (int)blockIdx.x * 64 + 16 * w;              // this wave's first column
-    const int nseg = p.K / kStripeSeg;
-    // copy instruction: lane L takes piece L >> 1 (16 bytes) of row 2i + (L & 1)
+    int stripe = (int)blockIdx.x, slice = 0, seg0 = 0, nseg = p.K / kStripeSeg;
+    if (SLICED) {
+        stripe = (int)blockIdx.x / p.splits; slice = (int)blockIdx.x % p.splits;
+        seg0 = slice * nseg / p.splits;
+        nseg = (slice + 1) * nseg / p.splits - seg0;
+    }
+    const int n0 = stripe * 64 + 16 * w;                       // the columns this wave copies and, at the end, writes
+    // copy instruction for row pair i: lane L lands at byte 16 L of the block and fetches piece (L >> 1) ^ (i & 7) of
+    // row 2i + (L & 1)
     const short* wsrc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-        wsrc[i] = (const short*)p.B + (int64_t)min(n0 + 2 * i + (lane & 1), p.N - 1) * p.ldb + 8 * (lane >> 1);
+        wsrc[i] = (const short*)p.B + (int64_t)min(n0 + 2 * i + (lane & 1), p.N - 1) * p.ldb + 8 * ((lane >> 1) ^ i);
     const short* xsrc[2 * MB];                                 // this wave's share of the activation rows: row pairs w, w + 4, ...
 #pragma unroll
     for (int j = 0; j < 2 * MB; ++j)
-        xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * (lane >> 1);
-    auto issue = [&](int t) {
-        char* st = lds[t % NST];
-        const int k0 = t * kStripeSeg;
+        xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * ((lane >> 1) ^ ((w + 4 * j) & 7));
+    // Stripe b starts at segment b mod nseg and wraps: the stripes running at one time then read different segments of
+    // the activation rows instead of the same few lines of the same few L2 channels
+    const int rot = (int)(blockIdx.x % (unsigned)nseg);
+    auto seg_k0 = [&](int t) { const int sg = t + rot; return (seg0 + (sg >= nseg ? sg - nseg : sg)) * kStripeSeg; };
+    auto issue_w = [&](int t) {
+        char* st = w_lds[t % WST];
+        const int k0 = seg_k0(t);
 #pragma unroll
         for (int i = 0; i < 8; ++i) copy16_global_to_lds(wsrc[i] + k0, st + (w * 8 + i) * kStripeBlock);
-#pragma unroll
-        for (int j = 0; j < 2 * MB; ++j) copy16_global_to_lds(xsrc[j] + k0, st + G::W_BYTES + (w + 4 * j) * kStripeBlock);
     };
-    // fragment of k step s (32 values) for row r = l16 of a 16-row set: piece 4s + quad, inside the pair block of the row
-    const int frag = (l16 >> 1) * kStripeBlock + 16 * (l16 & 1) + 32 * quad;
-    f32x4 acc[MB];
+    auto issue_x = [&](int t) {
+        char* st = x_lds[t % XST];
+        const int k0 = seg_k0(t);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) acc[mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < 2 * MB; ++j) copy16_global_to_lds(xsrc[j] + k0, st + (w + 4 * j) * kStripeBlock);
+    };
+    // Wave w multiplies k steps 2w and 2w + 1 of every segment for all 64 columns and all rows: every fragment is read
+    // from LDS once per workgroup (a wave that owned 16 columns over the whole segment would read all activation
+    // fragments, four times the traffic), and the four partial sums meet in LDS after the last segment.  Fragment of k
+    // step s for row r = l16 of a 16-row set: piece 4s + quad of the row, in pair block r >> 1.
+    const int row_off = (l16 >> 1) * kStripeBlock + 16 * (l16 & 1);
+    int frag[2];
 #pragma unroll
-    for (int t = 0; t < NST - 1; ++t)
-        if (t < nseg) issue(t);
+    for (int s = 0; s < 2; ++s) frag[s] = row_off + 32 * ((4 * (2 * w + s) + quad) ^ (l16 >> 1));
+    f32x4 acc[4][MB];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[c][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < WST - 1; ++t) {
+        if (t < XST - 1 && t < nseg) issue_x(t);
+        if (t < nseg) issue_w(t);
+    }
     for (int t = 0; t < nseg; ++t) {
-        __syncthreads();                                       // every wave has read segment t - 1: its stage may be refilled
-        if (t + NST - 1 < nseg) issue(t + NST - 1);
-        // segment t has landed once at most the copies of the segments after it are outstanding
-        const int after = min(NST - 1, nseg - 1 - t);
-        if (after >= 2) wait_vmcnt<2 * G::COPIES>(); else if (after == 1) wait_vmcnt<G::COPIES>(); else wait_vmcnt<0>();
-        __syncthreads();                                       // ... for every wave's copies (the activation rows are shared)
-        const char* wb = lds[t % NST] + w * 8 * kStripeBlock + frag;
-        const char* xb = lds[t % NST] + G::W_BYTES + frag;
+        __syncthreads();                                       // every wave has read segment t - 1: its stages may be refilled
+        if (t + XST - 1 < nseg) issue_x(t + XST - 1);
+        if (t + WST - 1 < nseg) issue_w(t + WST - 1);
+        // segment t has landed once at most the copies issued after it are outstanding: the weight of the next two
+        // segments and the activations of the next XST - 1
+        const int after = nseg - 1 - t;
+        if (after >= 2) wait_vmcnt<(WST - 1) * G::CW + (XST - 1) * G::CX>(); else if (after == 1) wait_vmcnt<G::CW + G::CX>(); else wait_vmcnt<0>();
+        __syncthreads();                                       // ... for every wave's copies
+        const char* wb = w_lds[t % WST];
+        const char* xb = x_lds[t % XST];
 #pragma unroll
-        for (int s = 0; s < kStripeSeg / 32; ++s) {
-            const s16x8 a = *reinterpret_cast<const s16x8*>(wb + 128 * s);
+        for (int s = 0; s < 2; ++s) {
+            s16x8 b[MB];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) {
-                const s16x8 b = *reinterpret_cast<const s16x8*>(xb + mb * 8 * kStripeBlock + 128 * s);
-                acc[mb] = T::mfma16(a, b, acc[mb]);
+            for (int mb = 0; mb < MB; ++mb) b[mb] = *reinterpret_cast<const s16x8*>(xb + mb * 8 * kStripeBlock + frag[s]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const s16x8 a = *reinterpret_cast<const s16x8*>(wb + c * 8 * kStripeBlock + frag[s]);
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) acc[c][mb] = T::mfma16(a, b[mb], acc[c][mb]);
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // fragments in registers before the barrier that frees the stage
     }
+    // partial sums of the four waves: wave u leaves column block c at red[u][c][mb][lane]; wave w adds up column block w
+    // in the order of the waves
+    __syncthreads();
+    f32x4* red = reinterpret_cast<f32x4*>(&w_lds[0][0]);   // 16 MB KiB of the 96
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red[((w * 4 + c) * MB + mb) * 64 + lane] = acc[c][mb];
+    __syncthreads();
     const int n = n0 + 4 * quad;                               // register r of a lane: weight row n + r, activation row 16mb + l16
     if (n >= p.N) return;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const int m = 16 * mb + l16;
         if (m >= p.M) continue;
+        f32x4 sum = red[((0 * 4 + w) * MB + mb) * 64 + lane];
+#pragma unroll
+        for (int u = 1; u < 4; ++u) sum += red[((u * 4 + w) * MB + mb) * 64 + lane];
+        if (SLICED) {
+            *reinterpret_cast<f32x4*>(p.part + ((int64_t)slice * p.M + m) * p.N + n) = sum;
+            continue;
+        }
         float v[4];
 #pragma unroll
-        for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[mb][e];
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
         if (p.beta != 0.f) {
             const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
 #pragma unroll
@@ -598,22 +646,31 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
     }
 }
-// It needs stripes enough to fill the chip (192 of 256 compute units at least).  Against a very wide weight (an output
+// It needs stripes enough to fill the chip (192 of 256 compute units at least), and then takes one row too (14336 x 4096:
+// 18.0 us against 19.6 for whole rows per wave, 12288 x 8192: 29.5 against 39).  Against a very wide weight (an output
 // head: 2004 stripes, eight rounds of one workgroup per compute unit) what each workgroup pays before its first segment
-// adds up, and up to eight rows the 16-column kernel, which keeps two workgroups on a unit, is faster (128256 x 4096:
-// 166-182 against 199 us); from 33 rows on it only equals K slices of the tiled kernel at some widths (28672 columns: 47
-// against 45 us) and beats them at others (14336: 24.9 against 28.8), so it takes those only without a workspace.
-static bool stripe_takes(int64_t M, int64_t N, int64_t K, bool can_split) {
+// adds up, and up to eight rows the kernels that keep more workgroups on a unit are faster (128256 x 4096: 157-181
+// against 185 us).  Where K slices of the tiled kernel are possible (fewer than 128 of its tiles: under 256 stripes) the
+// stripes win at every row count up to 64 (14336 columns, 64 rows: 24 against 28.8 us).
+static bool stripe_takes(int64_t M, int64_t N, int64_t K) {
     const int64_t stripes = (N + 63) / 64;
-    return M >= 2 && M <= 64 && K % kStripeSeg == 0 && stripes >= 192 && (M >= 9 || stripes <= 640) && (M <= 32 || !can_split || stripes <= 256);
+    return M >= 1 && M <= 64 && K % kStripeSeg == 0 && stripes >= 192 && (M >= 9 || stripes <= 640);
 }
-template <class T>
+template <class T, bool SLICED = false>
 static int launch_stripe(const GemmParams& p, hipStream_t stream) {
-    const dim3 grid((p.N + 63) / 64), block(4 * 64);
-    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1>), grid, block, 0, stream, p);
-    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((gemm_stripe_kernel<T, 4>), grid, block, 0, stream, p);
+    const dim3 grid((p.N + 63) / 64 * (SLICED ? p.splits : 1)), block(4 * 64);
+    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1, SLICED>), grid, block, 0, stream, p);
+    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2, SLICED>), grid, block, 0, stream, p);
+    else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_kernel<T, 3, SLICED>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_stripe_kernel<T, 4, SLICED>), grid, block, 0, stream, p);
     return check_launch("gemm_stripe_kernel");
+}
+// A weight of fewer than 192 stripes: with a workspace, K slices bring the workgroups up to the chip's 256 compute units
+// (every slice four segments at least); the slices' sums are added up by gemm_reduce_kernel.  1 = no slices.
+static int stripe_slices(int64_t M, int64_t N, int64_t K) {
+    const int64_t stripes = (N + 63) / 64;
+    if (M < 1 || M > 64 || K % kStripeSeg != 0 || N % 8 != 0 || stripes >= 192) return 1;
+    return (int)std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / stripes, K / kStripeSeg / 4), 16));
 }
 
 // One row against an [N, K] weight (a decode step's projection): a wave streams whole weight rows as consecutive 16-byte
@@ -1029,6 +1086,14 @@ static int gemm_splits(int64_t M, int64_t N, int64_t K) {
     return (int)s;
 }
 
+template <class T>
+static int launch_stripe_slices(GemmParams& p, hipStream_t stream) {
+    if (int rc = launch_stripe<T, true>(p, stream)) return rc;
+    const int grid = (int)std::min<int64_t>(((int64_t)p.M * (p.N / 4) + 255) / 256, 256 * 8);
+    hipLaunchKernelGGL((gemm_reduce_kernel<T>), dim3(grid), dim3(256), 0, stream, p);
+    return check_launch("gemm_reduce_kernel");
+}
+
 template <class T, bool NT>
 static int launch_split(GemmParams& p, hipStream_t stream) {
     using SH = GemmSmall;
@@ -1217,11 +1282,22 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     const int splits = fast && workspace && aligned16(workspace) ? gemm_splits(M, N, K) : 1;
     const bool can_split = splits > 1 && workspace_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
     // (with a workspace, K slices of the tiled kernel overtake it from 17 rows on: 32 rows against 4096 x 14336, 28 us against 52)
-    // one row: whole weight rows per wave while a row is one segment (14336 x 4096: 19.1 us against 21.9 for the LDS-staged
-    // MFMA kernel below); longer rows go to that kernel when it takes them (4096 x 14336: 18.0 against 22.1)
-    if (fast && nt && M == 1 && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
+    // a weight too narrow for one stripe per compute unit, with a workspace: K slices of the stripes.  Two launches, so
+    // not for the smallest weights; the 16-column kernels below, which read the activations once per 16 columns, keep up
+    // to 7 rows (4096 x 14336: 18 us against 21; 8 rows 21.5 against 20.9, 16 rows 27 against 21, 64 rows 28.6 against
+    // 23.6) unless their workgroups come to two per compute unit or more (8192 x 8192 at 1-16 rows: 28-33 against 25-26)
+    const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
+    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) &&
+        ((M >= 17 && N * K >= (INT64_C(1) << 24)) || (M >= 8 && N * K >= INT64_C(25000000)) || N >= 8192)) {
+        p.splits = slices; p.part = (float*)workspace;
+        return dtype == MINFER_ATTN_F16 ? launch_stripe_slices<F16>(p, stream) : launch_stripe_slices<BF16>(p, stream);
+    }
+    // one row against a weight too narrow or too wide for the stripes: whole weight rows per wave while a row is one
+    // segment (6144 x 4096: 11.7 us against 14.5 for the LDS-staged MFMA kernel below; 128256 x 4096: 157 against 185 for
+    // the stripes); longer rows go to that kernel when it takes them (4096 x 14336: 18.0 against 22.1)
+    if (fast && nt && M == 1 && !stripe_takes(M, N, K) && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
         return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
-    if (fast && nt && stripe_takes(M, N, K, can_split))
+    if (fast && nt && stripe_takes(M, N, K))
         return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, stream) : launch_stripe<BF16>(p, stream);
     if (fast && nt && rows_lds_takes(M, K))
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
@@ -1244,7 +1320,7 @@ MINFER_ATTN_EXPORT int minfer_gemm(int dtype, int b_layout, const void* A, const
 
 MINFER_ATTN_EXPORT size_t minfer_gemm_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
-    const int splits = gemm_splits(M, N, K);
+    const int splits = std::max(gemm_splits(M, N, K), stripe_slices(M, N, K));
     return splits > 1 ? (size_t)splits * (size_t)M * (size_t)N * sizeof(float) : 0;
 }
 

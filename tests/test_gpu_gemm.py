@@ -70,8 +70,9 @@ def make(M, N, K, layout, dtype, seed):
     (16, 4104, 1024, 1.0, 1.0),
     (3, 8, 512, 1.0, 0.0),           # a single half-empty group
     (9, 2048, 14336, 0.5, 0.0),      # 28 segments per wave
-    # 2-64 rows against a weight of 12288 columns or more, K a multiple of 256: 64-column stripes over the whole of K
+    # 1-64 rows against a weight of 12288 columns or more, K a multiple of 256: 64-column stripes over the whole of K
     (2, 12288, 256, 1.0, 0.0),       # one segment
+    (1, 12296, 1024, 2.0, 3.0),      # one row
     (9, 12296, 512, 2.0, 3.0),       # a last stripe of 8 columns; two segments (fewer than the three stages)
     (16, 14336, 1024, 1.0, 1.0),
     (17, 12288, 768, 1.0, 0.0),      # two blocks of activation rows, the second with one row
@@ -230,6 +231,12 @@ def test_qkv_op_and_reference_checks(kerns):
     (40, 512, 1984, 1.0, 0.0),       # K steps (31) not a multiple of the slice count
     (1, 4096, 4096, 1.0, 1.0),       # one row: with [K, N] the sliced tiles, with [N, K] still the few-row kernel
     (24, 1024, 2048, 1.0, 1.0),      # 17-32 rows: with a workspace the sliced tiles for both layouts
+    # [N, K] weights of fewer than 192 stripes of 64 columns: K slices of the stripe kernel
+    (8, 5120, 5120, 2.0, 3.0),       # 80 stripes, three slices of 6, 7 and 7 segments
+    (16, 4104, 8192, 1.0, 1.0),      # a last stripe of 8 columns
+    (33, 8192, 2048, 0.5, 0.0),      # three blocks of activation rows, two slices of four segments
+    (1, 8192, 4096, 1.0, 0.0),       # one row
+    (64, 6144, 4096, 1.0, 1.0),
 ])
 def test_gemm_k_slices_against_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, seed=M + N + K)
@@ -243,7 +250,7 @@ def test_gemm_k_slices_against_oracle(layout, dtype, M, N, K, alpha, beta):
     assert_close(d, exact, dtype, "k slices")
     # a workspace that is too small, or none, is the plain call
     d2 = torch.zeros_like(d)
-    assert capi.gemm_ws(da, db, dc, d2, alpha, beta, ws[: need // 2], layout) == capi.OK, capi.last_error()
+    assert capi.gemm_ws(da, db, dc, d2, alpha, beta, ws[: 4 * M * N], layout) == capi.OK, capi.last_error()   # room for one slice: no path takes it
     d3 = torch.zeros_like(d)
     assert capi.gemm(da, db, dc, d3, alpha, beta, layout) == capi.OK, capi.last_error()
     assert torch.equal(d2, d3)
