@@ -203,12 +203,16 @@ def gemm(backend: str, which: str, workload: str, repeat: int):
     torch.cuda.synchronize()
 
 
+DECODE_TOKENS = 64   # --tokens
+
+
 def gemm_decode(backend: str, which: str, workload: str, repeat: int):
-    """64 decode tokens against an fp16 weight stored [N, K]: x [1,64,4096], W [14336,4096] (Llama-3-8B FFN up)."""
+    """A batch of decode tokens (64 unless --tokens says otherwise) against an fp16 weight stored [N, K]:
+    x [1,tokens,4096], W [14336,4096] (Llama-3-8B FFN up)."""
     kerns = KernelBackend(backend)
     w = workloads.gemm_input(16, 14336, 4096, seed=3, device="cuda")[1].t().contiguous()
-    x = workloads.gemm_input(64, 16, 4096, seed=5, device="cuda")[0]
-    out = torch.zeros(1, 64, 14336, dtype=torch.float16, device="cuda")
+    x = workloads.gemm_input(DECODE_TOKENS, 16, 4096, seed=5, device="cuda")[0]
+    out = torch.zeros(1, DECODE_TOKENS, 14336, dtype=torch.float16, device="cuda")
     fn = (lambda: kerns.gemm(QT, QB, QS, 1.0, 0.0, x, w, out, out)) if which == "minfer" else (lambda: torch.matmul(x, w.t(), out=out))
     for _ in range(repeat):
         fn()
@@ -292,5 +296,7 @@ if __name__ == "__main__":
     parser.add_argument("--which", choices=["minfer", "ref"], required=True)
     parser.add_argument("--workload", choices=["llama8b", "reference", "long"], default="llama8b")
     parser.add_argument("--repeat", type=int, default=1)
+    parser.add_argument("--tokens", type=int, default=64, help="gemm_decode: rows of the activation matrix (1-64 take the stripe kernel)")
     args = parser.parse_args()
+    DECODE_TOKENS = args.tokens
     KERNELS[args.kernel](args.backend, args.which, args.workload, args.repeat)
