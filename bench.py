@@ -324,7 +324,8 @@ def main():
     for _ in range(max(args.warmup, 100)):
         dstep()
     torch.cuda.synchronize()
-    d_avg_ms, d_med_ms = ev.time_each(dstep, stream, min(max(args.steps, 20), 100))
+    _, d_med_ms = ev.time_each(dstep, stream, min(max(args.steps, 20), 100))
+    d_avg_ms = ev.time_region(dstep, stream, min(max(args.steps, 20), 100))
     dbytes = workloads.decode_bytes(ctx.tolist(), 32, 8, 128)
     d_gbs = dbytes / (d_avg_ms * 1e-3) / 1e9
     # the same decode over Q8_0 caches (34 bytes per 32 values), quantised on the device from the fp16 caches
@@ -336,7 +337,8 @@ def main():
     for _ in range(max(args.warmup, 100)):
         d8step()
     torch.cuda.synchronize()
-    d8_avg_ms, d8_med_ms = ev.time_each(d8step, stream, min(max(args.steps, 20), 100))
+    _, d8_med_ms = ev.time_each(d8step, stream, min(max(args.steps, 20), 100))
+    d8_avg_ms = ev.time_region(d8step, stream, min(max(args.steps, 20), 100))
     d8bytes = workloads.decode_bytes_q8_0(ctx.tolist(), 32, 8, 128)
     d8_gbs = d8bytes / (d8_avg_ms * 1e-3) / 1e9
     del kq8, vq8
@@ -350,7 +352,8 @@ def main():
     for _ in range(5):
         lstep()
     torch.cuda.synchronize()
-    l_avg_ms, l_med_ms = ev.time_each(lstep, stream, 10)
+    _, l_med_ms = ev.time_each(lstep, stream, 10)
+    l_avg_ms = ev.time_region(lstep, stream, 10)
     lflops = workloads.prefill_flops(32, 128, [lq.shape[2]])
     l_tf = lflops / (l_avg_ms * 1e-3) / 1e12
     del lq, lk, lv, lmask, lout
@@ -361,7 +364,8 @@ def main():
     for _ in range(50):
         vstep()
     torch.cuda.synchronize()
-    v_avg_ms, v_med_ms = ev.time_each(vstep, stream, 50)
+    _, v_med_ms = ev.time_each(vstep, stream, 50)
+    v_avg_ms = ev.time_region(vstep, stream, 50)
     vflops = workloads.prefill_flops(64, 128, vlens)
     v_tf = vflops / (v_avg_ms * 1e-3) / 1e12
     del vq, vk, vv, vout
@@ -372,7 +376,8 @@ def main():
     for _ in range(200):
         rstep()
     torch.cuda.synchronize()
-    r_avg_ms, r_med_ms = ev.time_each(rstep, stream, 50)
+    _, r_med_ms = ev.time_each(rstep, stream, 50)
+    r_avg_ms = ev.time_region(rstep, stream, 50)
     rbytes = workloads.rope_bytes(8, 4096, 48, 64)
     r_gbs = rbytes / (r_avg_ms * 1e-3) / 1e9
     del x
@@ -381,7 +386,8 @@ def main():
     for _ in range(100):
         astep()
     torch.cuda.synchronize()
-    a_avg_ms, a_med_ms = ev.time_each(astep, stream, 50)
+    _, a_med_ms = ev.time_each(astep, stream, 50)
+    a_avg_ms = ev.time_region(astep, stream, 50)
     abytes = workloads.kv_append_bytes(8, 4096, 32, 8, 128, 128)
     a_gbs = abytes / (a_avg_ms * 1e-3) / 1e9
     # the same producer with the per-head q/k RMSNorm (Qwen3/Gemma3-style) applied first, in the same launch
@@ -391,7 +397,8 @@ def main():
     for _ in range(100):
         anstep()
     torch.cuda.synchronize()
-    an_avg_ms, an_med_ms = ev.time_each(anstep, stream, 50)
+    _, an_med_ms = ev.time_each(anstep, stream, 50)
+    an_avg_ms = ev.time_region(anstep, stream, 50)
     an_gbs = abytes / (an_avg_ms * 1e-3) / 1e9
     del akc, avc
     akq = torch.zeros(8, 8, 4096, 128 // 32 * 34, dtype=torch.uint8, device=dev)
@@ -400,7 +407,8 @@ def main():
     for _ in range(100):
         a8step()
     torch.cuda.synchronize()
-    a8_avg_ms, a8_med_ms = ev.time_each(a8step, stream, 50)
+    _, a8_med_ms = ev.time_each(a8step, stream, 50)
+    a8_avg_ms = ev.time_region(a8step, stream, 50)
     a8bytes = workloads.kv_append_bytes_q8_0(8, 4096, 32, 8, 128, 128)
     a8_gbs = a8bytes / (a8_avg_ms * 1e-3) / 1e9
     del aq, ak, av, akq, avq
@@ -411,7 +419,8 @@ def main():
     for _ in range(100):
         nstep()
     torch.cuda.synchronize()
-    n_avg_ms, n_med_ms = ev.time_each(nstep, stream, 50)
+    _, n_med_ms = ev.time_each(nstep, stream, 50)
+    n_avg_ms = ev.time_region(nstep, stream, 50)
     nbytes = workloads.rmsnorm_bytes(nshape)
     n_gbs = nbytes / (n_avg_ms * 1e-3) / 1e9
     del nx, nout
@@ -422,7 +431,8 @@ def main():
     for _ in range(100):
         gstep()
     torch.cuda.synchronize()
-    g_avg_ms, g_med_ms = ev.time_each(gstep, stream, 50)
+    _, g_med_ms = ev.time_each(gstep, stream, 50)
+    g_avg_ms = ev.time_region(gstep, stream, 50)
     gflops = workloads.gemm_flops(4096, 4096, 4096)
     g_tf = gflops / (g_avg_ms * 1e-3) / 1e12
     del ga, gw, gbias, gout
@@ -438,7 +448,8 @@ def main():
     for _ in range(100):
         pstep()
     torch.cuda.synchronize()
-    p_avg_ms, p_med_ms = ev.time_each(pstep, stream, 50)
+    _, p_med_ms = ev.time_each(pstep, stream, 50)
+    p_avg_ms = ev.time_region(pstep, stream, 50)
     pflops = workloads.gemm_flops(4096, 6144, 4096)
     p_tf = pflops / (p_avg_ms * 1e-3) / 1e12
     del px, pwq, pwk, pwv, pq, pk, pv
@@ -455,7 +466,8 @@ def main():
     for _ in range(100):
         q8step()
     torch.cuda.synchronize()
-    q8_avg_ms, q8_med_ms = ev.time_each(q8step, stream, 50)
+    _, q8_med_ms = ev.time_each(q8step, stream, 50)
+    q8_avg_ms = ev.time_region(q8step, stream, 200)
     q8bytes = 14336 * (4096 // 32 * 34) + 4096 * 2 + 14336 * 2
     q8_gbs = q8bytes / (q8_avg_ms * 1e-3) / 1e9
     del wq8, xa, xo
@@ -468,7 +480,8 @@ def main():
     for _ in range(100):
         gdstep()
     torch.cuda.synchronize()
-    gd_avg_ms, gd_med_ms = ev.time_each(gdstep, stream, 50)
+    _, gd_med_ms = ev.time_each(gdstep, stream, 50)
+    gd_avg_ms = ev.time_region(gdstep, stream, 200)
     gdbytes = 14336 * 4096 * 2 + 64 * 4096 * 2 + 64 * 14336 * 2
     gd_gbs = gdbytes / (gd_avg_ms * 1e-3) / 1e9
     del gwn, gxa, gxo
@@ -482,7 +495,8 @@ def main():
     for _ in range(50):
         cstep()
     torch.cuda.synchronize()
-    c_avg_ms, c_med_ms = ev.time_each(cstep, stream, 50)
+    _, c_med_ms = ev.time_each(cstep, stream, 50)
+    c_avg_ms = ev.time_region(cstep, stream, 50)
     cflops = workloads.prefill_flops(8, 64, [256])
 
     # ---- calibration: what the chip sustains on the matrix instruction alone, on operand values of the benchmarks'
@@ -510,6 +524,8 @@ def main():
         "ms_per_step": wall_ms, "event_ms_per_step": region_ms, "event_steps": event_steps,
         "prewarm_ms": prewarm_ms, "prewarm_calls": prewarm_calls, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "f16", "data": "synthetic", "launch": "hipgraph replay of one op call" if args.graph else "eager",
+        "ms_is": "every row's ms: back-to-back calls between ONE pair of HIP events on the op's stream, divided by the calls (a pair around "
+                 "every call adds 2-3 us, a tenth of the shortest kernels here); median_ms: a pair around every call",
         "config": {"workload": "prefill B=1 Hq=32 Hkv=8 S=4096 D=128 fp16 causal dense-mask (BASELINE configs[1])",
                    "global_batch": 1, "seq_len": L, "parallelism": "single-gpu"},
         "roofline": mfma_roofline(achieved, sus_f16, mix_f16, traffic=PREFILL_TRAFFIC_BYTES, traffic_source=TRAFFIC_SOURCE,
