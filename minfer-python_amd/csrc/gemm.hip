@@ -526,8 +526,10 @@ template <int MB> struct StripeGeom {
 };
 // SLICED: p.splits workgroups per stripe, each over its share of the segments; they leave raw fp32 sums in p.part
 // ([slice][M][N]) for gemm_reduce_kernel.
-template <class T, int MB, bool SLICED = false>
+// GROUPED: the stripes of up to three weights numbered through (p.grp.end in stripes), alpha = 1 and no C.
+template <class T, int MB, bool SLICED = false, bool GROUPED = false>
 __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p) {
+    static_assert(!(SLICED && GROUPED), "the grouped launch has no workspace");
     using G = StripeGeom<MB>;
     constexpr int WST = G::WST, XST = G::XST;
     __shared__ __attribute__((aligned(16))) char w_lds[WST][G::W_BYTES];
@@ -540,20 +542,34 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         seg0 = slice * nseg / p.splits;
         nseg = (slice + 1) * nseg / p.splits - seg0;
     }
+    const short* Bg = (const short*)p.B;
+    short* Dg = (short*)p.D;
+    int N = p.N;
+    int64_t ldb = p.ldb, ldd = p.ldd;
+    if (GROUPED) {   // the stripe's weight, output and place inside them (uniform)
+        int local;
+        const int sg = group_of_unit(p.grp, stripe, local);
+        stripe = local;
+        Bg = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]);
+        Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
+        N = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
+        ldb = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
+        ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
+    }
     const int n0 = stripe * 64 + 16 * w;                       // the columns this wave copies and, at the end, writes
     // copy instruction for row pair i: lane L lands at byte 16 L of the block and fetches piece (L >> 1) ^ (i & 7) of
     // row 2i + (L & 1)
     const short* wsrc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i)
-        wsrc[i] = (const short*)p.B + (int64_t)min(n0 + 2 * i + (lane & 1), p.N - 1) * p.ldb + 8 * ((lane >> 1) ^ i);
+        wsrc[i] = Bg + (int64_t)min(n0 + 2 * i + (lane & 1), N - 1) * ldb + 8 * ((lane >> 1) ^ i);
     const short* xsrc[2 * MB];                                 // this wave's share of the activation rows: row pairs w, w + 4, ...
 #pragma unroll
     for (int j = 0; j < 2 * MB; ++j)
         xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * ((lane >> 1) ^ ((w + 4 * j) & 7));
     // Stripe b starts at segment b mod nseg and wraps: the stripes running at one time then read different segments of
     // the activation rows instead of the same few lines of the same few L2 channels
-    const int rot = (int)(blockIdx.x % (unsigned)nseg);
+    const int rot = (int)((SLICED ? blockIdx.x : (unsigned)stripe) % (unsigned)nseg);   // (a stripe's place in its own weight: the grouped launch adds it up as the plain one does)
     auto seg_k0 = [&](int t) { const int sg = t + rot; return (seg0 + (sg >= nseg ? sg - nseg : sg)) * kStripeSeg; };
     auto issue_w = [&](int t) {
         char* st = w_lds[t % WST];
@@ -620,7 +636,7 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         for (int mb = 0; mb < MB; ++mb) red[((w * 4 + c) * MB + mb) * 64 + lane] = acc[c][mb];
     __syncthreads();
     const int n = n0 + 4 * quad;                               // register r of a lane: weight row n + r, activation row 16mb + l16
-    if (n >= p.N) return;
+    if (n >= N) return;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const int m = 16 * mb + l16;
@@ -635,7 +651,7 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
-        if (p.beta != 0.f) {
+        if (!GROUPED && p.beta != 0.f) {
             const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
 #pragma unroll
             for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
@@ -643,26 +659,29 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         uint2 pk;
         pk.x = T::pack2(v[0], v[1]);
         pk.y = T::pack2(v[2], v[3]);
-        *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+        *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
     }
 }
-// It needs stripes enough to fill the chip (192 of 256 compute units at least), and then takes one row too (14336 x 4096:
-// 18.0 us against 19.6 for whole rows per wave, 12288 x 8192: 29.5 against 39).  Against a very wide weight (an output
-// head: 2004 stripes, eight rounds of one workgroup per compute unit) what each workgroup pays before its first segment
-// adds up, and up to eight rows the kernels that keep more workgroups on a unit are faster (128256 x 4096: 157-181
-// against 185 us).  Where K slices of the tiled kernel are possible (fewer than 128 of its tiles: under 256 stripes) the
-// stripes win at every row count up to 64 (14336 columns, 64 rows: 24 against 28.8 us).
-static bool stripe_takes(int64_t M, int64_t N, int64_t K) {
-    const int64_t stripes = (N + 63) / 64;
-    return M >= 1 && M <= 64 && K % kStripeSeg == 0 && stripes >= 192 && (M >= 9 || stripes <= 640);
+// It needs stripes enough to keep the memory busy, which is fewer than there are compute units: 128 workgroups stream an
+// 8192 x 8192 weight at 6.5 TB/s (20.6 us at 1-8 rows, where the 16-column kernels take 28-31), 96 a 6144 x 4096 one in
+// 10.8-13.4 us at 1-32 rows (11.5-20.1).  From 96 stripes on it takes every row count up to 64, one row too (14336 x 4096:
+// 18.0 us against 19.6 for whole rows per wave, 12288 x 8192: 29.5 against 39); 80 stripes from 8 rows on (5120 x 5120:
+// 13.6 against 15.4, one row 13.3 against 12.4), 64 from 32 rows on (4096 x 4096: 13.2 against 15.6).  Against a very wide
+// weight (an output head: 2004 stripes, eight rounds of one workgroup per compute unit) what each workgroup pays before
+// its first segment adds up, and up to eight rows the kernels that keep more workgroups on a unit are faster (128256 x
+// 4096: 157-181 against 185 us).
+static bool stripe_takes(int64_t M, int64_t stripes, int64_t K) {
+    if (M < 1 || M > 64 || K % kStripeSeg != 0) return false;
+    if (stripes > 640) return M >= 9;
+    return stripes >= 96 || (stripes >= 80 && M >= 8) || (stripes >= 64 && M >= 32);
 }
-template <class T, bool SLICED = false>
-static int launch_stripe(const GemmParams& p, hipStream_t stream) {
-    const dim3 grid((p.N + 63) / 64 * (SLICED ? p.splits : 1)), block(4 * 64);
-    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1, SLICED>), grid, block, 0, stream, p);
-    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2, SLICED>), grid, block, 0, stream, p);
-    else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_kernel<T, 3, SLICED>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((gemm_stripe_kernel<T, 4, SLICED>), grid, block, 0, stream, p);
+template <class T, bool SLICED = false, bool GROUPED = false>
+static int launch_stripe(const GemmParams& p, int stripes, hipStream_t stream) {
+    const dim3 grid(stripes * (SLICED ? p.splits : 1)), block(4 * 64);
+    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1, SLICED, GROUPED>), grid, block, 0, stream, p);
+    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2, SLICED, GROUPED>), grid, block, 0, stream, p);
+    else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_kernel<T, 3, SLICED, GROUPED>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_stripe_kernel<T, 4, SLICED, GROUPED>), grid, block, 0, stream, p);
     return check_launch("gemm_stripe_kernel");
 }
 // A weight of fewer than 192 stripes: with a workspace, K slices bring the workgroups up to the chip's 256 compute units
@@ -1088,7 +1107,7 @@ static int gemm_splits(int64_t M, int64_t N, int64_t K) {
 
 template <class T>
 static int launch_stripe_slices(GemmParams& p, hipStream_t stream) {
-    if (int rc = launch_stripe<T, true>(p, stream)) return rc;
+    if (int rc = launch_stripe<T, true>(p, (p.N + 63) / 64, stream)) return rc;
     const int grid = (int)std::min<int64_t>(((int64_t)p.M * (p.N / 4) + 255) / 256, 256 * 8);
     hipLaunchKernelGGL((gemm_reduce_kernel<T>), dim3(grid), dim3(256), 0, stream, p);
     return check_launch("gemm_reduce_kernel");
@@ -1171,6 +1190,13 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
         int acc = 0;
         for (int s = 0; s < kMaxGroup; ++s) { if (s < n_w) acc += p.grp.N[s]; p.grp.end[s] = acc; }
         return launch_gemv<T, true>(p, (int)n_sum, stream);
+    }
+    // a batch of decode steps: 64-column stripes over the three weights (4096 + 1024 + 1024 columns of 4096 values: 8 rows
+    // 12.7 -> 10.8 us, 16 rows 16.3 -> 11.5, 64 rows 26.9 -> 17.5); up to three rows the kernels above and below are as fast
+    {
+        int64_t stripes = 0;
+        for (int s = 0; s < n_w; ++s) stripes += (p.grp.N[s] + 63) / 64;
+        if (p.M >= 4 && stripes <= 640 && stripe_takes(p.M, stripes, p.K)) return launch_stripe<T, false, true>(p, fill_ends(64), stream);
     }
     if (rows_lds_takes(p.M, p.K)) return launch_rows_lds<T, true>(p, fill_ends(16), stream);
     if (p.M <= 32 || (p.M <= 64 && n_sum * p.K <= (INT64_C(1) << 25))) {
@@ -1282,23 +1308,25 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     const int splits = fast && workspace && aligned16(workspace) ? gemm_splits(M, N, K) : 1;
     const bool can_split = splits > 1 && workspace_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
     // (with a workspace, K slices of the tiled kernel overtake it from 17 rows on: 32 rows against 4096 x 14336, 28 us against 52)
-    // a weight too narrow for one stripe per compute unit, with a workspace: K slices of the stripes.  Two launches, so
+    // a weight of fewer stripes than keep the memory busy, with a workspace: K slices of the stripes.  Two launches, so
     // not for the smallest weights; the 16-column kernels below, which read the activations once per 16 columns, keep up
     // to 7 rows (4096 x 14336: 18 us against 21; 8 rows 21.5 against 20.9, 16 rows 27 against 21, 64 rows 28.6 against
-    // 23.6) unless their workgroups come to two per compute unit or more (8192 x 8192 at 1-16 rows: 28-33 against 25-26)
+    // 23.6).  From 96 stripes on the plain stripes are as fast up to 32 rows (6144 x 4096: 10.8-13.4 us against 11.9-12.5)
+    // and the slices win above (64 rows 15.6 against 17.5; 8192 x 8192 29.9 against 34.7)
     const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
-    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) &&
-        ((M >= 17 && N * K >= (INT64_C(1) << 24)) || (M >= 8 && N * K >= INT64_C(25000000)) || N >= 8192)) {
+    const int64_t stripes = (N + 63) / 64;
+    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && !(stripes >= 96 && M <= 32) &&
+        ((M >= 17 && N * K >= (INT64_C(1) << 24)) || (M >= 8 && N * K >= INT64_C(25000000)))) {
         p.splits = slices; p.part = (float*)workspace;
         return dtype == MINFER_ATTN_F16 ? launch_stripe_slices<F16>(p, stream) : launch_stripe_slices<BF16>(p, stream);
     }
     // one row against a weight too narrow or too wide for the stripes: whole weight rows per wave while a row is one
     // segment (6144 x 4096: 11.7 us against 14.5 for the LDS-staged MFMA kernel below; 128256 x 4096: 157 against 185 for
     // the stripes); longer rows go to that kernel when it takes them (4096 x 14336: 18.0 against 22.1)
-    if (fast && nt && M == 1 && !stripe_takes(M, N, K) && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
+    if (fast && nt && M == 1 && !stripe_takes(M, stripes, K) && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
         return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
-    if (fast && nt && stripe_takes(M, N, K))
-        return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, stream) : launch_stripe<BF16>(p, stream);
+    if (fast && nt && stripe_takes(M, stripes, K))
+        return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, (int)stripes, stream) : launch_stripe<BF16>(p, (int)stripes, stream);
     if (fast && nt && rows_lds_takes(M, K))
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
     if (fast && nt && (M <= 16 || (!can_split && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))))

@@ -73,6 +73,9 @@ def make(M, N, K, layout, dtype, seed):
     # 1-64 rows against a weight of 12288 columns or more, K a multiple of 256: 64-column stripes over the whole of K
     (2, 12288, 256, 1.0, 0.0),       # one segment
     (1, 12296, 1024, 2.0, 3.0),      # one row
+    (1, 6144, 4096, 1.0, 0.0),       # 96 stripes: the narrowest weight it takes at any row count
+    (8, 5120, 768, 2.0, 3.0),        # 80 stripes from 8 rows on
+    (40, 4104, 1024, 1.0, 1.0),      # 65 stripes from 32 rows on, the last one of 8 columns
     (9, 12296, 512, 2.0, 3.0),       # a last stripe of 8 columns; two segments (fewer than the three stages)
     (16, 14336, 1024, 1.0, 1.0),
     (17, 12288, 768, 1.0, 0.0),      # two blocks of activation rows, the second with one row
@@ -163,10 +166,17 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
     (24, 1024, 5120, 1280, 1288),      # few rows, two column groups per workgroup, a ragged last group
     (64, 512, 768, 256, 256),          # few-row kernel at its largest row count
     (33, 50, 17, 17, 9),               # nothing tileable: three plain launches
+    # 4-64 rows, K a multiple of 256, 96 stripes of 64 columns or more over the three weights: the stripe kernel, numbered through
+    (4, 4096, 4096, 1024, 1024),
+    (16, 512, 4096, 1024, 1032),       # a last stripe of 8 columns in the third weight
+    (40, 1024, 4104, 1024, 1024),      # ... in the first; three blocks of activation rows
+    (64, 256, 5120, 520, 8),           # one segment; a weight of a single partial stripe
 ])
 def test_qkv_one_launch_equals_three_gemms(dtype, M, K, Nq, Nk, Nv):
-    """minfer_qkv (one grid over the column tiles of the three weights) against minfer_gemm per weight: the same
-    tiles run the same arithmetic, so the results are equal bit for bit; q additionally against the oracle."""
+    """minfer_qkv (one grid over the column tiles of the three weights) against minfer_gemm per weight: where the same
+    tiles run the same arithmetic the results are equal bit for bit; at 4-64 rows the one-launch form may run 64-column
+    stripes over the three weights where a single weight is too narrow for them, and then the results are equal up to
+    the order of the fp32 sums (every output against the oracle there); k always against the oracle."""
     g = torch.Generator().manual_seed(M + K + Nq)
     x = torch.randn(M, K, generator=g).to(dtype).to(DEV)
     ws = [((1 / K ** 0.5) * torch.randn(n, K, generator=g)).to(dtype).to(DEV) for n in (Nq, Nk, Nv)]
@@ -177,7 +187,11 @@ def test_qkv_one_launch_equals_three_gemms(dtype, M, K, Nq, Nk, Nv):
         ref = torch.full_like(o, float("nan"))
         assert capi.gemm(x, w, None, ref, 1.0, 0.0, NK) == capi.OK, capi.last_error()
         torch.cuda.synchronize()
-        assert torch.equal(o, ref), name
+        if M < 4 or M > 64:
+            assert torch.equal(o, ref), name
+        else:
+            assert_close(o, oracle.gemm(x.cpu(), w.cpu(), None, 1.0, 0.0, NK), dtype, name + " against the oracle")
+            assert float((o.float() - ref.float()).abs().max()) <= 2.0 ** -MANT[dtype] * float(ref.float().abs().max()), name
     rows = torch.arange(0, M, max(1, M // 24))
     assert_close(outs[1][rows], oracle.gemm(x[rows].cpu(), ws[1].cpu(), None, 1.0, 0.0, NK), dtype, "k against the oracle")
 
