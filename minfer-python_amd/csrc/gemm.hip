@@ -1093,11 +1093,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
 
 // How many K slices a problem is cut into when a workspace is at hand: problems whose 128 x 128 tiles would leave most
 // of the chip idle (a few dozen rows against a wide weight), every slice at least 4 steps of 64 long.  1 = no split.
+// Up to 256 tiles: one workgroup of these tiles per compute unit leaves its matrix pipes waiting for every K step, two
+// overlap (256 x 8192 x 8192, 128 tiles: 75 -> 52 us; 512 x 8192 x 28672, 256 tiles: 400 -> 317).
 static int gemm_splits(int64_t M, int64_t N, int64_t K) {
     if (K % kBK != 0 || N % 8 != 0) return 1;
     const int64_t tiles = ((M + GemmSmall::BM - 1) / GemmSmall::BM) * ((N + GemmSmall::BN - 1) / GemmSmall::BN);
     const int64_t kt = K / kBK;
-    if (tiles >= 128 || kt < 8) return 1;
+    if (tiles > 256 || kt < 8) return 1;
     int64_t s = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, kt / 4), 32));
     // 64-127 tiles get two or three slices that way and fill the chip once; twice as many, while a slice stays 16 steps long,
     // keep two workgroups on a compute unit ([K,N] 4096 x 14336 at 1-16 rows: 27.5 -> 22 us; 128 rows 37 -> 32)

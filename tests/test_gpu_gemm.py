@@ -245,6 +245,7 @@ def test_qkv_op_and_reference_checks(kerns):
     (40, 512, 1984, 1.0, 0.0),       # K steps (31) not a multiple of the slice count
     (1, 4096, 4096, 1.0, 1.0),       # one row: with [K, N] the sliced tiles, with [N, K] still the few-row kernel
     (24, 1024, 2048, 1.0, 1.0),      # 17-32 rows: with a workspace the sliced tiles for both layouts
+    (256, 8192, 1024, 1.0, 1.0),     # 128 tiles: two slices, so that two workgroups share a compute unit
     # [N, K] weights of fewer than 192 stripes of 64 columns: K slices of the stripe kernel
     (8, 5120, 5120, 2.0, 3.0),       # 80 stripes, three slices of 6, 7 and 7 segments
     (16, 4104, 8192, 1.0, 1.0),      # a last stripe of 8 columns
