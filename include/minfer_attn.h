@@ -244,10 +244,9 @@ int minfer_gemm_q8_0(const void* A, const void* Bq, const void* C, void* D, int6
  * expected values test/kernels.py:172-216).  One grid covers the column tiles of all three weights, so x is
  * read by one kernel and the narrow k and v projections share the launch with the wide q projection; every element
  * equals what minfer_gemm with MINFER_GEMM_B_NK, alpha 1, beta 0 gives for its weight, up to the order of the fp32
- * sums (bit for bit from 65 rows on and up to 3, where both take the same kernel; at 4-64 rows the one launch may run
- * 64-column stripes over the three weights where a single weight is too narrow for them, and a single weight of 6144
- * columns or more runs them at 1-3 rows too).  Shapes the tiled kernels cannot take (see minfer_gemm) run as three
- * plain launches.
+ * sums (bit for bit from 65 rows on, where both run the same tiles; up to 64 rows the few-row kernel is chosen by the
+ * width, which is the three weights' together here and one weight's there).  Shapes the tiled kernels cannot take (see
+ * minfer_gemm) run as three plain launches.
  */
 int minfer_qkv(int dtype, const void* x, const void* wq, const void* wk, const void* wv,
                void* q_out, void* k_out, void* v_out, int64_t M, int64_t K, int64_t Nq, int64_t Nk, int64_t Nv,

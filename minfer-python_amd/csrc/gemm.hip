@@ -662,14 +662,13 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
     }
 }
-// It needs stripes enough to keep the memory busy, which is fewer than there are compute units: 128 workgroups stream an
-// 8192 x 8192 weight at 6.5 TB/s (20.6 us at 1-8 rows, where the 16-column kernels take 28-31), 96 a 6144 x 4096 one in
-// 10.8-13.4 us at 1-32 rows (11.5-20.1).  From 96 stripes on it takes every row count up to 64, one row too (14336 x 4096:
-// 18.0 us against 19.6 for whole rows per wave, 12288 x 8192: 29.5 against 39); 80 stripes from 8 rows on (5120 x 5120:
-// 13.6 against 15.4, one row 13.3 against 12.4), 64 from 32 rows on (4096 x 4096: 13.2 against 15.6).  Against a very wide
-// weight (an output head: 2004 stripes, eight rounds of one workgroup per compute unit) what each workgroup pays before
-// its first segment adds up, and up to eight rows the kernels that keep more workgroups on a unit are faster (128256 x
-// 4096: 157-181 against 185 us).
+// How many stripes it needs: from 96 on it is the fastest kernel without a workspace from 9 rows up (6144 x 4096, the
+// weight coming from memory, at 16 rows: 15.8 us against 17.4 for the 16-column kernel, 32 rows 18.2 against 21.5); with
+// the weight in the last-level cache 80 stripes were enough from 8 rows on (5120 x 5120: 13.6 against 15.4) and 64 from
+// 32 rows on (4096 x 4096: 13.2 against 15.6).  Which row counts below 9 reach it is the caller's rule (gemm_impl).
+// Against a very wide weight (an output head: 2004 stripes, eight rounds of one workgroup per compute unit) what each
+// workgroup pays before its first segment adds up, and up to eight rows the kernels that keep more workgroups on a unit
+// are faster (128256 x 4096: 157-181 against 185 us).
 static bool stripe_takes(int64_t M, int64_t stripes, int64_t K) {
     if (M < 1 || M > 64 || K % kStripeSeg != 0) return false;
     if (stripes > 640) return M >= 9;
@@ -1188,17 +1187,17 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
         }
         return acc;
     };
-    if (p.M == 1 && (p.K <= kGemvSegHalfs || (p.K <= kGemvMaxKHalfs && !rows_lds_takes(p.M, p.K))) && n_sum <= 0x7fffffffLL) {   // one row: whole weight rows per wave, numbered through
+    if (p.M == 1 && p.K <= kGemvMaxKHalfs && (n_sum * p.K >= (INT64_C(1) << 25) || !rows_lds_takes(p.M, p.K)) && n_sum <= 0x7fffffffLL) {   // one row: whole weight rows per wave, numbered through (the rule of gemm_impl)
         int acc = 0;
         for (int s = 0; s < kMaxGroup; ++s) { if (s < n_w) acc += p.grp.N[s]; p.grp.end[s] = acc; }
         return launch_gemv<T, true>(p, (int)n_sum, stream);
     }
-    // a batch of decode steps: 64-column stripes over the three weights (4096 + 1024 + 1024 columns of 4096 values: 8 rows
-    // 12.7 -> 10.8 us, 16 rows 16.3 -> 11.5, 64 rows 26.9 -> 17.5); up to three rows the kernels above and below are as fast
+    // a batch of decode steps: 64-column stripes over the three weights from 9 rows on (4096 + 1024 + 1024 columns of 4096
+    // values, weights coming from memory: 16 rows 15.8 us against 17.4 for the 16-column kernel, 32 rows 18.2 against 21.5)
     {
         int64_t stripes = 0;
         for (int s = 0; s < n_w; ++s) stripes += (p.grp.N[s] + 63) / 64;
-        if (p.M >= 4 && stripes <= 640 && stripe_takes(p.M, stripes, p.K)) return launch_stripe<T, false, true>(p, fill_ends(64), stream);
+        if (p.M >= 9 && stripes <= 640 && stripe_takes(p.M, stripes, p.K)) return launch_stripe<T, false, true>(p, fill_ends(64), stream);
     }
     if (rows_lds_takes(p.M, p.K)) return launch_rows_lds<T, true>(p, fill_ends(16), stream);
     if (p.M <= 32 || (p.M <= 64 && n_sum * p.K <= (INT64_C(1) << 25))) {
@@ -1304,33 +1303,41 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
                       aligned16(A) && aligned16(B) && ((uintptr_t)D & 7u) == 0 && ((uintptr_t)C & 7u) == 0 &&
                       (int64_t)GemmBig::BM * lda < (1LL << 30) && (int64_t)std::max<int64_t>(GemmBig::BN, kBK) * ldb < (1LL << 30);
     hipStream_t stream = (hipStream_t)stream_v;
-    // a decode step's few tokens against an [N, K] weight: stream the weight once
-    // (up to 32 rows it beats the tiled kernel at every weight size measured, 7-34 us against 40-133 us; with 33-64 rows,
-    // whose fragments are re-read from L2 for every 16 columns, only while the weight is small and no workspace allows K slices)
+    // A decode step's few tokens against an [N, K] weight: stream the weight once.  Which kernel does that best was
+    // measured with the calls cycling over copies of the weight, 640 MiB in all: a weight of up to 256 MiB called again
+    // and again is served by the chip's last-level cache, where the order of the kernels is a different one (14336 x
+    // 4096 at one row: stripes 18.0 us against 19.5 for whole rows per wave from the cache, 24.2 against 21.9 from memory).
     const int splits = fast && workspace && aligned16(workspace) ? gemm_splits(M, N, K) : 1;
     const bool can_split = splits > 1 && workspace_bytes >= (size_t)splits * (size_t)M * (size_t)N * sizeof(float);
-    // (with a workspace, K slices of the tiled kernel overtake it from 17 rows on: 32 rows against 4096 x 14336, 28 us against 52)
-    // a weight of fewer stripes than keep the memory busy, with a workspace: K slices of the stripes.  Two launches, so
-    // not for the smallest weights; the 16-column kernels below, which read the activations once per 16 columns, keep up
-    // to 7 rows (4096 x 14336: 18 us against 21; 8 rows 21.5 against 20.9, 16 rows 27 against 21, 64 rows 28.6 against
-    // 23.6).  From 96 stripes on the plain stripes are as fast up to 32 rows (6144 x 4096: 10.8-13.4 us against 11.9-12.5)
-    // and the slices win above (64 rows 15.6 against 17.5; 8192 x 8192 29.9 against 34.7)
-    const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
     const int64_t stripes = (N + 63) / 64;
-    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && !(stripes >= 96 && M <= 32) &&
-        ((M >= 17 && N * K >= (INT64_C(1) << 24)) || (M >= 8 && N * K >= INT64_C(25000000)))) {
+    const bool rows_takes = rows_lds_takes(M, K);
+    // one row: whole weight rows per wave (14336 x 4096: 21.9 us, the 16-column kernel 23.6, stripes 24.2; 28672 x 8192:
+    // 75.8 / 91 / 97); a weight under 32 M values goes to the 16-column kernel when it takes it (4096 x 4096: 8.5 against 10.5)
+    if (fast && nt && M == 1 && K <= kGemvMaxKHalfs && (N * K >= (INT64_C(1) << 25) || !rows_takes))
+        return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
+    // up to 8 rows: the 16-column kernel, whose many small bursts spread over the memory channels better than a stripe's
+    // 64 rows at one K offset (28672 x 4096 at 2-8 rows: 41.4-44.5 us against 46.5; 6144 x 4096: 12.1-14.0 against
+    // 14.4-15.0), except where it was measured behind: rows of 8192-16384 values against 96-256 stripes (10240 x 8192:
+    // 38.8-43.3 against 35.5-36.6) and 4 rows or more against 192-256 stripes (14336 x 4096 at 8 rows: 25.8 against 23.6)
+    const bool rows_first = rows_takes && M <= 8 &&
+                            !(stripes >= 96 && stripes <= 256 && ((K >= 8192 && K <= 16384) || (M >= 4 && stripes >= 192)));
+    if (fast && nt && rows_first)
+        return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
+    // fewer than 192 stripes, with a workspace: K slices of the stripes from 9 rows on (6144 x 4096 at 16 rows: 14.2 us
+    // against 15.8 for the plain stripes and 17.4 for the 16-column kernel; 8192 x 28672 at 16-32 rows: 83 against
+    // 102-116; 4096 x 14336 at 16 rows 24.5 against 29.3).  Two launches, so not for the smallest weights.
+    const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
+    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && M >= 9 &&
+        N * K >= (M >= 17 ? (INT64_C(1) << 24) : INT64_C(25000000))) {
         p.splits = slices; p.part = (float*)workspace;
         return dtype == MINFER_ATTN_F16 ? launch_stripe_slices<F16>(p, stream) : launch_stripe_slices<BF16>(p, stream);
     }
-    // one row against a weight too narrow or too wide for the stripes: whole weight rows per wave while a row is one
-    // segment (6144 x 4096: 11.7 us against 14.5 for the LDS-staged MFMA kernel below; 128256 x 4096: 157 against 185 for
-    // the stripes); longer rows go to that kernel when it takes them (4096 x 14336: 18.0 against 22.1)
-    if (fast && nt && M == 1 && !stripe_takes(M, stripes, K) && (K <= kGemvSegHalfs || (K <= kGemvMaxKHalfs && !rows_lds_takes(M, K))))
-        return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
     if (fast && nt && stripe_takes(M, stripes, K))
         return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, (int)stripes, stream) : launch_stripe<BF16>(p, (int)stripes, stream);
-    if (fast && nt && rows_lds_takes(M, K))
+    if (fast && nt && rows_takes)
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
+    if (fast && nt && M == 1 && K <= kGemvMaxKHalfs)
+        return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
     if (fast && nt && (M <= 16 || (!can_split && (M <= 32 || (M <= 64 && N * K <= (INT64_C(1) << 25))))))
         return dtype == MINFER_ATTN_F16 ? launch_skinny<F16>(p, stream) : launch_skinny<BF16>(p, stream);
     if (can_split) {
