@@ -718,9 +718,11 @@ template <> MA_DEV float dot8<BF16>(uint4 a, uint4 b, float acc) {   // a bf16 i
 constexpr int kGemvMaxKHalfs = 16384;                      // activation row kept in LDS: 32 KiB
 // GROUPED: the rows of up to three weights numbered through (p.grp.end[s] = rows of weights 0 .. s), every weight with
 // its own output; alpha = 1, no C.
-template <class T, bool XREG, bool GROUPED>
+// MR: activation rows (1-4; more than one only ungrouped): every weight piece is multiplied with the same piece of each.
+template <class T, bool XREG, bool GROUPED, int MR = 1>
 __global__ __launch_bounds__(4 * 64) void gemv_kernel(const GemmParams p, int rows_per_wave) {
-    __shared__ __attribute__((aligned(16))) short x_lds[XREG ? 8 : kGemvMaxKHalfs];
+    static_assert(MR == 1 || !GROUPED, "several activation rows: one weight only");
+    __shared__ __attribute__((aligned(16))) short x_lds[XREG ? 8 : (MR == 1 ? kGemvMaxKHalfs : 2 * kGemvMaxKHalfs)];   // MR rows of K values: MR * K <= 32768
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
     const int npiece = p.K / 8, nseg = XREG ? 1 : (p.K + kGemvSegHalfs - 1) / kGemvSegHalfs;
     const int wave = (int)blockIdx.x * 4 + w;
@@ -753,17 +755,23 @@ __global__ __launch_bounds__(4 * 64) void gemv_kernel(const GemmParams p, int ro
     Unit ring[2];
     request(0, ring[0]);
     request(1, ring[1]);
-    uint4 xr[kGemvSegPieces];
+    uint4 xr[MR][kGemvSegPieces];
     if (XREG) {
 #pragma unroll
-        for (int j = 0; j < kGemvSegPieces; ++j)
-            xr[j] = *reinterpret_cast<const uint4*>((const short*)p.A + 8 * min(64 * j + lane, npiece - 1));
+        for (int m = 0; m < MR; ++m)
+#pragma unroll
+            for (int j = 0; j < kGemvSegPieces; ++j)
+                xr[m][j] = *reinterpret_cast<const uint4*>((const short*)p.A + (int64_t)min(m, p.M - 1) * p.lda + 8 * min(64 * j + lane, npiece - 1));
     } else {
-        for (int i = tid; i < npiece; i += 4 * 64)
-            *reinterpret_cast<uint4*>(x_lds + 8 * i) = *reinterpret_cast<const uint4*>((const short*)p.A + 8 * i);
+        for (int i = tid; i < MR * npiece; i += 4 * 64) {
+            const int m = i / npiece, pc = i - m * npiece;
+            *reinterpret_cast<uint4*>(x_lds + 8 * i) = *reinterpret_cast<const uint4*>((const short*)p.A + (int64_t)min(m, p.M - 1) * p.lda + 8 * pc);
+        }
         __syncthreads();
     }
-    float acc = 0.f;
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
     auto consume = [&](int u, Unit& un) {
         const int row = r0 + u / nseg, seg = u % nseg;
         uint4 wv[kGemvSegPieces];
@@ -773,21 +781,29 @@ __global__ __launch_bounds__(4 * 64) void gemv_kernel(const GemmParams p, int ro
 #pragma unroll
         for (int j = 0; j < kGemvSegPieces; ++j) {
             const int piece = seg * (kGemvSegHalfs / 8) + 64 * j + lane;
-            if (piece < npiece) acc = dot8<T>(wv[j], XREG ? xr[j] : *reinterpret_cast<const uint4*>(x_lds + 8 * piece), acc);
+            if (piece < npiece) {
+#pragma unroll
+                for (int m = 0; m < MR; ++m)
+                    acc[m] = dot8<T>(wv[j], XREG ? xr[m][j] : *reinterpret_cast<const uint4*>(x_lds + 8 * (m * npiece + piece)), acc[m]);
+            }
         }
         if (seg == nseg - 1) {
-            float v = acc;
-            acc = 0.f;
 #pragma unroll
-            for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
-            if (lane == 0) {
-                const short* unused; short* out;
-                locate(row, unused, out);
-                if (!GROUPED) {
-                    v *= p.alpha;
-                    if (p.beta != 0.f) v += p.beta * T::to_float(((const short*)p.C)[row]);
+            for (int m = 0; m < MR; ++m) {
+                float v = acc[m];
+                acc[m] = 0.f;
+#pragma unroll
+                for (int off = 32; off >= 1; off >>= 1) v += __shfl_xor(v, off);
+                if (lane == 0 && m < p.M) {
+                    const short* unused; short* out;
+                    locate(row, unused, out);
+                    if (!GROUPED) {
+                        v *= p.alpha;
+                        if (p.beta != 0.f) v += p.beta * T::to_float(((const short*)p.C)[(int64_t)m * p.ldc + row]);
+                        out += (int64_t)m * p.ldd;
+                    }
+                    *out = (short)(T::pack2(v, 0.f) & 0xffffu);
                 }
-                *out = (short)(T::pack2(v, 0.f) & 0xffffu);
             }
         }
     };
@@ -802,10 +818,17 @@ static int launch_gemv(const GemmParams& p, int n_rows, hipStream_t stream) {
     const int rows_per_wave = (n_rows + max_waves - 1) / max_waves;
     const int waves = (n_rows + rows_per_wave - 1) / rows_per_wave;
     const dim3 grid((waves + 3) / 4), block(4 * 64);
-    if (p.K <= kGemvSegHalfs) hipLaunchKernelGGL((gemv_kernel<T, true, GROUPED>), grid, block, 0, stream, p, rows_per_wave);
-    else hipLaunchKernelGGL((gemv_kernel<T, false, GROUPED>), grid, block, 0, stream, p, rows_per_wave);
+    const bool xreg = p.K <= kGemvSegHalfs;
+#define MINFER_GEMV(XR, MR) hipLaunchKernelGGL((gemv_kernel<T, XR, GROUPED, MR>), grid, block, 0, stream, p, rows_per_wave)
+    if (GROUPED || p.M == 1) { if (xreg) MINFER_GEMV(true, 1); else MINFER_GEMV(false, 1); }
+    else if (p.M == 2) MINFER_GEMV(false, GROUPED ? 1 : 2);   // (several rows: rows longer than a segment only, see gemv_takes)
+    else if (p.M == 3) MINFER_GEMV(false, GROUPED ? 1 : 3);
+    else MINFER_GEMV(false, GROUPED ? 1 : 4);
+#undef MINFER_GEMV
     return check_launch("gemv_kernel");
 }
+// which calls it takes: one row, or up to four rows longer than a segment whose activations fit its LDS area
+static bool gemv_takes(int64_t M, int64_t K) { return M >= 1 && M <= 4 && K <= kGemvMaxKHalfs && (M == 1 || (K > kGemvSegHalfs && M * K <= 2 * kGemvMaxKHalfs)); }
 
 template <class T>
 static int launch_skinny(const GemmParams& p, hipStream_t stream) {
@@ -1314,6 +1337,11 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     // one row: whole weight rows per wave (14336 x 4096: 21.9 us, the 16-column kernel 23.6, stripes 24.2; 28672 x 8192:
     // 75.8 / 91 / 97); a weight under 32 M values goes to the 16-column kernel when it takes it (4096 x 4096: 8.5 against 10.5)
     if (fast && nt && M == 1 && K <= kGemvMaxKHalfs && (N * K >= (INT64_C(1) << 25) || !rows_takes))
+        return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
+    // two to four rows against long rows of a wide weight go the same way, every weight piece multiplied with the same
+    // piece of each activation row (28672 x 8192 at 2-4 rows: 78.6-82.6 us against 93-95 for the 16-column kernel, 10240 x
+    // 8192 at 2-3 rows 33.2-34.6 against 36.3; 8192 x 8192 30.5-33.9 against 29.2-29.6, and rows of 4096 values gain nothing)
+    if (fast && nt && M >= 2 && gemv_takes(M, K) && K >= 8192 && N >= 10240 && (M <= 3 || N >= 16384))
         return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
     // up to 8 rows: the 16-column kernel, whose many small bursts spread over the memory channels better than a stripe's
     // 64 rows at one K offset (28672 x 4096 at 2-8 rows: 41.4-44.5 us against 46.5; 6144 x 4096: 12.1-14.0 against

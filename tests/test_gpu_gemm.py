@@ -90,6 +90,10 @@ def make(M, N, K, layout, dtype, seed):
     (1, 264, 16384, 1.0, 1.0),       # the longest activation row its LDS area holds
     (1, 264, 16448, 1.0, 0.0),       # longer: the 16-rows-per-instruction kernel
     (1, 8, 192, 1.0, 1.0),           # two waves with rows, the others none
+    # two to four rows against long rows of a wide weight: whole weight rows per wave, every piece times the same piece of each activation row
+    (2, 10240, 8192, 1.0, 0.0),
+    (3, 10248, 8192, 2.0, 3.0),      # a last wave with fewer rows
+    (4, 16384, 8192, 1.0, 1.0),
 ])
 def test_gemm_matches_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, M + N + K)
