@@ -536,27 +536,43 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
     __shared__ __attribute__((aligned(16))) char x_lds[XST][G::X_BYTES];
     const int lane = threadIdx.x & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    int stripe = (int)blockIdx.x, slice = 0, seg0 = 0, nseg = p.K / kStripeSeg;
+    int slice = 0, seg0 = 0, nseg = p.K / kStripeSeg;
     if (SLICED) {
-        stripe = (int)blockIdx.x / p.splits; slice = (int)blockIdx.x % p.splits;
+        slice = (int)blockIdx.x % p.splits;
         seg0 = slice * nseg / p.splits;
         nseg = (slice + 1) * nseg / p.splits - seg0;
     }
+    // Which columns.  SLICED: workgroup b / splits owns stripe b / splits.  Plain launches: the 16-column blocks of the weight
+    // are shared out evenly: workgroup g of G owns blocks g * blocks / G ..
+    // (g + 1) * blocks / G - 1 and goes through them four at a time, a chunk ending early at the end of the workgroup's
+    // range; the waves without a block of their own in such a chunk copy its last row again (from L2) and
+    // multiply what is never stored.  Every compute unit so streams the same share of the weight to within one block,
+    // whatever the number of columns (448 stripes of 64 columns are one and three quarter rounds of 256 workgroups:
+    // 28672 x 4096 from memory 46.5 -> 41.5-42.3 us), and a narrow weight is spread over the whole chip (6144 x 4096 at
+    // 9-16 rows: 96 stripes 15.2-15.9 us, 256 workgroups of one or two blocks 12.3-12.7).
+    // (GROUPED: one workgroup per stripe of 64 columns, the stripes of the weights numbered through, as SLICED has one per
+    // stripe and slice: with the lookup of the chunk's weight inside the chunk loop the grouped launch ran 20 us where the
+    // plain one ran 11, for the same instructions and the same memory traffic)
+    const int blk_first = SLICED ? 4 * ((int)blockIdx.x / p.splits) : GROUPED ? 0 : (int)((int64_t)blockIdx.x * p.tiles_n / (int)gridDim.x);
+    const int blk_last = SLICED ? min(blk_first + 4, p.tiles_n) : GROUPED ? 1 : (int)((int64_t)(blockIdx.x + 1) * p.tiles_n / (int)gridDim.x);
     const short* Bg = (const short*)p.B;
     short* Dg = (short*)p.D;
-    int N = p.N;
+    int Nw = p.N, grp_local = 0;
     int64_t ldb = p.ldb, ldd = p.ldd;
     if (GROUPED) {   // the stripe's weight, output and place inside them (uniform)
-        int local;
-        const int sg = group_of_unit(p.grp, stripe, local);
-        stripe = local;
+        const int sg = group_of_unit(p.grp, (int)blockIdx.x, grp_local);
         Bg = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]);
         Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
-        N = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
+        Nw = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
         ldb = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
         ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
     }
-    const int n0 = stripe * 64 + 16 * w;                       // the columns this wave copies and, at the end, writes
+    for (int cb = blk_first; cb < blk_last;) {
+    const int local = GROUPED ? 4 * grp_local : cb;
+    const int nb = GROUPED ? 4 : min(4, blk_last - cb);
+    int N = Nw;
+    N = min(N, 16 * (local + nb));                             // rows past the chunk are not this chunk's
+    const int n0 = 16 * local + 16 * w;                        // the columns this wave copies and, at the end, writes
     // copy instruction for row pair i: lane L lands at byte 16 L of the block and fetches piece (L >> 1) ^ (i & 7) of
     // row 2i + (L & 1)
     const short* wsrc[8];
@@ -567,9 +583,9 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
 #pragma unroll
     for (int j = 0; j < 2 * MB; ++j)
         xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * ((lane >> 1) ^ ((w + 4 * j) & 7));
-    // Stripe b starts at segment b mod nseg and wraps: the stripes running at one time then read different segments of
-    // the activation rows instead of the same few lines of the same few L2 channels
-    const int rot = (int)((SLICED ? blockIdx.x : (unsigned)stripe) % (unsigned)nseg);   // (a stripe's place in its own weight: the grouped launch adds it up as the plain one does)
+    // A chunk starts at segment (its place in the weight) mod nseg and wraps: the chunks running at one time then read
+    // different segments of the activation rows instead of the same few lines of the same few L2 channels
+    const int rot = (int)((SLICED ? blockIdx.x : (unsigned)(local >> 2)) % (unsigned)nseg);
     auto seg_k0 = [&](int t) { const int sg = t + rot; return (seg0 + (sg >= nseg ? sg - nseg : sg)) * kStripeSeg; };
     auto issue_w = [&](int t) {
         char* st = w_lds[t % WST];
@@ -612,18 +628,23 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         __syncthreads();                                       // ... for every wave's copies
         const char* wb = w_lds[t % WST];
         const char* xb = x_lds[t % XST];
+        // all fragments of the wave's two k steps first, then the MFMAs: left to itself the compiler pipelines these reads
+        // in one instantiation and waits for each before its MFMA in another (the grouped one ran twice as long for it)
+        s16x8 a[2][4], b[2][MB];
 #pragma unroll
         for (int s = 0; s < 2; ++s) {
-            s16x8 b[MB];
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) b[mb] = *reinterpret_cast<const s16x8*>(xb + mb * 8 * kStripeBlock + frag[s]);
+            for (int mb = 0; mb < MB; ++mb) b[s][mb] = *reinterpret_cast<const s16x8*>(xb + mb * 8 * kStripeBlock + frag[s]);
 #pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const s16x8 a = *reinterpret_cast<const s16x8*>(wb + c * 8 * kStripeBlock + frag[s]);
-#pragma unroll
-                for (int mb = 0; mb < MB; ++mb) acc[c][mb] = T::mfma16(a, b[mb], acc[c][mb]);
-            }
+            for (int c = 0; c < 4; ++c) a[s][c] = *reinterpret_cast<const s16x8*>(wb + c * 8 * kStripeBlock + frag[s]);
         }
+        __builtin_amdgcn_sched_barrier(0);                     // (the scheduler moves nothing across this)
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) acc[c][mb] = T::mfma16(a[s][c], b[s][mb], acc[c][mb]);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // fragments in registers before the barrier that frees the stage
     }
     // partial sums of the four waves: wave u leaves column block c at red[u][c][mb][lane]; wave w adds up column block w
@@ -636,11 +657,10 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         for (int mb = 0; mb < MB; ++mb) red[((w * 4 + c) * MB + mb) * 64 + lane] = acc[c][mb];
     __syncthreads();
     const int n = n0 + 4 * quad;                               // register r of a lane: weight row n + r, activation row 16mb + l16
-    if (n >= N) return;
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb) {
         const int m = 16 * mb + l16;
-        if (m >= p.M) continue;
+        if (m >= p.M || n >= N) continue;
         f32x4 sum = red[((0 * 4 + w) * MB + mb) * 64 + lane];
 #pragma unroll
         for (int u = 1; u < 4; ++u) sum += red[((u * 4 + w) * MB + mb) * 64 + lane];
@@ -661,22 +681,26 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         pk.y = T::pack2(v[2], v[3]);
         *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
     }
+    cb += GROUPED ? 1 : nb;
+    if (cb < blk_last) __syncthreads();                        // the sums have been read: the next chunk's copies may land there
+    }
 }
-// How many stripes it needs: from 96 on it is the fastest kernel without a workspace from 9 rows up (6144 x 4096, the
-// weight coming from memory, at 16 rows: 15.8 us against 17.4 for the 16-column kernel, 32 rows 18.2 against 21.5); with
-// the weight in the last-level cache 80 stripes were enough from 8 rows on (5120 x 5120: 13.6 against 15.4) and 64 from
-// 32 rows on (4096 x 4096: 13.2 against 15.6).  Which row counts below 9 reach it is the caller's rule (gemm_impl).
-// Against a very wide weight (an output head: 2004 stripes, eight rounds of one workgroup per compute unit) what each
-// workgroup pays before its first segment adds up, and up to eight rows the kernels that keep more workgroups on a unit
-// are faster (128256 x 4096: 157-181 against 185 us).
+// Which widths it takes (in stripes of 64 columns; weights coming from memory): from 96 on every row count that reaches
+// it (14336 x 4096 at 2-32 rows 22.8-23.7 us, the 16-column kernel 24.3-32.4; 6144 x 4096 at 9-32 rows 12.3-15.5 against
+// 14.4-21.5); 80 from 8 rows on and 64 from 32 rows on, where no workspace allows K slices (5120 x 5120 at 16 rows 15.8
+// against 20.5; 4096 x 4096 at 32 rows 13.6 against 16.3); an output head from 5 rows on (128256 x 4096 at 8 rows 179 against
+// 183, 57344 x 8192 166 against 185; up to 4 rows the kernels that keep more workgroups on a compute unit are ahead).
 static bool stripe_takes(int64_t M, int64_t stripes, int64_t K) {
     if (M < 1 || M > 64 || K % kStripeSeg != 0) return false;
-    if (stripes > 640) return M >= 9;
+    if (stripes > 640) return M >= 5;
     return stripes >= 96 || (stripes >= 80 && M >= 8) || (stripes >= 64 && M >= 32);
 }
+// `blocks`: 16-column blocks in all (GROUPED: stripes of 64 columns in all, p.grp.end counting them per weight).
 template <class T, bool SLICED = false, bool GROUPED = false>
-static int launch_stripe(const GemmParams& p, int stripes, hipStream_t stream) {
-    const dim3 grid(stripes * (SLICED ? p.splits : 1)), block(4 * 64);
+static int launch_stripe(const GemmParams& p0, int blocks, hipStream_t stream) {
+    GemmParams p = p0;
+    p.tiles_n = blocks;
+    const dim3 grid(SLICED ? (blocks + 3) / 4 * p.splits : GROUPED ? blocks : std::min(blocks, 256)), block(4 * 64);   // (GROUPED: `blocks` counts stripes)
     if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1, SLICED, GROUPED>), grid, block, 0, stream, p);
     else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2, SLICED, GROUPED>), grid, block, 0, stream, p);
     else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_kernel<T, 3, SLICED, GROUPED>), grid, block, 0, stream, p);
@@ -1131,7 +1155,7 @@ static int gemm_splits(int64_t M, int64_t N, int64_t K) {
 
 template <class T>
 static int launch_stripe_slices(GemmParams& p, hipStream_t stream) {
-    if (int rc = launch_stripe<T, true>(p, (p.N + 63) / 64, stream)) return rc;
+    if (int rc = launch_stripe<T, true>(p, (p.N + 15) / 16, stream)) return rc;
     const int grid = (int)std::min<int64_t>(((int64_t)p.M * (p.N / 4) + 255) / 256, 256 * 8);
     hipLaunchKernelGGL((gemm_reduce_kernel<T>), dim3(grid), dim3(256), 0, stream, p);
     return check_launch("gemm_reduce_kernel");
@@ -1343,25 +1367,24 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     // 8192 at 2-3 rows 33.2-34.6 against 36.3; 8192 x 8192 30.5-33.9 against 29.2-29.6, and rows of 4096 values gain nothing)
     if (fast && nt && M >= 2 && gemv_takes(M, K) && K >= 8192 && N >= 10240 && (M <= 3 || N >= 16384))
         return dtype == MINFER_ATTN_F16 ? launch_gemv<F16>(p, p.N, stream) : launch_gemv<BF16>(p, p.N, stream);
-    // up to 8 rows: the 16-column kernel, whose many small bursts spread over the memory channels better than a stripe's
-    // 64 rows at one K offset (28672 x 4096 at 2-8 rows: 41.4-44.5 us against 46.5; 6144 x 4096: 12.1-14.0 against
-    // 14.4-15.0), except where it was measured behind: rows of 8192-16384 values against 96-256 stripes (10240 x 8192:
-    // 38.8-43.3 against 35.5-36.6) and 4 rows or more against 192-256 stripes (14336 x 4096 at 8 rows: 25.8 against 23.6)
-    const bool rows_first = rows_takes && M <= 8 &&
-                            !(stripes >= 96 && stripes <= 256 && ((K >= 8192 && K <= 16384) || (M >= 4 && stripes >= 192)));
+    // up to 8 rows against fewer than 96 stripes, and up to 4 against an output head: the 16-column kernel (4096 x 14336 at
+    // 2-8 rows: 23.5-24.4 us against 32.5 for the stripes' blocks shared out; 128256 x 4096 at 2-4 rows 166-170 against
+    // 176-178; 28672 x 4096 at 2-8 rows 42.2-44.5 against 41.5-41.7 and 14336 x 4096 24.3-25.8 against 22.8-23.0: those go on)
+    const bool rows_first = rows_takes && ((M <= 8 && stripes < 96) || (M <= 4 && stripes > 640));
     if (fast && nt && rows_first)
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
-    // fewer than 192 stripes, with a workspace: K slices of the stripes from 9 rows on (6144 x 4096 at 16 rows: 14.2 us
-    // against 15.8 for the plain stripes and 17.4 for the 16-column kernel; 8192 x 28672 at 16-32 rows: 83 against
-    // 102-116; 4096 x 14336 at 16 rows 24.5 against 29.3).  Two launches, so not for the smallest weights.
+    // with a workspace, K slices of the stripes: fewer than 96 stripes from 9 rows on (4096 x 14336 at 16 rows 24.5 us against
+    // 29.1 for the 16-column kernel and 33 for the blocks shared out; 5120 x 5120 14.6 / 20.5 / 15.8), 96-191 stripes from 33
+    // rows on (6144 x 4096 at 64 rows 18.6 against 20.2, 8192 x 8192 33.9 against 37.8; up to 32 rows the blocks shared out
+    // are ahead: 6144 x 4096 at 16 rows 12.7 against 14.3).  Two launches, so not for the smallest weights.
     const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
-    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && M >= 9 &&
+    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (stripes < 96 ? M >= 9 : M > 32) &&
         N * K >= (M >= 17 ? (INT64_C(1) << 24) : INT64_C(25000000))) {
         p.splits = slices; p.part = (float*)workspace;
         return dtype == MINFER_ATTN_F16 ? launch_stripe_slices<F16>(p, stream) : launch_stripe_slices<BF16>(p, stream);
     }
     if (fast && nt && stripe_takes(M, stripes, K))
-        return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, (int)stripes, stream) : launch_stripe<BF16>(p, (int)stripes, stream);
+        return dtype == MINFER_ATTN_F16 ? launch_stripe<F16>(p, (int)((N + 15) / 16), stream) : launch_stripe<BF16>(p, (int)((N + 15) / 16), stream);
     if (fast && nt && rows_takes)
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
     if (fast && nt && M == 1 && K <= kGemvMaxKHalfs)
