@@ -1097,6 +1097,163 @@ static int launch_skinny_q8(const GemmParams& p, hipStream_t stream) {
     return check_launch("gemm_skinny_q8_kernel");
 }
 
+// The stripe kernel over a weight of Q8_0 blocks ([N][K/32] blocks of 34 bytes, K a multiple of 256, rows 16-byte
+// aligned): the same sharing out of 16-column blocks, chunks of four, segments of 256 values, split of a segment's k
+// steps over the four waves and sum through LDS as gemm_stripe_kernel, with the weight staged as the raw blocks.  A
+// segment of a row is 8 blocks = 272 bytes = 17 pieces of 16 bytes; the 64 rows of a chunk are 1088 pieces = 17 copy
+// instructions of 64 lanes, lane L of instruction j taking piece 64 j + L of the chunk (row (64 j + L) / 17), so that
+// a stage is the 64 row segments one after the other, 272 bytes each (a fragment's 16 rows are 68 words apart: 16
+// different groups of four banks).  Every wave issues five of them per segment (j = w, w + 4, ..; the three past the
+// seventeenth fetch the chunk's last piece again and land behind the stage).  A k step is one block: the lane of row
+// r, k quarter q reads the three aligned words that cover values 8 q .. 8 q + 7 of block 2 w + s of its row's segment
+// and dequantises them exactly as minfer_dequant_q8_0 does (dequant8_shifted; block 2 w starts on a word boundary,
+// block 2 w + 1 two bytes past one), so the result is that of the fp16 kernels on the dequantised weight.
+constexpr int kQ8SegBytes = 272;
+constexpr int kQ8Stage = 22 * 1024;                            // 17 KiB of row segments, 3 KiB the extra copies land in; three stages hold the 64 KiB of partial sums
+template <int MB>
+__global__ __launch_bounds__(4 * 64) void gemm_stripe_q8_kernel(const GemmParams p) {
+    using T = F16;
+    using G = StripeGeom<MB>;
+    constexpr int WST = 3, XST = MB >= 3 ? 2 : 3, CW = 5, CX = 2 * MB;   // 90 / 114 / 114 / 130 KiB
+    static_assert(WST * kQ8Stage >= 4 * 4 * MB * 64 * 16, "the partial sums reuse the weight stages");
+    __shared__ __attribute__((aligned(16))) char w_lds[WST][kQ8Stage];
+    __shared__ __attribute__((aligned(16))) char x_lds[XST][G::X_BYTES];
+    const int lane = threadIdx.x & 63, w = wave_id();
+    const int l16 = lane & 15, quad = lane >> 4;
+    const int nseg = p.K / kStripeSeg;
+    const int blk_first = (int)((int64_t)blockIdx.x * p.tiles_n / (int)gridDim.x);
+    const int blk_last = (int)((int64_t)(blockIdx.x + 1) * p.tiles_n / (int)gridDim.x);
+    // x fragments as in gemm_stripe_kernel; weight fragment of (column block c, k step s): three words at
+    // 272 (16 c + l16) + 68 w + 32 s + 8 quad, the block's scale two bytes further for s = 1
+    const int row_off = (l16 >> 1) * kStripeBlock + 16 * (l16 & 1);
+    int frag[2];
+#pragma unroll
+    for (int s = 0; s < 2; ++s) frag[s] = row_off + 32 * ((4 * (2 * w + s) + quad) ^ (l16 >> 1));
+    const int wfrag = kQ8SegBytes * l16 + 68 * w + 8 * quad;
+    for (int cb = blk_first; cb < blk_last;) {
+    const int nb = min(4, blk_last - cb);
+    const int N = min(p.N, 16 * (cb + nb));                    // rows past the chunk are not this chunk's
+    const char* wsrc[CW];
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+        const int pc = min(64 * (w + 4 * i) + lane, 64 * 17 - 1), row = pc / 17;
+        wsrc[i] = (const char*)p.B + (int64_t)min(16 * cb + row, N - 1) * p.ldb + 16 * (pc - 17 * row);
+    }
+    const short* xsrc[CX];
+#pragma unroll
+    for (int j = 0; j < CX; ++j)
+        xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * ((lane >> 1) ^ ((w + 4 * j) & 7));
+    const int rot = (int)((unsigned)(cb >> 2) % (unsigned)nseg);
+    auto seg_of = [&](int t) { const int sg = t + rot; return sg >= nseg ? sg - nseg : sg; };
+    auto issue_w = [&](int t) {
+        char* st = w_lds[t % WST];
+        const int off = seg_of(t) * kQ8SegBytes;
+#pragma unroll
+        for (int i = 0; i < CW; ++i) copy16_global_to_lds(wsrc[i] + off, st + 1024 * (w + 4 * i));
+    };
+    auto issue_x = [&](int t) {
+        char* st = x_lds[t % XST];
+        const int k0 = seg_of(t) * kStripeSeg;
+#pragma unroll
+        for (int j = 0; j < CX; ++j) copy16_global_to_lds(xsrc[j] + k0, st + (w + 4 * j) * kStripeBlock);
+    };
+    f32x4 acc[4][MB];
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) acc[c][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int t = 0; t < WST - 1; ++t) {
+        if (t < XST - 1 && t < nseg) issue_x(t);
+        if (t < nseg) issue_w(t);
+    }
+    for (int t = 0; t < nseg; ++t) {
+        __syncthreads();                                       // every wave has read segment t - 1: its stages may be refilled
+        if (t + XST - 1 < nseg) issue_x(t + XST - 1);
+        if (t + WST - 1 < nseg) issue_w(t + WST - 1);
+        const int after = nseg - 1 - t;
+        if (after >= 2) wait_vmcnt<(WST - 1) * CW + (XST - 1) * CX>(); else if (after == 1) wait_vmcnt<CW + CX>(); else wait_vmcnt<0>();
+        __syncthreads();                                       // ... for every wave's copies
+        const char* wb = w_lds[t % WST] + wfrag;
+        const char* xb = x_lds[t % XST];
+        uint32_t wq[2][4][3], dbits[2][4];
+        s16x8 b[2][MB];
+#pragma unroll
+        for (int s = 0; s < 2; ++s) {
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) b[s][mb] = *reinterpret_cast<const s16x8*>(xb + mb * 8 * kStripeBlock + frag[s]);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint32_t* wp = reinterpret_cast<const uint32_t*>(wb + 16 * kQ8SegBytes * c + 32 * s);
+                wq[s][c][0] = wp[0]; wq[s][c][1] = wp[1]; wq[s][c][2] = wp[2];
+                dbits[s][c] = *reinterpret_cast<const uint16_t*>(wb + 16 * kQ8SegBytes * c + 34 * s - 8 * quad);
+            }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int s = 0; s < 2; ++s)
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const _Float16 dh = __builtin_bit_cast(_Float16, (uint16_t)dbits[s][c]);
+                const s16x8 a = dequant8_shifted(wq[s][c][0], wq[s][c][1], wq[s][c][2], s == 0 ? kQ8SelEven : kQ8SelOdd, h16x2{dh, dh});
+#pragma unroll
+                for (int mb = 0; mb < MB; ++mb) acc[c][mb] = T::mfma16(a, b[s][mb], acc[c][mb]);
+            }
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");     // fragments in registers before the barrier that frees the stage
+    }
+    __syncthreads();
+    f32x4* red = reinterpret_cast<f32x4*>(&w_lds[0][0]);   // 16 MB KiB of the 66
+#pragma unroll
+    for (int c = 0; c < 4; ++c)
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb) red[((w * 4 + c) * MB + mb) * 64 + lane] = acc[c][mb];
+    __syncthreads();
+    const int n = 16 * cb + 16 * w + 4 * quad;               // register r of a lane: weight row n + r, activation row 16mb + l16
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) {
+        const int m = 16 * mb + l16;
+        if (m >= p.M || n >= N) continue;
+        f32x4 sum = red[((0 * 4 + w) * MB + mb) * 64 + lane];
+#pragma unroll
+        for (int u = 1; u < 4; ++u) sum += red[((u * 4 + w) * MB + mb) * 64 + lane];
+        float v[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
+        if (p.beta != 0.f) {
+            const s16x4 c = *reinterpret_cast<const s16x4*>((const short*)p.C + (int64_t)m * p.ldc + n);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+        }
+        uint2 pk;
+        pk.x = T::pack2(v[0], v[1]);
+        pk.y = T::pack2(v[2], v[3]);
+        *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
+    }
+    cb += nb;
+    if (cb < blk_last) __syncthreads();
+    }
+}
+// Which calls it takes: 2-64 rows, whole segments of 8 blocks, rows that start on 16-byte boundaries, and a weight wide
+// enough for three blocks per workgroup, or two from 16 rows, or one and a half above 32 (weights coming from memory:
+// 14336 x 4096 at 2-16 rows 16.7-16.9 us against 20.8-26.8 for gemm_skinny_q8_kernel, 64 rows 23.4 against 50.9; 28672 x
+// 4096 29.7-43.4 against 36.8-97.7; 8192 x 8192 at 2 rows 27.0 against 23.5, at 16 rows 27.4 against 28.4; 6144 x 4096 at
+// 16 rows 15.7 against 15.2, at 64 rows 22.9 against 25.9).  A chunk of fewer than four blocks dequantises and multiplies
+// all four all the same: skipping the missing ones by a branch cost the full chunks a third (16.7 -> 22.8 us).
+static bool q8_stripe_ok(int64_t M, int64_t N, int64_t K, const void* Bq, int64_t row_bytes) {
+    return M >= 2 && M <= 64 && K % kStripeSeg == 0 && aligned16(Bq) && row_bytes % 16 == 0 &&
+           (N >= 12288 || (N >= 8192 && M >= 16) || (N >= 6144 && M > 32));
+}
+static int launch_stripe_q8(const GemmParams& p0, hipStream_t stream) {
+    GemmParams p = p0;
+    p.tiles_n = (p.N + 15) / 16;
+    const dim3 grid(std::min(p.tiles_n, 256)), block(4 * 64);
+    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_q8_kernel<1>), grid, block, 0, stream, p);
+    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_q8_kernel<2>), grid, block, 0, stream, p);
+    else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_q8_kernel<3>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_stripe_q8_kernel<4>), grid, block, 0, stream, p);
+    return check_launch("gemm_stripe_q8_kernel");
+}
+
 // Any shape and alignment: one thread per element of D, fp32 accumulation.  Small or odd problems only.
 template <class T, bool NT>
 __global__ __launch_bounds__(256) void gemm_plain_kernel(const GemmParams p) {
@@ -1457,6 +1614,7 @@ MINFER_ATTN_EXPORT int minfer_gemm_q8_0(const void* A, const void* Bq, const voi
         p.A = A; p.B = Bq; p.C = beta != 0.0 ? C : nullptr; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
         p.lda = lda; p.ldb = row_bytes; p.ldc = ldc; p.ldd = ldd; p.alpha = (float)alpha; p.beta = (float)beta;
         if (q8_gemv_ok(M, K, Bq, row_bytes)) return launch_gemv_q8(p, stream);
+        if (q8_stripe_ok(M, N, K, Bq, row_bytes)) return launch_stripe_q8(p, stream);
         return launch_skinny_q8(p, stream);
     }
     // otherwise: the weight as fp16 in the workspace, then the fp16 kernels on it

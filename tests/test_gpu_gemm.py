@@ -336,6 +336,13 @@ def make_q8(M, N, K, seed):
     (1, 4096, 16384, 1.0, 0.0),      # the longest activation row its LDS area holds
     (1, 512, 16640, 1.0, 0.0),       # longer: back to the 16-rows-per-instruction kernel
     (2, 2052, 768, 0.5, 1.0),        # two rows: that kernel as well
+    # 2-64 rows with K a multiple of 256: the stripe kernel over the raw blocks (16-column blocks shared out, chunks of four)
+    (9, 12296, 256, 1.0, 1.0),       # 769 blocks over 256 workgroups, the last one half empty; one segment
+    (33, 6152, 1024, 2.0, 3.0),      # from 33 rows on narrower weights too; three blocks of rows, chunks of one and two blocks
+    (48, 12288, 2560, 1.0, 0.0),     # ten segments
+    (64, 12304, 512, 0.5, 1.0),      # chunks of four and of three blocks
+    (16, 8192, 4096, 1.0, 0.0),      # two blocks per workgroup
+    (2, 14336, 4096, 1.0, 0.0),
 ])
 def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
     a, wq, c, w_deq = make_q8(M, N, K, seed=M * 7 + N + K)
