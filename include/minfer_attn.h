@@ -209,8 +209,8 @@ int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const voi
  * prefill chunk) has too few output tiles to occupy the chip; given minfer_gemm_workspace_bytes(M, N, K) bytes of
  * device memory (16-byte aligned; 0 = this shape does not use any), the K dimension is cut into slices that run as
  * separate workgroups and meet in the workspace as fp32 partial sums, which a second kernel adds up (alpha, beta and
- * C applied there, one rounding): slices of the 128 x 128 tiles, or, for up to 64 rows against an [N, K] weight of
- * fewer than 12288 columns, of 64-column stripes.  With a null workspace the call is minfer_gemm; a workspace smaller
+ * C applied there, one rounding): slices of the 128 x 128 tiles, or, for 9-64 rows against an [N, K] weight of fewer
+ * than 6144 columns and 33-64 rows against one of fewer than 12288, of 64-column stripes.  With a null workspace the call is minfer_gemm; a workspace smaller
  * than minfer_gemm_workspace_bytes is used only by a path whose slices fit in it.  No counterpart in the
  * reference, whose gemm_cuda takes no scratch memory (reference: gemm/op.cuh:218-316); same contract for the
  * workspace as the attention entry points (contents need not be initialised; one per stream).
