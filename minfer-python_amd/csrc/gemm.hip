@@ -550,26 +550,32 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
     // whatever the number of columns (448 stripes of 64 columns are one and three quarter rounds of 256 workgroups:
     // 28672 x 4096 from memory 46.5 -> 41.5-42.3 us), and a narrow weight is spread over the whole chip (6144 x 4096 at
     // 9-16 rows: 96 stripes 15.2-15.9 us, 256 workgroups of one or two blocks 12.3-12.7).
-    // (GROUPED: one workgroup per stripe of 64 columns, the stripes of the weights numbered through, as SLICED has one per
-    // stripe and slice: with the lookup of the chunk's weight inside the chunk loop the grouped launch ran 20 us where the
-    // plain one ran 11, for the same instructions and the same memory traffic)
-    const int blk_first = SLICED ? 4 * ((int)blockIdx.x / p.splits) : GROUPED ? 0 : (int)((int64_t)blockIdx.x * p.tiles_n / (int)gridDim.x);
-    const int blk_last = SLICED ? min(blk_first + 4, p.tiles_n) : GROUPED ? 1 : (int)((int64_t)(blockIdx.x + 1) * p.tiles_n / (int)gridDim.x);
+    // GROUPED: every weight has a run of workgroups of its own (p.grp.end counts them, cumulatively; the host hands them
+    // out in proportion to the weights' blocks), and a workgroup's share is worked out inside its weight, once, before the
+    // chunk loop: with the lookup of a chunk's weight inside the loop the grouped launch ran 20 us where the plain one ran
+    // 11, for the same instructions and the same L2 traffic.
+    int blk_first = SLICED ? 4 * ((int)blockIdx.x / p.splits) : (int)((int64_t)blockIdx.x * p.tiles_n / (int)gridDim.x);
+    int blk_last = SLICED ? min(blk_first + 4, p.tiles_n) : (int)((int64_t)(blockIdx.x + 1) * p.tiles_n / (int)gridDim.x);
     const short* Bg = (const short*)p.B;
     short* Dg = (short*)p.D;
-    int Nw = p.N, grp_local = 0;
+    int Nw = p.N;
     int64_t ldb = p.ldb, ldd = p.ldd;
-    if (GROUPED) {   // the stripe's weight, output and place inside them (uniform)
-        const int sg = group_of_unit(p.grp, (int)blockIdx.x, grp_local);
+    if (GROUPED) {   // the workgroup's weight, output and place among that weight's workgroups (uniform)
+        int idx;
+        const int sg = group_of_unit(p.grp, (int)blockIdx.x, idx);
         Bg = (const short*)(sg == 0 ? p.grp.B[0] : sg == 1 ? p.grp.B[1] : p.grp.B[2]);
         Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
         Nw = sg == 0 ? p.grp.N[0] : sg == 1 ? p.grp.N[1] : p.grp.N[2];
         ldb = sg == 0 ? p.grp.ldb[0] : sg == 1 ? p.grp.ldb[1] : p.grp.ldb[2];
         ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
+        const int wgs = (sg == 0 ? p.grp.end[0] : sg == 1 ? p.grp.end[1] - p.grp.end[0] : p.grp.end[2] - p.grp.end[1]);
+        const int blocks = (Nw + 15) / 16;
+        blk_first = (int)((int64_t)idx * blocks / wgs);
+        blk_last = (int)((int64_t)(idx + 1) * blocks / wgs);
     }
     for (int cb = blk_first; cb < blk_last;) {
-    const int local = GROUPED ? 4 * grp_local : cb;
-    const int nb = GROUPED ? 4 : min(4, blk_last - cb);
+    const int local = cb;
+    const int nb = min(4, blk_last - cb);
     int N = Nw;
     N = min(N, 16 * (local + nb));                             // rows past the chunk are not this chunk's
     const int n0 = 16 * local + 16 * w;                        // the columns this wave copies and, at the end, writes
@@ -681,7 +687,7 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_kernel(const GemmParams p)
         pk.y = T::pack2(v[2], v[3]);
         *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
     }
-    cb += GROUPED ? 1 : nb;
+    cb += nb;
     if (cb < blk_last) __syncthreads();                        // the sums have been read: the next chunk's copies may land there
     }
 }
@@ -695,12 +701,12 @@ static bool stripe_takes(int64_t M, int64_t stripes, int64_t K) {
     if (stripes > 640) return M >= 5;
     return stripes >= 96 || (stripes >= 80 && M >= 8) || (stripes >= 64 && M >= 32);
 }
-// `blocks`: 16-column blocks in all (GROUPED: stripes of 64 columns in all, p.grp.end counting them per weight).
+// `blocks`: 16-column blocks in all (GROUPED: workgroups in all, p.grp.end counting them per weight).
 template <class T, bool SLICED = false, bool GROUPED = false>
 static int launch_stripe(const GemmParams& p0, int blocks, hipStream_t stream) {
     GemmParams p = p0;
     p.tiles_n = blocks;
-    const dim3 grid(SLICED ? (blocks + 3) / 4 * p.splits : GROUPED ? blocks : std::min(blocks, 256)), block(4 * 64);   // (GROUPED: `blocks` counts stripes)
+    const dim3 grid(SLICED ? (blocks + 3) / 4 * p.splits : GROUPED ? blocks : std::min(blocks, 256)), block(4 * 64);   // (GROUPED: `blocks` is the number of workgroups)
     if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_kernel<T, 1, SLICED, GROUPED>), grid, block, 0, stream, p);
     else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_kernel<T, 2, SLICED, GROUPED>), grid, block, 0, stream, p);
     else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_kernel<T, 3, SLICED, GROUPED>), grid, block, 0, stream, p);
@@ -1396,12 +1402,27 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
         for (int s = 0; s < kMaxGroup; ++s) { if (s < n_w) acc += p.grp.N[s]; p.grp.end[s] = acc; }
         return launch_gemv<T, true>(p, (int)n_sum, stream);
     }
-    // a batch of decode steps: 64-column stripes over the three weights from 9 rows on (4096 + 1024 + 1024 columns of 4096
-    // values, weights coming from memory: 16 rows 15.8 us against 17.4 for the 16-column kernel, 32 rows 18.2 against 21.5)
+    // a batch of decode steps: the stripe kernel over the three weights from 5 rows on (4096 + 1024 + 1024 columns of 4096
+    // values, weights coming from memory: 8 rows 12.3 us against 14.2 for the 16-column kernel, 16 rows 12.7 against 17.4,
+    // 32 rows 15.6 against 21.5; up to 4 rows both take 12.1-12.6)
     {
         int64_t stripes = 0;
         for (int s = 0; s < n_w; ++s) stripes += (p.grp.N[s] + 63) / 64;
-        if (p.M >= 9 && stripes <= 640 && stripe_takes(p.M, stripes, p.K)) return launch_stripe<T, false, true>(p, fill_ends(64), stream);
+        if (p.M >= 5 && stripes <= 640 && stripe_takes(p.M, stripes, p.K)) {
+            // every weight a run of workgroups in proportion to its 16-column blocks, 256 or nearly in all
+            int64_t blocks = 0;
+            for (int s = 0; s < n_w; ++s) blocks += (p.grp.N[s] + 15) / 16;
+            const int64_t total = std::min<int64_t>(blocks, 256);
+            int acc = 0;
+            for (int s = 0; s < kMaxGroup; ++s) {
+                if (s < n_w) {
+                    const int64_t bs = (p.grp.N[s] + 15) / 16;
+                    acc += (int)std::max<int64_t>(1, std::min<int64_t>(bs, total * bs / blocks));
+                }
+                p.grp.end[s] = acc;
+            }
+            return launch_stripe<T, false, true>(p, acc, stream);
+        }
     }
     if (rows_lds_takes(p.M, p.K)) return launch_rows_lds<T, true>(p, fill_ends(16), stream);
     if (p.M <= 32 || (p.M <= 64 && n_sum * p.K <= (INT64_C(1) << 25))) {

@@ -170,8 +170,9 @@ def test_gemm_op_reference_test_recipe(kerns, S, alpha, beta):
     (24, 1024, 5120, 1280, 1288),      # few rows, two column groups per workgroup, a ragged last group
     (64, 512, 768, 256, 256),          # few-row kernel at its largest row count
     (33, 50, 17, 17, 9),               # nothing tileable: three plain launches
-    # 4-64 rows, K a multiple of 256, 96 stripes of 64 columns or more over the three weights: the stripe kernel, numbered through
-    (4, 4096, 4096, 1024, 1024),
+    # 5-64 rows, K a multiple of 256, 96 stripes of 64 columns or more over the three weights: the stripe kernel, every weight
+    # with workgroups of its own in proportion to its width
+    (5, 4096, 4096, 1024, 1024),
     (16, 512, 4096, 1024, 1032),       # a last stripe of 8 columns in the third weight
     (40, 1024, 4104, 1024, 1024),      # ... in the first; three blocks of activation rows
     (64, 256, 5120, 520, 8),           # one segment; a weight of a single partial stripe
