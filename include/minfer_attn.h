@@ -209,9 +209,11 @@ int minfer_gemm(int dtype, int b_layout, const void* A, const void* B, const voi
  * prefill chunk) has too few output tiles to occupy the chip; given minfer_gemm_workspace_bytes(M, N, K) bytes of
  * device memory (16-byte aligned; 0 = this shape does not use any), the K dimension is cut into slices that run as
  * separate workgroups and meet in the workspace as fp32 partial sums, which a second kernel adds up (alpha, beta and
- * C applied there, one rounding): slices of the 128 x 128 tiles, or, for 9-64 rows against an [N, K] weight of fewer
- * than 6144 columns and 33-64 rows against one of fewer than 12288, of 64-column stripes.  With a null workspace the call is minfer_gemm; a workspace smaller
- * than minfer_gemm_workspace_bytes is used only by a path whose slices fit in it.  No counterpart in the
+ * C applied there, one rounding): slices of the 128 x 128 tiles, or, up to 64 rows against an [N, K] weight of fewer
+ * than 12288 columns, of 64-column stripes (where two launches pay: from 9 rows on below 6144 columns, from 2 on rows
+ * of 8192 values and more of at most 1536 columns, from 33 between 6144 and 12288 columns).  With a null workspace the
+ * call is minfer_gemm; a workspace smaller than minfer_gemm_workspace_bytes is used only by a path whose slices fit
+ * in it.  No counterpart in the
  * reference, whose gemm_cuda takes no scratch memory (reference: gemm/op.cuh:218-316); same contract for the
  * workspace as the attention entry points (contents need not be initialised; one per stream).
  */
@@ -226,8 +228,11 @@ int minfer_gemm_ws(int dtype, int b_layout, const void* A, const void* B, const 
  * minfer_dequant_q8_0 does, fp16 A, C and D, fp32 accumulation, one rounding: the result is that of minfer_gemm
  * (MINFER_GEMM_B_NK) on the dequantised weight, element for element up to the order of the fp32 sums.  Up to 64 rows of A
  * and an even number of blocks per weight row, a kernel streams the blocks once (34 bytes per 32 weights instead of
- * 64: the projections of a decode step) and no workspace is needed; other shapes dequantise the weight into the
- * workspace (minfer_gemm_q8_0_workspace_bytes) and run the fp16 kernels on it.  This is the case the reference's
+ * 64: the projections of a decode step) and no workspace is needed; for 2-64 rows against fewer than 12288 columns
+ * minfer_gemm_q8_0_workspace_bytes still names one, for K slices as in minfer_gemm_ws (fp32 partial sums, a second
+ * launch), which the call uses when it is given in full and does without otherwise.  Other shapes dequantise the
+ * weight into the workspace and run the fp16 kernels on it: for them a missing or too small workspace is
+ * MINFER_ATTN_EWORKSPACE.  This is the case the reference's
  * gemm_cuda routes to dispatch_quant_abt, whose body is empty (reference: gemm/op.cuh:199-210, 299-312); block format
  * common/types.hpp:141-146, dequantisation cuda/quants/impls.cuh:121-143.
  */

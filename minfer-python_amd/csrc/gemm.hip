@@ -1116,7 +1116,9 @@ static int launch_skinny_q8(const GemmParams& p, hipStream_t stream) {
 // block 2 w + 1 two bytes past one), so the result is that of the fp16 kernels on the dequantised weight.
 constexpr int kQ8SegBytes = 272;
 constexpr int kQ8Stage = 22 * 1024;                            // 17 KiB of row segments, 3 KiB the extra copies land in; three stages hold the 64 KiB of partial sums
-template <int MB>
+// SLICED: p.splits workgroups per chunk of four blocks, each over its share of the segments; raw fp32 sums into p.part
+// ([slice][M][N]) for gemm_reduce_kernel (a narrow weight with a workspace, as gemm_stripe_kernel has it).
+template <int MB, bool SLICED = false>
 __global__ __launch_bounds__(4 * 64) void gemm_stripe_q8_kernel(const GemmParams p) {
     using T = F16;
     using G = StripeGeom<MB>;
@@ -1126,9 +1128,14 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_q8_kernel(const GemmParams
     __shared__ __attribute__((aligned(16))) char x_lds[XST][G::X_BYTES];
     const int lane = threadIdx.x & 63, w = wave_id();
     const int l16 = lane & 15, quad = lane >> 4;
-    const int nseg = p.K / kStripeSeg;
-    const int blk_first = (int)((int64_t)blockIdx.x * p.tiles_n / (int)gridDim.x);
-    const int blk_last = (int)((int64_t)(blockIdx.x + 1) * p.tiles_n / (int)gridDim.x);
+    int slice = 0, seg0 = 0, nseg = p.K / kStripeSeg;
+    if (SLICED) {
+        slice = (int)blockIdx.x % p.splits;
+        seg0 = slice * nseg / p.splits;
+        nseg = (slice + 1) * nseg / p.splits - seg0;
+    }
+    const int blk_first = SLICED ? 4 * ((int)blockIdx.x / p.splits) : (int)((int64_t)blockIdx.x * p.tiles_n / (int)gridDim.x);
+    const int blk_last = SLICED ? min(blk_first + 4, p.tiles_n) : (int)((int64_t)(blockIdx.x + 1) * p.tiles_n / (int)gridDim.x);
     // x fragments as in gemm_stripe_kernel; weight fragment of (column block c, k step s): three words at
     // 272 (16 c + l16) + 68 w + 32 s + 8 quad, the block's scale two bytes further for s = 1
     const int row_off = (l16 >> 1) * kStripeBlock + 16 * (l16 & 1);
@@ -1149,8 +1156,8 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_q8_kernel(const GemmParams
 #pragma unroll
     for (int j = 0; j < CX; ++j)
         xsrc[j] = (const short*)p.A + (int64_t)min(2 * (w + 4 * j) + (lane & 1), p.M - 1) * p.lda + 8 * ((lane >> 1) ^ ((w + 4 * j) & 7));
-    const int rot = (int)((unsigned)(cb >> 2) % (unsigned)nseg);
-    auto seg_of = [&](int t) { const int sg = t + rot; return sg >= nseg ? sg - nseg : sg; };
+    const int rot = (int)((SLICED ? blockIdx.x : (unsigned)(cb >> 2)) % (unsigned)nseg);
+    auto seg_of = [&](int t) { const int sg = t + rot; return seg0 + (sg >= nseg ? sg - nseg : sg); };
     auto issue_w = [&](int t) {
         char* st = w_lds[t % WST];
         const int off = seg_of(t) * kQ8SegBytes;
@@ -1222,6 +1229,10 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_q8_kernel(const GemmParams
         f32x4 sum = red[((0 * 4 + w) * MB + mb) * 64 + lane];
 #pragma unroll
         for (int u = 1; u < 4; ++u) sum += red[((u * 4 + w) * MB + mb) * 64 + lane];
+        if (SLICED) {
+            *reinterpret_cast<f32x4*>(p.part + ((int64_t)slice * p.M + m) * p.N + n) = sum;
+            continue;
+        }
         float v[4];
 #pragma unroll
         for (int e = 0; e < 4; ++e) v[e] = p.alpha * sum[e];
@@ -1240,23 +1251,36 @@ __global__ __launch_bounds__(4 * 64) void gemm_stripe_q8_kernel(const GemmParams
     }
 }
 // Which calls it takes: 2-64 rows, whole segments of 8 blocks, rows that start on 16-byte boundaries, and a weight wide
-// enough for three blocks per workgroup, or two from 16 rows, or one and a half above 32 (weights coming from memory:
+// enough for two and a half blocks per workgroup, or two from 16 rows, or one and a half above 32 (weights coming from memory:
 // 14336 x 4096 at 2-16 rows 16.7-16.9 us against 20.8-26.8 for gemm_skinny_q8_kernel, 64 rows 23.4 against 50.9; 28672 x
 // 4096 29.7-43.4 against 36.8-97.7; 8192 x 8192 at 2 rows 27.0 against 23.5, at 16 rows 27.4 against 28.4; 6144 x 4096 at
 // 16 rows 15.7 against 15.2, at 64 rows 22.9 against 25.9).  A chunk of fewer than four blocks dequantises and multiplies
 // all four all the same: skipping the missing ones by a branch cost the full chunks a third (16.7 -> 22.8 us).
+// K slices of it for a weight of fewer than 192 stripes when a workspace is given (1 = none): 256 / stripes workgroups
+// per chunk of four blocks, full chunks whatever the width (weights coming from memory: 4096 x 14336 at 16 / 32 / 64 rows
+// 19.0 / 21.8 / 26.4 us against 29.6 / 43.0 / 68.4 for gemm_skinny_q8_kernel, 8192 x 8192 at 2-64 rows 19.6-28.5 against
+// 23.7-40.3, 6144 x 4096 12.4-17.7 against 12.7-22.2; 4096 x 4096 up to 8 rows 10.2 against 7.7-8.3: two launches, so a
+// weight of 16 M values or fewer only from 16 rows on, or from 8 when its rows are 6144 values and longer, or from 2
+// when they are 8192 values and longer and the stripes 24 at most, as for the 16-bit weights).
+static int q8_slices(int64_t M, int64_t N, int64_t K) {
+    if (M < 2 || M > 64 || K % kStripeSeg != 0 || N % 8 != 0) return 1;
+    const bool long_rows = (K >= 6144 && M >= 8) || (K >= 8192 && N <= 24 * 64);
+    if (N * K <= (INT64_C(1) << 24) && M < 16 && !long_rows) return 1;
+    return stripe_slices(M, N, K);
+}
 static bool q8_stripe_ok(int64_t M, int64_t N, int64_t K, const void* Bq, int64_t row_bytes) {
     return M >= 2 && M <= 64 && K % kStripeSeg == 0 && aligned16(Bq) && row_bytes % 16 == 0 &&
-           (N >= 12288 || (N >= 8192 && M >= 16) || (N >= 6144 && M > 32));
+           (N >= 10240 || (N >= 8192 && M >= 16) || (N >= 6144 && M > 32));
 }
+template <bool SLICED = false>
 static int launch_stripe_q8(const GemmParams& p0, hipStream_t stream) {
     GemmParams p = p0;
     p.tiles_n = (p.N + 15) / 16;
-    const dim3 grid(std::min(p.tiles_n, 256)), block(4 * 64);
-    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_q8_kernel<1>), grid, block, 0, stream, p);
-    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_q8_kernel<2>), grid, block, 0, stream, p);
-    else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_q8_kernel<3>), grid, block, 0, stream, p);
-    else hipLaunchKernelGGL((gemm_stripe_q8_kernel<4>), grid, block, 0, stream, p);
+    const dim3 grid(SLICED ? (p.tiles_n + 3) / 4 * p.splits : std::min(p.tiles_n, 256)), block(4 * 64);
+    if (p.M <= 16) hipLaunchKernelGGL((gemm_stripe_q8_kernel<1, SLICED>), grid, block, 0, stream, p);
+    else if (p.M <= 32) hipLaunchKernelGGL((gemm_stripe_q8_kernel<2, SLICED>), grid, block, 0, stream, p);
+    else if (p.M <= 48) hipLaunchKernelGGL((gemm_stripe_q8_kernel<3, SLICED>), grid, block, 0, stream, p);
+    else hipLaunchKernelGGL((gemm_stripe_q8_kernel<4, SLICED>), grid, block, 0, stream, p);
     return check_launch("gemm_stripe_q8_kernel");
 }
 
@@ -1298,6 +1322,13 @@ __global__ __launch_bounds__(256) void gemm_reduce_kernel(const GemmParams p) {
         pk.y = T::pack2(v[2], v[3]);
         *reinterpret_cast<uint2*>((short*)p.D + (int64_t)m * p.ldd + n) = pk;
     }
+}
+
+static int launch_stripe_q8_slices(GemmParams& p, hipStream_t stream) {
+    if (int rc = launch_stripe_q8<true>(p, stream)) return rc;
+    const int grid = (int)std::min<int64_t>(((int64_t)p.M * (p.N / 4) + 255) / 256, 256 * 8);
+    hipLaunchKernelGGL((gemm_reduce_kernel<F16>), dim3(grid), dim3(256), 0, stream, p);
+    return check_launch("gemm_reduce_kernel");
 }
 
 // How many K slices a problem is cut into when a workspace is at hand: problems whose 128 x 128 tiles would leave most
@@ -1549,15 +1580,26 @@ static int gemm_impl(int dtype, int b_layout, const void* A, const void* B, cons
     // 2-8 rows: 23.5-24.4 us against 32.5 for the stripes' blocks shared out; 128256 x 4096 at 2-4 rows 166-170 against
     // 176-178; 28672 x 4096 at 2-8 rows 42.2-44.5 against 41.5-41.7 and 14336 x 4096 24.3-25.8 against 22.8-23.0: those go on)
     const bool rows_first = rows_takes && ((M <= 8 && stripes < 96) || (M <= 4 && stripes > 640));
-    if (fast && nt && rows_first)
+    const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
+    const bool sliceable = slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float);
+    // ... except long rows of a narrow weight when a workspace allows K slices: one wave per 16 columns walks a whole row
+    // by itself (1024 x 14336 at 2-8 rows 16.5-20.8 us, in slices 13.1-14.1; 1536 x 8960 15.2-17.4 and 11.8-12.5; 2048 x
+    // 8192 at 5-8 rows 12.5-13.4 and 12.5-12.6, at 2-4 rows and for rows of 6144 values no gain)
+    const bool long_rows_few_stripes = K >= 8192 && ((M >= 5 && stripes <= 32) || (M >= 2 && stripes <= 24));
+    if (fast && nt && rows_first && !(sliceable && long_rows_few_stripes))
         return dtype == MINFER_ATTN_F16 ? launch_rows_lds<F16>(p, (int)((N + 15) / 16), stream) : launch_rows_lds<BF16>(p, (int)((N + 15) / 16), stream);
     // with a workspace, K slices of the stripes: fewer than 96 stripes from 9 rows on (4096 x 14336 at 16 rows 24.5 us against
     // 29.1 for the 16-column kernel and 33 for the blocks shared out; 5120 x 5120 14.6 / 20.5 / 15.8), 96-191 stripes from 33
     // rows on (6144 x 4096 at 64 rows 18.6 against 20.2, 8192 x 8192 33.9 against 37.8; up to 32 rows the blocks shared out
-    // are ahead: 6144 x 4096 at 16 rows 12.7 against 14.3).  Two launches, so not for the smallest weights.
-    const int slices = fast && nt && workspace && aligned16(workspace) ? stripe_slices(M, N, K) : 1;
-    if (slices > 1 && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float) && (stripes < 96 ? M >= 9 : M > 32) &&
-        N * K >= (M >= 17 ? (INT64_C(1) << 24) : INT64_C(25000000))) {
+    // are ahead: 6144 x 4096 at 16 rows 12.7 against 14.3).  Two launches, 10.5 us at least, where one launch over rows of
+    // 4096 values takes 8-10 at 9-16 rows: up to 16 rows only for 25 M weight values or rows of 6144 values and more (2048 x
+    // 8192 at 9-16 rows 12.7-13.0 against 13.9-16.5, 1024 x 14336 13.7-14.6 against 21.5-26.7; 4096 x 4096 12.0 against
+    // 9.3-10.2), from 17 rows on for 8 M values where the other choice is gemm_skinny_kernel (2048 x 4096 at 24-64 rows
+    // 10.9-13.0 against 13.9-16.7, 4096 x 2048 at 24 rows 10.8 against 12.3) and 16 M where it is the blocks shared out
+    // (4096 x 2048 at 32 / 64 rows: 10.8 / 12.6 against 8.9 / 11.5).
+    const bool slices_pay = stripes >= 96 ? M > 32 && N * K >= (INT64_C(1) << 24)
+        : long_rows_few_stripes || (M >= 9 && (N * K >= INT64_C(25000000) || K >= 6144 || (M >= 17 && N * K >= (INT64_C(1) << (stripe_takes(M, stripes, K) ? 24 : 23)))));
+    if (sliceable && slices_pay) {
         p.splits = slices; p.part = (float*)workspace;
         return dtype == MINFER_ATTN_F16 ? launch_stripe_slices<F16>(p, stream) : launch_stripe_slices<BF16>(p, stream);
     }
@@ -1612,7 +1654,10 @@ static bool q8_stream_operands(const void* A, const void* C, const void* D, int6
 
 MINFER_ATTN_EXPORT size_t minfer_gemm_q8_0_workspace_bytes(int64_t M, int64_t N, int64_t K) {
     if (M <= 0 || N <= 0 || K <= 0 || K % 32 != 0 || M > 0x7fffffffLL || N > 0x7fffffffLL || K > 0x7fffffffLL) return 0;
-    if (q8_streams(M, N, K)) return 0;
+    if (q8_streams(M, N, K)) {   // optional: K slices of the stripe kernel for a narrow weight
+        const int slices = q8_slices(M, N, K);
+        return slices > 1 ? (size_t)slices * (size_t)M * (size_t)N * sizeof(float) : 0;
+    }
     return q8_dequant_bytes(N, K) + minfer_gemm_workspace_bytes(M, N, K);
 }
 
@@ -1635,6 +1680,11 @@ MINFER_ATTN_EXPORT int minfer_gemm_q8_0(const void* A, const void* Bq, const voi
         p.A = A; p.B = Bq; p.C = beta != 0.0 ? C : nullptr; p.D = D; p.M = (int)M; p.N = (int)N; p.K = (int)K;
         p.lda = lda; p.ldb = row_bytes; p.ldc = ldc; p.ldd = ldd; p.alpha = (float)alpha; p.beta = (float)beta;
         if (q8_gemv_ok(M, K, Bq, row_bytes)) return launch_gemv_q8(p, stream);
+        const int slices = aligned16(Bq) && row_bytes % 16 == 0 ? q8_slices(M, N, K) : 1;
+        if (slices > 1 && workspace && aligned16(workspace) && workspace_bytes >= (size_t)slices * (size_t)M * (size_t)N * sizeof(float)) {
+            p.splits = slices; p.part = (float*)workspace;
+            return launch_stripe_q8_slices(p, stream);
+        }
         if (q8_stripe_ok(M, N, K, Bq, row_bytes)) return launch_stripe_q8(p, stream);
         return launch_skinny_q8(p, stream);
     }

@@ -258,6 +258,9 @@ def test_qkv_op_and_reference_checks(kerns):
     (33, 8192, 2048, 0.5, 0.0),      # three blocks of activation rows, two slices of four segments
     (1, 8192, 4096, 1.0, 0.0),       # one row
     (64, 6144, 4096, 1.0, 1.0),
+    (12, 1024, 14336, 1.0, 0.0),     # long rows of a small weight: 16 stripes, 14 slices of 4 segments
+    (24, 2048, 4096, 2.0, 1.0),      # 8 M weight values from 17 rows on: 8 slices of 2 segments, two blocks of rows
+    (3, 1536, 8960, 1.0, 1.0),       # long rows, 24 stripes: slices from 2 rows on (10 slices of 3 or 4 segments)
 ])
 def test_gemm_k_slices_against_oracle(layout, dtype, M, N, K, alpha, beta):
     a, b, c = make(M, N, K, layout, dtype, seed=M + N + K)
@@ -344,6 +347,13 @@ def make_q8(M, N, K, seed):
     (64, 12304, 512, 0.5, 1.0),      # chunks of four and of three blocks
     (16, 8192, 4096, 1.0, 0.0),      # two blocks per workgroup
     (2, 14336, 4096, 1.0, 0.0),
+    # fewer than 192 stripes and a workspace: K slices of the stripe kernel, summed by a second launch
+    (16, 4096, 14336, 1.0, 1.0),     # 4 slices of 14 segments
+    (33, 5120, 5120, 2.0, 0.0),      # 3 slices of 7, 7 and 6 segments; three blocks of rows
+    (8, 8192, 8192, 1.0, 0.0),       # 2 slices
+    (64, 4104, 2048, 0.5, 1.0),      # 65 stripes, the last of 8 columns: 2 slices of 4 segments; a small weight, from 16 rows
+    (2, 6144, 4096, 1.0, 0.0),
+    (3, 1536, 8960, 1.0, 1.0),       # long rows, 24 stripes: 10 slices of 3 or 4 segments
 ])
 def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
     a, wq, c, w_deq = make_q8(M, N, K, seed=M * 7 + N + K)
@@ -351,15 +361,25 @@ def test_gemm_q8_0_weights_against_oracle(M, N, K, alpha, beta):
     da, dwq, dc = a.to(DEV), wq.to(DEV), c.to(DEV)
     d = torch.zeros(M, N, dtype=torch.float16, device=DEV)
     need = capi.lib().minfer_gemm_q8_0_workspace_bytes(M, N, K)
-    assert (need == 0) == (M <= 64 and (K // 32) % 2 == 0 and N % 4 == 0)
+    streams = M <= 64 and (K // 32) % 2 == 0 and N % 4 == 0      # the raw blocks are multiplied: a workspace only for K slices
+    assert streams or need > 0
+    if streams:
+        stripes = (N + 63) // 64
+        slices = min(256 // stripes, K // 1024, 16) if M >= 2 and K % 256 == 0 and N % 8 == 0 and stripes < 192 and (N * K > 1 << 24 or M >= 16 or (K >= 6144 and M >= 8) or (K >= 8192 and stripes <= 24)) else 1
+        assert need == (slices * M * N * 4 if slices > 1 else 0)
     ws = torch.full((max(need, 16),), 0xFF, dtype=torch.uint8, device=DEV)
     assert capi.gemm_q8_0(da, dwq, dc, d, alpha, beta, ws if need else None) == capi.OK, capi.last_error()
     assert_close(d, exact, torch.float16, "q8_0 weight")
+    if streams and need:            # the slices are optional: without the workspace, or with too small a one, one launch
+        for small in (None, ws[:need // 2]):
+            d.fill_(float("nan"))
+            assert capi.gemm_q8_0(da, dwq, dc, d, alpha, beta, small) == capi.OK, capi.last_error()
+            assert_close(d, exact, torch.float16, "q8_0 weight, no slices")
     # the same numbers as the fp16 kernel on the dequantised weight, up to the order of the fp32 sums
     d_ref = torch.zeros_like(d)
     assert capi.gemm(da, w_deq.to(DEV), dc, d_ref, alpha, beta, NK) == capi.OK, capi.last_error()
     assert_close(d_ref, exact, torch.float16, "fp16 kernel on the dequantised weight")
-    if need:
+    if not streams:
         assert capi.gemm_q8_0(da, dwq, dc, d, alpha, beta, None) == capi.EWORKSPACE and "workspace" in capi.last_error()
 
 
