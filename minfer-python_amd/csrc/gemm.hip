@@ -169,14 +169,20 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     const int kt_all = p.K / kBK;
     const int kt_first = SPLIT ? (int)((int64_t)slice * kt_all / p.splits) : 0;
     const int KT = SPLIT ? (int)((int64_t)(slice + 1) * kt_all / p.splits) - kt_first : kt_all;
-    auto issue = [&](int kt_rel, int stage) __attribute__((always_inline)) {
+    // copy c of a step (the wave's A copies, then its B copies) into a stage
+    auto copy_one = [&](int kt_rel, int stage, int c) __attribute__((always_inline)) {
         const int kt = kt_first + kt_rel;
-        const short* abase = Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK;
-        const short* bbase = NT ? Bg + (int64_t)n0 * ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * ldb + n0;
+        if (c < CA) {
+            copy16_global_to_lds(Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK, a_off[c], &a_lds[stage][a_dst[c]]);
+        } else {
+            const int j = c - CA;
+            const short* bbase = NT ? Bg + (int64_t)n0 * ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * ldb + n0;
+            copy16_global_to_lds(CONCAT ? b_src[CONCAT ? j : 0] + (int64_t)kt * kBK : bbase, b_off[j], &b_lds[stage][b_dst[j]]);
+        }
+    };
+    auto issue = [&](int kt_rel, int stage) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < CA; ++j) copy16_global_to_lds(abase, a_off[j], &a_lds[stage][a_dst[j]]);
-#pragma unroll
-        for (int j = 0; j < CB; ++j) copy16_global_to_lds(CONCAT ? b_src[CONCAT ? j : 0] + (int64_t)kt * kBK : bbase, b_off[j], &b_lds[stage][b_dst[j]]);
+        for (int c = 0; c < CA + CB; ++c) copy_one(kt_rel, stage, c);
     };
 
     // ---- per-lane LDS read addresses (stage 0; stage, sub-tile and block offsets are immediates) ---------
@@ -213,49 +219,81 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
 #pragma unroll
             for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.f;
 
-    auto load_frags = [&](auto stage_tag, int kk, s16x8 (&nf)[NB], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
+    // fragment r of slice kk of a stage: r < NB the n fragments (MFMA A operand), then the m fragments
+    auto read_one = [&](auto stage_tag, int kk, int r, s16x8 (&nf)[NB], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
         constexpr int AOFF = decltype(stage_tag)::value * SH::A_PANEL, BOFF = decltype(stage_tag)::value * SH::B_PANEL;
-#pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            if (NT) {
-                nf[nb] = lds_read_b128(n_rd[kk], BOFF + nb * (kRowTile / 2));
-            } else {
-                const s16x4 t0 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk) * 256);
-                const s16x4 t1 = lds_read_tr16(n_rd[nb], BOFF + (16 * kk + 4) * 256);
-                nf[nb] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
-            }
+        if (r >= NB) {
+            mf[r - NB] = lds_read_b128(m_rd[kk], AOFF + (r - NB) * (kRowTile / 2));
+        } else if (NT) {
+            nf[r] = lds_read_b128(n_rd[kk], BOFF + r * (kRowTile / 2));
+        } else {
+            const s16x4 t0 = lds_read_tr16(n_rd[r], BOFF + (16 * kk) * 256);
+            const s16x4 t1 = lds_read_tr16(n_rd[r], BOFF + (16 * kk + 4) * 256);
+            nf[r] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
         }
+    };
+    auto load_frags = [&](auto stage_tag, int kk, s16x8 (&nf)[NB], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb) mf[mb] = lds_read_b128(m_rd[kk], AOFF + mb * (kRowTile / 2));
+        for (int r = 0; r < NB + MB; ++r) read_one(stage_tag, kk, r, nf, mf);
     };
     // ---- main loop ---------------------------------------------------------------------------------------
-    // Fragments are double-buffered in registers: while the 8 (4) MFMAs of one 16-wide k slice run, the fragments
-    // of the next slice are read from LDS.  The workgroup's only barrier per K step sits between the third and
-    // the last slice: a wave arrives when it has read the last fragments of the current stage and its own share
-    // of the next stage's copy has landed; after the barrier it issues the copy of the step after next into the
-    // stage just vacated and reads the next step's first fragments, all of which overlaps with the last slice's
-    // MFMAs, so the matrix pipe does not drain at step boundaries.
+    // Fragments are double-buffered in registers: between the 8 (4, 6) MFMAs of one 16-wide k slice the fragments of
+    // the next slice are read from LDS, one read after each MFMA.  The workgroup's only barrier per K step sits
+    // before the last slice: a wave arrives when it has read the last fragments of the current stage and its own
+    // share of the next stage's copy has landed; between the last slice's MFMAs it then reads the next step's first
+    // fragments and issues the copy of the step after next into the stage just vacated, so the matrix pipe does not
+    // drain at step boundaries.  Every MFMA, read and copy is pinned where it is written (scheduling barriers): left
+    // alone the compiler moved a slice's reads behind the previous slice's MFMAs, where nothing of the wave covers
+    // their latency, and put all copies and reads of a step's end in front of its MFMAs (4096^3 139 -> 127 us).
     s16x8 nf[2][NB], mf[2][MB];
-    auto mfmas = [&](int buf) __attribute__((always_inline)) {
+    constexpr int NM = NB * MB, NR = NB + MB, NC = CA + CB;
+    auto pin = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
+    auto mfma_one = [&](int buf, int i) __attribute__((always_inline)) {
+        const int mb = i / NB, nb = i % NB;
+        acc[nb][mb] = T::mfma32(nf[buf][nb], mf[buf][mb], acc[nb][mb]);
+    };
+    // the MFMAs of the slice held in buffer `buf`, the fragments of slice kk_next of the stage read into the other one
+    auto k_slice = [&](auto stage_tag, int kk_next, int buf) __attribute__((always_inline)) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+        for (int i = 0; i < NM; ++i) {
+            mfma_one(buf, i);
+            pin();
 #pragma unroll
-            for (int nb = 0; nb < NB; ++nb) acc[nb][mb] = T::mfma32(nf[buf][nb], mf[buf][mb], acc[nb][mb]);
+            for (int r = (NR * i + NM - 1) / NM; r < (NR * (i + 1) + NM - 1) / NM; ++r) read_one(stage_tag, kk_next, r, nf[buf ^ 1], mf[buf ^ 1]);
+            pin();
+        }
+    };
+    // the last slice's MFMAs; between them the first fragments of the next stage (if there is a next step) and the
+    // copies of step kt + 2 into this stage (if there is one)
+    auto last_slice = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        const bool next = kt + 1 < KT, more = kt + 2 < KT;
+#pragma unroll
+        for (int i = 0; i < NM; ++i) {
+            mfma_one(1, i);
+            pin();
+            if (next) {
+#pragma unroll
+                for (int r = (NR * i + NM - 1) / NM; r < (NR * (i + 1) + NM - 1) / NM; ++r)
+                    read_one(std::integral_constant<int, STAGE ^ 1>{}, 0, r, nf[0], mf[0]);
+            }
+            if (more) {
+#pragma unroll
+                for (int c = (NC * i + NM - 1) / NM; c < (NC * (i + 1) + NM - 1) / NM; ++c) copy_one(kt + 2, STAGE, c);
+            }
+            pin();
+        }
     };
     auto step = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
-        constexpr int STAGE = decltype(stage_tag)::value;
-        load_frags(stage_tag, 1, nf[1], mf[1]);
-        mfmas(0);
-        load_frags(stage_tag, 2, nf[0], mf[0]);
-        mfmas(1);
-        load_frags(stage_tag, 3, nf[1], mf[1]);
-        mfmas(0);
+        pin();
+        k_slice(stage_tag, 1, 0);
+        k_slice(stage_tag, 2, 1);
+        k_slice(stage_tag, 3, 0);
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read everything it needs from this stage
         wait_vmcnt<0>();                                       // and its share of the next stage has landed
         __syncthreads();
-        if (kt + 2 < KT) issue(kt + 2, STAGE);
-        if (kt + 1 < KT) load_frags(std::integral_constant<int, STAGE ^ 1>{}, 0, nf[0], mf[0]);
-        mfmas(1);
+        pin();
+        last_slice(stage_tag, kt);
     };
     issue(0, 0);
     if (KT > 1) issue(1, 1);
