@@ -506,6 +506,17 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         // at the same speed and held 24 registers more).  The accumulators start from -reference (neg_ref, a register
         // block that changes only when the reference does), so the MFMA output is the exponent relative to the reference.
         f32x16 e_acc[2];
+        // V^T fragments of a 16-key chunk; the first two chunks are requested between the last MFMAs of S^T, where the K
+        // ring is no longer refilled: their latency hides behind those, the row maximum and the first exponentials
+        s16x8 va[2][DB];
+        auto load_v = [&](int c, s16x8 (&a)[DB]) __attribute__((always_inline)) {
+#pragma unroll
+            for (int db = 0; db < DB; ++db) {
+                const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (16 * c) * RB);
+                const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (16 * c + 8) * RB);
+                a[db] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
+            }
+        };
         {
             s16x8 kf[2][2][2];   // [buffer][chunk in buffer][key block]
             auto load_k = [&](int buf, int c0) __attribute__((always_inline)) {
@@ -517,6 +528,9 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
             };
             load_k(0, 0);
             load_k(1, 2);
+            __builtin_amdgcn_sched_barrier(0);
+            // (the scheduling barriers keep the refill where it is written, four chunks ahead of its use: left alone
+            // the compiler moved every pair of reads down to just before the MFMAs that use them)
 #pragma unroll
             for (int c0 = 0; c0 < KC; c0 += 2) {
                 const int buf = (c0 >> 1) & 1;
@@ -529,23 +543,17 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
                         e_acc[0] = T::mfma32(kf[buf][i][0], qf[c0 + i], e_acc[0]);
                         e_acc[1] = T::mfma32(kf[buf][i][1], qf[c0 + i], e_acc[1]);
                     }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (c0 + 4 < KC) {
+                        kf[buf][i][0] = lds_read_b128(k_rd[c0 + 4 + i], SOFF);
+                        kf[buf][i][1] = lds_read_b128(k_rd[c0 + 4 + i], SOFF + 32 * RB);
+                    } else if (c0 + 4 == KC) {
+                        load_v(i, va[i]);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                if (c0 + 4 < KC) load_k(buf, c0 + 4);
             }
         }
-        // first two chunks of V^T fragments: their latency hides behind the max and the first exponentials
-        s16x8 va[2][DB];
-        auto load_v = [&](int c, s16x8 (&a)[DB]) {
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (16 * c) * RB);
-                const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (16 * c + 8) * RB);
-                a[db] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
-            }
-        };
-        load_v(0, va[0]);
-        load_v(1, va[1]);
-        __builtin_amdgcn_sched_barrier(0);
 
         // ---- masking ----------------------------------------------------------------------
         // Register 4j + e of block kb is key key0 + 32kb + 8j + 4h + e.  The test by position (keys past the end of the

@@ -79,7 +79,7 @@ MA_DEV int group_of_unit(const GemmGroup& g, int c, int& local) {
 
 // swizzles: granule index of a row XORed with a function of the row (see the attention kernel's TileGeom)
 MA_DEV int swz_row_tile(int row) { return (row >> 1) & 7; }        // 128-byte rows, read 32 rows x 16 bytes
-MA_DEV int swz_col_tile(int row) { return (row & 3) << 2; }        // 256-byte rows, read 4 rows x 64 bytes (transposing)
+MA_DEV int swz_col_tile(int row) { return ((row & 3) << 2) | ((row >> 2) & 2); }   // 256-byte rows, transposing reads of 4 rows x 32 bytes by each of two 16-lane groups 8 rows apart
 
 // CONCAT (with GROUPED, [N, K] weights whose widths are multiples of 64): the weights' columns are numbered through as
 // one wide matrix and tiled without regard to where one weight ends, so a tile may hold columns of two weights; every
@@ -186,163 +186,156 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     };
 
     // ---- per-lane LDS read addresses (stage 0; stage, sub-tile and block offsets are immediates) ---------
-    // m fragments (MFMA B operand): tile row 32*MB*wm + 32*mb + l32, i.e. row 32*(mb&1) + l32 of sub-tile
-    // MB*wm/2 + (mb>>1), granule (2kk + h) ^ swizzle
-    uint32_t m_rd[4], n_rd[4];
+    // The matrix instruction is v_mfma_f32_16x16x32 (on random operands the chip sustains 1.86-1.90 PFLOP/s of it and
+    // 1.57-1.62 of v_mfma_f32_32x32x16, whose rate is what a power-bound GEMM then runs at).  A K step is two slices of
+    // 32 values; a fragment is 16 rows x 32 k, lane (l16, quad) holding row l16, k = 8 quad + 0..7 of the slice: 16 bytes
+    // at granule (4 slice + quad) ^ swizzle of the row.  A 16-row block is a quarter of a 64-row sub-tile; the swizzle of
+    // row 16 b + l16 does not depend on b.
+    constexpr int M16 = 2 * MB, N16 = 2 * NB, BLK = kRowTile / 4;
+    const int l16 = lane & 15, quad = lane >> 4;
+    uint32_t m_rd[2], n_rd[4];
     {
-        const int sw = swz_row_tile(l32);
+        const int sw = swz_row_tile(l16);
 #pragma unroll
-        for (int kk = 0; kk < 4; ++kk) {
-            const uint32_t o = l32 * 128 + 16 * ((2 * kk + h) ^ sw);
-            // (a 32-row block is half a 64-row sub-tile: block g of a panel starts g * kRowTile / 2 bytes into it)
-            m_rd[kk] = lds_addr(&a_lds[0][0]) + MB * wm * (kRowTile / 2) + o;
-            if (NT) n_rd[kk] = lds_addr(&b_lds[0][0]) + NB * wn * (kRowTile / 2) + o;    // n fragments: as the m fragments
+        for (int ks = 0; ks < 2; ++ks) {
+            const uint32_t o = l16 * 128 + 16 * ((4 * ks + quad) ^ sw);
+            m_rd[ks] = lds_addr(&a_lds[0][0]) + M16 * wm * BLK + o;
+            if (NT) n_rd[ks] = lds_addr(&b_lds[0][0]) + N16 * wn * BLK + o;    // n fragments: as the m fragments
         }
         if (!NT) {
-            // n fragments through transpose reads of the [k][n] sub-tile wn>>1: per 16-lane group 4 k rows x 16 columns
-            const int blk = lane >> 4, li = lane & 15;
-            const int krow = 8 * h + (li >> 2);   // lane half h contracts k = 16kk + 8h + 0..7, like the 16-byte reads of A
+            // n fragments through transpose reads of the [k][n] sub-tile: the 16-lane group `quad` addresses k rows
+            // 8 quad + 0..3 (second read: + 4) of the slice, 16 columns, and lane l16 receives column l16
+            static_assert(NT || N16 <= 4, "one read address per 16-column block");
+            const int krow = 8 * quad + (l16 >> 2);
             const int swv = swz_col_tile(krow);
 #pragma unroll
             for (int nb = 0; nb < 4; ++nb) {
-                const int n = 32 * (NB * wn + (nb < NB ? nb : 0)), col = (n & 127) + 16 * (blk & 1) + 4 * (li & 3);
+                const int n = 16 * (N16 * wn + (nb < N16 ? nb : 0)), col = (n & 127) + 4 * (l16 & 3);
                 n_rd[nb] = lds_addr(&b_lds[0][0]) + (n >> 7) * kColTile + krow * 256 + 16 * ((col >> 3) ^ swv) + 2 * (col & 7);
             }
         }
     }
 
-    f32x16 acc[NB][MB];
+    f32x4 acc[N16][M16];
 #pragma unroll
-    for (int nb = 0; nb < NB; ++nb)
+    for (int nb = 0; nb < N16; ++nb)
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[nb][mb][r] = 0.f;
+        for (int mb = 0; mb < M16; ++mb) acc[nb][mb] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // fragment r of slice kk of a stage: r < NB the n fragments (MFMA A operand), then the m fragments
-    auto read_one = [&](auto stage_tag, int kk, int r, s16x8 (&nf)[NB], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
-        constexpr int AOFF = decltype(stage_tag)::value * SH::A_PANEL, BOFF = decltype(stage_tag)::value * SH::B_PANEL;
-        if (r >= NB) {
-            mf[r - NB] = lds_read_b128(m_rd[kk], AOFF + (r - NB) * (kRowTile / 2));
-        } else if (NT) {
-            nf[r] = lds_read_b128(n_rd[kk], BOFF + r * (kRowTile / 2));
-        } else {
-            const s16x4 t0 = lds_read_tr16(n_rd[r], BOFF + (16 * kk) * 256);
-            const s16x4 t1 = lds_read_tr16(n_rd[r], BOFF + (16 * kk + 4) * 256);
-            nf[r] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
-        }
+    // n fragment nb / m fragment mb of slice ks of a stage
+    auto read_n = [&](auto stage_tag, int ks, int nb) __attribute__((always_inline)) -> s16x8 {
+        constexpr int BOFF = decltype(stage_tag)::value * SH::B_PANEL;
+        if (NT) return lds_read_b128(n_rd[ks], BOFF + nb * BLK);
+        const s16x4 t0 = lds_read_tr16(n_rd[nb], BOFF + (32 * ks) * 256);
+        const s16x4 t1 = lds_read_tr16(n_rd[nb], BOFF + (32 * ks + 4) * 256);
+        return s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
     };
-    auto load_frags = [&](auto stage_tag, int kk, s16x8 (&nf)[NB], s16x8 (&mf)[MB]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int r = 0; r < NB + MB; ++r) read_one(stage_tag, kk, r, nf, mf);
+    auto read_m = [&](auto stage_tag, int ks, int mb) __attribute__((always_inline)) -> s16x8 {
+        constexpr int AOFF = decltype(stage_tag)::value * SH::A_PANEL;
+        return lds_read_b128(m_rd[ks], AOFF + mb * BLK);
     };
     // ---- main loop ---------------------------------------------------------------------------------------
-    // Fragments are double-buffered in registers: between the 8 (4, 6) MFMAs of one 16-wide k slice the fragments of
-    // the next slice are read from LDS, one read after each MFMA.  The workgroup's only barrier per K step sits
-    // before the last slice: a wave arrives when it has read the last fragments of the current stage and its own
-    // share of the next stage's copy has landed; between the last slice's MFMAs it then reads the next step's first
-    // fragments and issues the copy of the step after next into the stage just vacated, so the matrix pipe does not
-    // drain at step boundaries.  Every MFMA, read and copy is pinned where it is written (scheduling barriers): left
-    // alone the compiler moved a slice's reads behind the previous slice's MFMAs, where nothing of the wave covers
-    // their latency, and put all copies and reads of a step's end in front of its MFMAs (4096^3 139 -> 127 us).
-    s16x8 nf[2][NB], mf[2][MB];
-    constexpr int NM = NB * MB, NR = NB + MB, NC = CA + CB;
+    // A slice is N16 groups of M16 MFMAs (group nb: n fragment nb against every m fragment).  The n fragments are
+    // double-buffered: the next slice's are read during groups 1 .. N16-2, one read after an MFMA; the m fragments have
+    // one buffer, refilled in the last group, fragment mb right after the last MFMA that uses it.  The workgroup's only
+    // barrier per K step sits after group 0 of the step's second slice: by then every read of the stage has returned
+    // (the last were issued a group earlier) and the wave's share of the next stage's copy, issued a whole step
+    // before, has landed; what follows the barrier reads the next stage and copies the step after next into the stage
+    // just vacated, one copy after an MFMA.  Every MFMA, read and copy is pinned where it is written (scheduling
+    // barriers): left alone the compiler moves reads down to just before their use, where nothing of the wave covers
+    // their latency.
+    s16x8 nf[2][N16], mf[M16];
+    constexpr int NC = CA + CB;
+    constexpr int MID = (N16 - 2) * M16;    // MFMAs of groups 1 .. N16-2
     auto pin = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
-    auto mfma_one = [&](int buf, int i) __attribute__((always_inline)) {
-        const int mb = i / NB, nb = i % NB;
-        acc[nb][mb] = T::mfma32(nf[buf][nb], mf[buf][mb], acc[nb][mb]);
-    };
-    // the MFMAs of the slice held in buffer `buf`, the fragments of slice kk_next of the stage read into the other one
-    auto k_slice = [&](auto stage_tag, int kk_next, int buf) __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            mfma_one(buf, i);
-            pin();
-#pragma unroll
-            for (int r = (NR * i + NM - 1) / NM; r < (NR * (i + 1) + NM - 1) / NM; ++r) read_one(stage_tag, kk_next, r, nf[buf ^ 1], mf[buf ^ 1]);
-            pin();
-        }
-    };
-    // the last slice's MFMAs; between them the first fragments of the next stage (if there is a next step) and the
-    // copies of step kt + 2 into this stage (if there is one)
-    auto last_slice = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
+    // one slice: MFMAs on nf[buf] and mf; `next_tag`/`ks_next` name the slice read meanwhile (has_next: there is one);
+    // SECOND: the step's second slice, with the barrier after group 0 and, if copy_kt >= 0, that step's copies after it
+    auto k_slice = [&](auto next_tag, int ks_next, int buf, bool has_next, auto second_tag, int copy_kt, auto stage_tag) __attribute__((always_inline)) {
+        constexpr bool SECOND = decltype(second_tag)::value;
         constexpr int STAGE = decltype(stage_tag)::value;
-        const bool next = kt + 1 < KT, more = kt + 2 < KT;
 #pragma unroll
-        for (int i = 0; i < NM; ++i) {
-            mfma_one(1, i);
-            pin();
-            if (next) {
+        for (int nb = 0; nb < N16; ++nb) {
 #pragma unroll
-                for (int r = (NR * i + NM - 1) / NM; r < (NR * (i + 1) + NM - 1) / NM; ++r)
-                    read_one(std::integral_constant<int, STAGE ^ 1>{}, 0, r, nf[0], mf[0]);
+            for (int mb = 0; mb < M16; ++mb) {
+                acc[nb][mb] = T::mfma16(nf[buf][nb], mf[mb], acc[nb][mb]);
+                pin();
+                if (nb >= 1 && nb <= N16 - 2) {
+                    const int i = (nb - 1) * M16 + mb;   // 0 .. MID-1
+                    if (has_next) {
+#pragma unroll
+                        for (int r = (N16 * i + MID - 1) / MID; r < (N16 * (i + 1) + MID - 1) / MID; ++r) nf[buf ^ 1][r] = read_n(next_tag, ks_next, r);
+                    }
+                    if (SECOND && copy_kt >= 0) {
+#pragma unroll
+                        for (int c = (NC * i + MID - 1) / MID; c < (NC * (i + 1) + MID - 1) / MID; ++c) copy_one(copy_kt, STAGE, c);
+                    }
+                } else if (nb == N16 - 1) {
+                    if (has_next) mf[mb] = read_m(next_tag, ks_next, mb);
+                }
+                pin();
             }
-            if (more) {
-#pragma unroll
-                for (int c = (NC * i + NM - 1) / NM; c < (NC * (i + 1) + NM - 1) / NM; ++c) copy_one(kt + 2, STAGE, c);
+            if (SECOND && nb == 0) {
+                asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read everything it needs from this stage
+                wait_vmcnt<0>();                                       // and its share of the next stage has landed
+                __syncthreads();
+                pin();
             }
-            pin();
         }
     };
     auto step = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
+        constexpr int STAGE = decltype(stage_tag)::value;
+        using Next = std::integral_constant<int, STAGE ^ 1>;
         pin();
-        k_slice(stage_tag, 1, 0);
-        k_slice(stage_tag, 2, 1);
-        k_slice(stage_tag, 3, 0);
-        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read everything it needs from this stage
-        wait_vmcnt<0>();                                       // and its share of the next stage has landed
-        __syncthreads();
-        pin();
-        last_slice(stage_tag, kt);
+        k_slice(stage_tag, 1, 0, true, std::false_type{}, -1, stage_tag);
+        k_slice(Next{}, 0, 1, kt + 1 < KT, std::true_type{}, kt + 2 < KT ? kt + 2 : -1, stage_tag);
     };
     issue(0, 0);
     if (KT > 1) issue(1, 1);
     if (KT > 1) wait_vmcnt<CA + CB>(); else wait_vmcnt<0>();   // the copies of step 0 retire first
     __syncthreads();
-    load_frags(std::integral_constant<int, 0>{}, 0, nf[0], mf[0]);
+#pragma unroll
+    for (int nb = 0; nb < N16; ++nb) nf[0][nb] = read_n(std::integral_constant<int, 0>{}, 0, nb);
+#pragma unroll
+    for (int mb = 0; mb < M16; ++mb) mf[mb] = read_m(std::integral_constant<int, 0>{}, 0, mb);
     for (int kt = 0; kt < KT; kt += 2) {
         step(std::integral_constant<int, 0>{}, kt);
         if (kt + 1 < KT) step(std::integral_constant<int, 1>{}, kt + 1);
     }
 
-    // ---- epilogue: D = alpha * acc + beta * C; register r of a block is n = 8(r/4) + 4h + r%4, m = l32 ----
+    // ---- epilogue: D = alpha * acc + beta * C; register e of a block is n = 4 quad + e, m = l16 ----
     const short* Cg = (const short*)p.C;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) {
-        const int m = m0 + 32 * MB * wm + 32 * mb + l32;
+    for (int mb = 0; mb < M16; ++mb) {
+        const int m = m0 + 16 * M16 * wm + 16 * mb + l16;
         if (m >= p.M) continue;
 #pragma unroll
-        for (int nb = 0; nb < NB; ++nb) {
-            int nb0 = n0 + 32 * NB * wn + 32 * nb;   // first column of the block
-            if (CONCAT) {                             // ... inside the weight that holds the block
+        for (int nb = 0; nb < N16; ++nb) {
+            int nb0 = n0 + 16 * N16 * wn + 16 * nb;   // first column of the block
+            if (CONCAT) {                              // ... inside the weight that holds the block
                 int local;
                 const int sg = group_of_unit(p.grp, nb0, local);
                 nb0 = local;
                 Dg = (short*)(sg == 0 ? p.grp.D[0] : sg == 1 ? p.grp.D[1] : p.grp.D[2]);
                 ldd = sg == 0 ? p.grp.ldd[0] : sg == 1 ? p.grp.ldd[1] : p.grp.ldd[2];
             }
-#pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const int n = nb0 + 8 * j + 4 * h;
-                if (!CONCAT && n >= N) continue;
-                if (SPLIT) {   // the slice's raw sums; gemm_reduce_kernel adds the slices up and applies alpha, beta and C
-                    const f32x4 raw = {acc[nb][mb][4 * j], acc[nb][mb][4 * j + 1], acc[nb][mb][4 * j + 2], acc[nb][mb][4 * j + 3]};
-                    *reinterpret_cast<f32x4*>(p.part + ((int64_t)slice * p.M + m) * N + n) = raw;
-                    continue;
-                }
-                float v[4];
-#pragma unroll
-                for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[nb][mb][4 * j + e];
-                if (p.beta != 0.f) {
-                    const s16x4 c = *reinterpret_cast<const s16x4*>(Cg + (int64_t)m * p.ldc + n);
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
-                }
-                uint2 pk;
-                pk.x = T::pack2(v[0], v[1]);
-                pk.y = T::pack2(v[2], v[3]);
-                *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
+            const int n = nb0 + 4 * quad;
+            if (!CONCAT && n >= N) continue;
+            if (SPLIT) {   // the slice's raw sums; gemm_reduce_kernel adds the slices up and applies alpha, beta and C
+                *reinterpret_cast<f32x4*>(p.part + ((int64_t)slice * p.M + m) * N + n) = acc[nb][mb];
+                continue;
             }
+            float v[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) v[e] = p.alpha * acc[nb][mb][e];
+            if (p.beta != 0.f) {
+                const s16x4 c = *reinterpret_cast<const s16x4*>(Cg + (int64_t)m * p.ldc + n);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[e] += p.beta * T::to_float(c[e]);
+            }
+            uint2 pk;
+            pk.x = T::pack2(v[0], v[1]);
+            pk.y = T::pack2(v[2], v[3]);
+            *reinterpret_cast<uint2*>(Dg + (int64_t)m * ldd + n) = pk;
         }
     }
 }
