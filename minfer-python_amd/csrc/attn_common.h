@@ -172,10 +172,23 @@ MA_DEV float max_across_halves(float x) {
     auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
 }
+// The same over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the 16-lane groups of a 16x16 MFMA block's column): rows
+// 1 and 3 of one operand are swapped with rows 0 and 2 of the other, then the halves.
+MA_DEV float max_across_quads(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return max_across_halves(fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1])));
+}
 MA_DEV float sum_across_halves(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
     return __builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]);
+}
+
+MA_DEV float sum_across_quads(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    return sum_across_halves(__builtin_bit_cast(float, (uint32_t)r[0]) + __builtin_bit_cast(float, (uint32_t)r[1]));
 }
 
 MA_DEV float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }

@@ -181,18 +181,18 @@ template <int D, int NW> struct TileGeom {
     static constexpr int RPW = 256 / RB;      // rows per 256-byte bank window
     static constexpr int TILE_BYTES = 64 * RB;
     // XOR swizzles applied to the granule index of a row.  K is read 16 rows x one granule at a
-    // time (ds_read_b128), V 4 rows x 64 bytes at a time (transpose reads); both become
-    // conflict-free.
+    // time (ds_read_b128), V 4 rows x 32 bytes by each 16-lane group, the groups on consecutive
+    // 4-row blocks (transpose reads); both become conflict-free.
     static MA_DEV int swz_k(int row) { return (row / RPW) & (G - 1); }
-    static MA_DEV int swz_v(int row) { return D == 128 ? ((row & 3) << 2) : (((row >> 1) & 1) << 2); }
+    static MA_DEV int swz_v(int row) { return D == 128 ? ((row & 7) << 1) : (((row >> 1) & 3) << 1); }
 };
 
 template <class T, int D, int MODE, int NW>
 __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams p) {
     using GEO = TileGeom<D, NW>;
     constexpr int RB = GEO::RB, G = GEO::G, RPI = GEO::RPI, NLD = GEO::NLD;
-    constexpr int KC = D / 16;   // 16-wide contraction chunks of Q K^T
-    constexpr int DB = D / 32;   // 32-row blocks of O^T
+    constexpr int KC = D / 32;   // 32-wide contraction chunks of Q K^T
+    constexpr int DB = D / 16;   // 16-row blocks of O^T
     constexpr int kWaves = NW;
     constexpr int STAGE_BYTES = 2 * GEO::TILE_BYTES;   // a stage = the K tile followed by the V tile
     constexpr int ROWS_BYTES = 32 * RB;                // a wave's 32 query (or output) rows
@@ -211,7 +211,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     __shared__ __attribute__((aligned(1024))) char q_lds_own[kAliasRows ? 1 : NW][kAliasRows ? 16 : ROWS_BYTES];
 
     const int tid = threadIdx.x, lane = tid & 63, w = wave_id();
-    const int h = lane >> 5, l32 = lane & 31;
+    const int l16 = lane & 15, quad = lane >> 4;
     const int HPW = 1 << p.hpw_log2, QBW = kWaves >> p.hpw_log2;  // heads, 32-row query blocks per workgroup
     char* const q_stage = kAliasRows ? &kv_lds[1][w * ROWS_BYTES] : &q_lds_own[kAliasRows ? 0 : w][0];
 
@@ -275,13 +275,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     const int q_row0 = qblk * 32;                                // first query row (sequence-local)
     const bool wave_on = q_row0 < seq_len;
     const int last_row = seq_len - 1;
-    const int qrow = q_row0 + l32;                               // this lane's query row
+    const int qrow[2] = {q_row0 + l16, q_row0 + 16 + l16};       // this lane's two query rows (one per 16-row block)
 
     const short* Qh = (const short*)p.q + (kDense ? (int64_t)b * p.q0 : 0) + (int64_t)head * p.q1 + (int64_t)seq_lo * p.q2;
     const short* Kh = (const short*)p.k + (kDense ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
     const short* Vh = (const short*)p.v + (kDense ? (int64_t)b * p.kv0 : 0) + (int64_t)g * p.kv1 + (int64_t)seq_lo * p.kv2;
     short* Oh = (short*)p.out + (kDense ? (int64_t)b * p.o0 : 0) + (int64_t)head * p.o1 + (int64_t)seq_lo * p.o2;
-    const uint8_t* mrow = kDense ? p.mask + ((size_t)b * p.L + min(qrow, last_row)) * p.L : nullptr;
+    const uint8_t* mrow[2] = {kDense ? p.mask + ((size_t)b * p.L + min(qrow[0], last_row)) * p.L : nullptr,
+                              kDense ? p.mask + ((size_t)b * p.L + min(qrow[1], last_row)) * p.L : nullptr};
 
     // The wave's Q rows are requested now and used after the tile list is built, so that the two latencies overlap.
     // They are copied global->LDS as whole rows (RPI rows per instruction, with the K tile's swizzle) and read back as
@@ -382,7 +383,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     }
 
     const float c2 = p.scale_log2;
-    s16x8 qf[KC];   // the wave's query rows as B-operand fragments; filled once the first K/V tile has been requested
+    s16x8 qf[2][KC];   // the wave's query rows as B-operand fragments; filled once the first K/V tile has been requested
 
     // ---- global -> LDS tile copy ----------------------------------------------------------
     // Instruction j of this wave fills rows (j*kWaves + w)*RPI .. +RPI-1 of the tile.  The lane's byte offset from the
@@ -424,37 +425,39 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     };
 
     // ---- per-lane LDS read addresses (stage 0; the other stage and the row blocks are immediates) ----
-    // K fragment c of key block kb: row 32kb + l32, granule (2c+h) ^ swz_k(row); swz_k is the same for
-    // rows l32 and 32 + l32.  V^T fragment (chunk c, half, db): row 16c + 8half + 4h + li/4, columns
-    // 32db + 16(blk&1) + 4(li&3); swz_v depends on li only.
-    const int blk = lane >> 4, li = lane & 15;
+    // The matrix instruction is v_mfma_f32_16x16x32: lane (l16, quad) holds row l16, contraction values 8 quad + 0..7 of
+    // an A or B fragment and rows 4 quad + 0..3, column l16 of a result block.  K fragment (chunk c of 32 head
+    // dimensions, key block kb of 16): row 16kb + l16, granule (4c + quad) ^ swz_k(row); swz_k is the same for rows l16
+    // and 16kb + l16.  V^T fragment (chunk ck of 32 keys, block db of 16 head dimensions): two transpose reads, the
+    // 16-lane group `quad` addressing key rows 32ck + 4 quad + 0..3 and 32ck + 16 + 4 quad + 0..3, columns 16db + 4(li&3);
+    // swz_v depends on quad and li only.
+    const int li = l16;
     uint32_t k_rd[KC], v_rd[DB];
     {
-        const int sw = GEO::swz_k(l32);
+        const int sw = GEO::swz_k(l16);
 #pragma unroll
-        for (int c = 0; c < KC; ++c) k_rd[c] = lds_addr(&kv_lds[0][0]) + l32 * RB + 16 * ((2 * c + h) ^ sw);
-        const int vrow = 4 * h + (li >> 2);
+        for (int c = 0; c < KC; ++c) k_rd[c] = lds_addr(&kv_lds[0][0]) + l16 * RB + 16 * ((4 * c + quad) ^ sw);
+        const int vrow = 4 * quad + (li >> 2);
         const int swv = GEO::swz_v(vrow);
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
-            const int dcol = 32 * db + 16 * (blk & 1) + 4 * (li & 3);
+            const int dcol = 16 * db + 4 * (li & 3);
             v_rd[db] = lds_addr(&kv_lds[0][GEO::TILE_BYTES]) + vrow * RB + 16 * ((dcol >> 3) ^ swv) + 2 * (dcol & 7);
         }
     }
 
-    f32x16 o_acc[DB];
+    f32x4 o_acc[DB][2];   // [block of 16 head dimensions][block of 16 query rows]: rows d = 16db + 4 quad + 0..3, column l16
 #pragma unroll
     for (int db = 0; db < DB; ++db)
 #pragma unroll
-        for (int r = 0; r < 16; ++r) o_acc[db][r] = 0.f;
-    // Reference exponent of the lane's query row (log2 units; -inf until a key has been seen) and the
-    // lane's share of the softmax denominator.  The reference moves only when a tile's largest exponent
+        for (int qb = 0; qb < 2; ++qb) o_acc[db][qb] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // Reference exponent of each of the lane's two query rows (log2 units; -inf until a key has been seen) and the
+    // lane's share of the softmax denominators.  The reference moves only when a tile's largest exponent
     // exceeds it by more than kLazyLog2, so most tiles rescale nothing and weights stay below 2^kLazyLog2.
-    float m_ref = -INFINITY, l_sum = 0.f;
+    float m_ref[2] = {-INFINITY, -INFINITY}, l_sum[2] = {0.f, 0.f};
     constexpr float kLazyLog2 = 8.f;
-    f32x16 neg_ref;   // -m_ref in every register (0 while there is no reference): the MFMA C operand of Q K^T
-#pragma unroll
-    for (int r = 0; r < 16; ++r) neg_ref[r] = 0.f;
+    f32x4 neg_ref[2];   // -m_ref in every register (0 while there is no reference): the MFMA C operand of Q K^T
+    neg_ref[0] = neg_ref[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 
     auto tile_of = [&](uint32_t e, int it, int& kt, uint32_t& cls_w) {
         if (kDense) {
@@ -470,26 +473,26 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         if (!kDense || n_active <= 0) return 0u;
         return __builtin_amdgcn_readfirstlane(tile_list[min(it, n_active - 1)]);
     };
-    // mask words of a MIXED dense tile: word [kb][j] covers keys key0 + 32kb + 8j + 4h + 0..3
+    // mask words of a MIXED dense tile: word [qb][kb] covers keys key0 + 16kb + 4 quad + 0..3 of query row qrow[qb]
     uint32_t mw[2][4] = {{0u, 0u, 0u, 0u}, {0u, 0u, 0u, 0u}};
     auto fetch_mask = [&](int kt) {
         const int key0 = kt * 64;
         if (p.mask_vec && key0 + 64 <= seq_len) {
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
-                    mw[kb][j] = *reinterpret_cast<const uint32_t*>(mrow + key0 + 32 * kb + 8 * j + 4 * h);
+                for (int kb = 0; kb < 4; ++kb)
+                    mw[qb][kb] = *reinterpret_cast<const uint32_t*>(mrow[qb] + key0 + 16 * kb + 4 * quad);
         } else {  // unaligned rows or a tile crossing the end: bytes, clamped (the range test comes later)
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int qb = 0; qb < 2; ++qb)
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const int kbase = key0 + 32 * kb + 8 * j + 4 * h;
+                for (int kb = 0; kb < 4; ++kb) {
+                    const int kbase = key0 + 16 * kb + 4 * quad;
                     uint32_t x = 0;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) x |= (uint32_t)mrow[min(kbase + e, last_row)] << (8 * e);
-                    mw[kb][j] = x;
+                    for (int e = 0; e < 4; ++e) x |= (uint32_t)mrow[qb][min(kbase + e, last_row)] << (8 * e);
+                    mw[qb][kb] = x;
                 }
         }
     };
@@ -499,138 +502,142 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         constexpr int STAGE = decltype(stage_tag)::value;
         constexpr int SOFF = STAGE * STAGE_BYTES;
         const int key0 = kt * 64;
+        auto pin = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
 
-        // S^T = K Q^T, accumulated on top of -reference: register r of block kb is key 32kb + 8(r/4) + 4h + r%4.
-        // K fragments go through two register buffers of two contraction chunks each (both key blocks): the buffer just
-        // consumed is refilled while the other one feeds the matrix pipe (all sixteen fragments requested up front ran
-        // at the same speed and held 24 registers more).  The accumulators start from -reference (neg_ref, a register
-        // block that changes only when the reference does), so the MFMA output is the exponent relative to the reference.
-        f32x16 e_acc[2];
-        // V^T fragments of a 16-key chunk; the first two chunks are requested between the last MFMAs of S^T, where the K
-        // ring is no longer refilled: their latency hides behind those, the row maximum and the first exponentials
-        s16x8 va[2][DB];
-        auto load_v = [&](int c, s16x8 (&a)[DB]) __attribute__((always_inline)) {
-#pragma unroll
-            for (int db = 0; db < DB; ++db) {
-                const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (16 * c) * RB);
-                const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (16 * c + 8) * RB);
-                a[db] = s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
-            }
+        // V^T fragment of key chunk ck (32 keys), block db (16 head dimensions)
+        auto read_v = [&](int ck, int db) __attribute__((always_inline)) -> s16x8 {
+            const s16x4 t0 = lds_read_tr16(v_rd[db], SOFF + (32 * ck) * RB);
+            const s16x4 t1 = lds_read_tr16(v_rd[db], SOFF + (32 * ck + 16) * RB);
+            return s16x8{t0[0], t0[1], t0[2], t0[3], t1[0], t1[1], t1[2], t1[3]};
         };
+        s16x8 va[DB];   // the V^T fragments of one key chunk; refilled with the next chunk's as they are used the last time
+
+        // S^T = K Q^T, accumulated on top of -reference: register e of block [kb][qb] is key 16kb + 4 quad + e, query row
+        // 16qb + l16.  K fragments go through two register buffers of one contraction chunk each (four key blocks): the
+        // fragment just used for the last time is refilled two chunks ahead, between the MFMAs (every MFMA and read is
+        // pinned where it is written: left alone the compiler moved every read down to just before the MFMAs that use it).
+        // Between the MFMAs of the last chunk, whose fragments are not refilled, the first key chunk's V^T fragments are
+        // requested.  The accumulators start from -reference (neg_ref, a register block that changes only when the
+        // reference does), so the MFMA output is the exponent relative to the reference.
+        f32x4 e_acc[4][2];
         {
-            s16x8 kf[2][2][2];   // [buffer][chunk in buffer][key block]
-            auto load_k = [&](int buf, int c0) __attribute__((always_inline)) {
+            s16x8 kf[2][4];   // [buffer][key block]
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    kf[buf][i][0] = lds_read_b128(k_rd[c0 + i], SOFF);
-                    kf[buf][i][1] = lds_read_b128(k_rd[c0 + i], SOFF + 32 * RB);
-                }
-            };
-            load_k(0, 0);
-            load_k(1, 2);
-            __builtin_amdgcn_sched_barrier(0);
-            // (the scheduling barriers keep the refill where it is written, four chunks ahead of its use: left alone
-            // the compiler moved every pair of reads down to just before the MFMAs that use them)
+            for (int c = 0; c < 2 && c < KC; ++c)
 #pragma unroll
-            for (int c0 = 0; c0 < KC; c0 += 2) {
-                const int buf = (c0 >> 1) & 1;
+                for (int kb = 0; kb < 4; ++kb) kf[c][kb] = lds_read_b128(k_rd[c], SOFF + 16 * kb * RB);
+            pin();
 #pragma unroll
-                for (int i = 0; i < 2; ++i) {
-                    if (c0 + i == 0) {
-                        e_acc[0] = T::mfma32(kf[buf][i][0], qf[0], neg_ref);
-                        e_acc[1] = T::mfma32(kf[buf][i][1], qf[0], neg_ref);
-                    } else {
-                        e_acc[0] = T::mfma32(kf[buf][i][0], qf[c0 + i], e_acc[0]);
-                        e_acc[1] = T::mfma32(kf[buf][i][1], qf[c0 + i], e_acc[1]);
+            for (int c = 0; c < KC; ++c) {
+#pragma unroll
+                for (int kb = 0; kb < 4; ++kb) {
+#pragma unroll
+                    for (int qb = 0; qb < 2; ++qb)
+                        e_acc[kb][qb] = T::mfma16(kf[c & 1][kb], qf[qb][c], c == 0 ? neg_ref[qb] : e_acc[kb][qb]);
+                    pin();
+                    if (c + 2 < KC) {
+                        kf[c & 1][kb] = lds_read_b128(k_rd[c + 2], SOFF + 16 * kb * RB);
+                    } else if (c + 1 == KC) {
+#pragma unroll
+                        for (int db = kb * (DB / 4); db < (kb + 1) * (DB / 4); ++db) va[db] = read_v(0, db);
                     }
-                    __builtin_amdgcn_sched_barrier(0);
-                    if (c0 + 4 < KC) {
-                        kf[buf][i][0] = lds_read_b128(k_rd[c0 + 4 + i], SOFF);
-                        kf[buf][i][1] = lds_read_b128(k_rd[c0 + 4 + i], SOFF + 32 * RB);
-                    } else if (c0 + 4 == KC) {
-                        load_v(i, va[i]);
-                    }
-                    __builtin_amdgcn_sched_barrier(0);
+                    pin();
                 }
             }
         }
 
         // ---- masking ----------------------------------------------------------------------
-        // Register 4j + e of block kb is key key0 + 32kb + 8j + 4h + e.  The test by position (keys past the end of the
-        // sequence; in a packed batch also keys after the lane's query row) is one compare of a constant with a per-lane
-        // limit; dense MIXED tiles test their mask bytes as well.
+        // The test by position (keys past the end of the sequence; in a packed batch also keys after the lane's query
+        // row) is one compare of a constant with a per-lane limit; dense MIXED tiles test their mask bytes as well.
         if (cls_w == TILE_MIXED || key0 + 64 > seq_len) {
             const bool use_bytes = kDense && cls_w == TILE_MIXED;
-            int lim = last_row - key0 - 4 * h;                              // largest kept 32kb + 8j + e
-            if (MODE == MODE_VARLEN) lim = min(lim, qrow - key0 - 4 * h);
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int qb = 0; qb < 2; ++qb) {
+                int lim = last_row - key0 - 4 * quad;                              // largest kept 16kb + e
+                if (MODE == MODE_VARLEN) lim = min(lim, qrow[qb] - key0 - 4 * quad);
 #pragma unroll
-                for (int j = 0; j < 4; ++j)
+                for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        bool keep = 32 * kb + 8 * j + e <= lim;
-                        if (kDense) keep = keep && (!use_bytes || ((mw[kb][j] >> (8 * e)) & 0xffu) != 0u);
-                        e_acc[kb][4 * j + e] = keep ? e_acc[kb][4 * j + e] : -INFINITY;
+                        bool keep = 16 * kb + e <= lim;
+                        if (kDense) keep = keep && (!use_bytes || ((mw[qb][kb] >> (8 * e)) & 0xffu) != 0u);
+                        e_acc[kb][qb][e] = keep ? e_acc[kb][qb][e] : -INFINITY;
                     }
+            }
         }
         // ---- reference update (rare after the first tiles) --------------------------------------
         {
-            float mx = e_acc[0][0];
+            float mx[2];
 #pragma unroll
-            for (int kb = 0; kb < 2; ++kb)
+            for (int qb = 0; qb < 2; ++qb) {
+                float x = e_acc[0][qb][0];
 #pragma unroll
-                for (int r = 0; r < 16; ++r) mx = fmaxf(mx, e_acc[kb][r]);
-            mx = max_across_halves(mx);   // largest exponent of the row in this tile, relative to the reference
-            const bool grow = mx > kLazyLog2 || (m_ref == -INFINITY && mx > -INFINITY);
-            if (__any(grow)) {  // wave-uniform branch
-                const float delta = grow ? mx : 0.f;
-                const float alpha = (m_ref == -INFINITY) ? 0.f : fast_exp2(-delta);
-                m_ref = grow ? ((m_ref == -INFINITY) ? mx : m_ref + mx) : m_ref;
-                const float nr = (m_ref == -INFINITY) ? 0.f : -m_ref;
+                for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) neg_ref[r] = nr;
-                l_sum *= alpha;
+                    for (int e = 0; e < 4; ++e) x = fmaxf(x, e_acc[kb][qb][e]);
+                mx[qb] = max_across_quads(x);   // largest exponent of the row in this tile, relative to the reference
+            }
+            const bool grow0 = mx[0] > kLazyLog2 || (m_ref[0] == -INFINITY && mx[0] > -INFINITY);
+            const bool grow1 = mx[1] > kLazyLog2 || (m_ref[1] == -INFINITY && mx[1] > -INFINITY);
+            if (__any(grow0 || grow1)) {  // wave-uniform branch
 #pragma unroll
-                for (int kb = 0; kb < 2; ++kb)
+                for (int qb = 0; qb < 2; ++qb) {
+                    const bool grow = qb == 0 ? grow0 : grow1;
+                    const float delta = grow ? mx[qb] : 0.f;
+                    const float alpha = (m_ref[qb] == -INFINITY) ? 0.f : fast_exp2(-delta);
+                    m_ref[qb] = grow ? ((m_ref[qb] == -INFINITY) ? mx[qb] : m_ref[qb] + mx[qb]) : m_ref[qb];
+                    const float nr = (m_ref[qb] == -INFINITY) ? 0.f : -m_ref[qb];
+                    neg_ref[qb] = f32x4{nr, nr, nr, nr};
+                    l_sum[qb] *= alpha;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) e_acc[kb][r] -= delta;
+                    for (int kb = 0; kb < 4; ++kb)
 #pragma unroll
-                for (int db = 0; db < DB; ++db)
+                        for (int e = 0; e < 4; ++e) e_acc[kb][qb][e] -= delta;
 #pragma unroll
-                    for (int r = 0; r < 16; ++r) o_acc[db][r] *= alpha;
+                    for (int db = 0; db < DB; ++db)
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) o_acc[db][qb][e] *= alpha;
+                }
             }
         }
-        // ---- P = 2^E and O^T += V^T P^T, one 16-key chunk at a time -------------------------------
-        // Chunk c contracts keys 16c..16c+15 in the order 16c + 8(i/4) + 4h + i%4 (i = element of the
-        // lane's 8-wide k slice), which is the order the exponent registers already have.  The weights of
-        // chunk c+1 are computed before the MFMAs of chunk c are issued, so they run while that chunk is in
-        // the matrix pipe.
-        float ls = 0.f;
-        auto weights = [&](int c) -> s16x8 {
+        // ---- P = 2^E and O^T += V^T P^T, one 32-key chunk and one 16-row query block at a time ---------
+        // Chunk ck contracts keys 32ck .. 32ck+31 in the order 32ck + 16(i/4) + 4 quad + i%4 (i = element of the lane's
+        // 8-wide slice), which is the order the exponent registers of key blocks 2ck and 2ck+1 already have and the
+        // order the two transpose reads of a V^T fragment deliver.  The weights of the next (chunk, query block) are
+        // computed before the MFMAs of the current one are issued, so they run while those are in the matrix pipe.
+        float ls[2] = {0.f, 0.f};
+        auto weights = [&](int ck, int qb) -> s16x8 {
             uint32_t pk[4];
 #pragma unroll
             for (int i = 0; i < 8; i += 2) {
-                const int kb = c >> 1, r = 8 * (c & 1) + i;
-                pk[i >> 1] = T::pack2(fast_exp2(e_acc[kb][r]), fast_exp2(e_acc[kb][r + 1]));
-                ls = T::add_pair(pk[i >> 1], ls);   // the denominator sums the rounded weights the MFMA uses
+                const int kb = 2 * ck + (i >> 2), r = i & 3;
+                pk[i >> 1] = T::pack2(fast_exp2(e_acc[kb][qb][r]), fast_exp2(e_acc[kb][qb][r + 1]));
+                ls[qb] = T::add_pair(pk[i >> 1], ls[qb]);   // the denominator sums the rounded weights the MFMA uses
             }
             uint4 pu; pu.x = pk[0]; pu.y = pk[1]; pu.z = pk[2]; pu.w = pk[3];
             return __builtin_bit_cast(s16x8, pu);
         };
-        s16x8 pcur = weights(0);
-        __builtin_amdgcn_sched_barrier(0);
+        s16x8 pcur = weights(0, 0);
+        pin();
 #pragma unroll
-        for (int c = 0; c < 4; ++c) {
+        for (int s = 0; s < 4; ++s) {   // (ck, qb) = (s >> 1, s & 1)
+            const int ck = s >> 1, qb = s & 1;
             s16x8 pnext = pcur;
-            if (c + 1 < 4) pnext = weights(c + 1);
+            if (s + 1 < 4) pnext = weights((s + 1) >> 1, (s + 1) & 1);
 #pragma unroll
-            for (int db = 0; db < DB; ++db) o_acc[db] = T::mfma32(va[c & 1][db], pcur, o_acc[db]);
-            __builtin_amdgcn_sched_barrier(0);
-            if (c + 2 < 4) load_v(c + 2, va[c & 1]);
+            for (int db = 0; db < DB; ++db) {
+                o_acc[db][qb] = T::mfma16(va[db], pcur, o_acc[db][qb]);
+                if (qb == 1 && ck == 0) {   // the chunk's fragments are used for the last time: the next chunk's take their place
+                    pin();
+                    va[db] = read_v(1, db);
+                    pin();
+                }
+            }
+            pin();
             pcur = pnext;
         }
-        l_sum += ls;
+        l_sum[0] += ls[0];
+        l_sum[1] += ls[1];
     };
 
     // ---- main loop: one barrier per tile; the copy of tile t+1 is issued right after the barrier that
@@ -641,17 +648,19 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         tile_of(e_cur, 0, kt_first, cls_first);
         issue_tile(kt_first, 0);
     }
-    // ---- Q fragments (B operand): lane = query row l32, d = 16c + 8h + 0..7 --------------------
+    // ---- Q fragments (B operand): lane = query row 16qb + l16, d = 32c + 8 quad + 0..7 --------------------
     // Q is multiplied by scale*log2(e) once, here, so that the MFMA accumulator of Q K^T is directly
     // the base-2 exponent of the softmax weight (minus the running reference it is initialised with).
     // The rows were requested before the tile list was built, and the first K/V tile after them: copies retire in
     // order, so the rows have landed once no more than that tile's copies are outstanding.
     if (n_active > 0) wait_vmcnt<2 * NLD>(); else wait_vmcnt<0>();
     {
-        const uint32_t qa = lds_addr(q_stage) + l32 * RB;
-        const int sw = GEO::swz_k(l32);
+        const uint32_t qa = lds_addr(q_stage) + l16 * RB;
+        const int sw = GEO::swz_k(l16);   // the same for row 16 + l16
 #pragma unroll
-        for (int c = 0; c < KC; ++c) qf[c] = T::scale8(lds_read_b128(qa + 16 * ((2 * c + h) ^ sw), 0), c2);
+        for (int qb = 0; qb < 2; ++qb)
+#pragma unroll
+            for (int c = 0; c < KC; ++c) qf[qb][c] = T::scale8(lds_read_b128(qa + 16 * ((4 * c + quad) ^ sw), 16 * qb * RB), c2);
     }
     if (kDense && n_active > 0 && cls_first == TILE_MIXED) fetch_mask(kt_first);
     auto iteration = [&](auto stage_tag, int it) {
@@ -678,8 +687,12 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     // per lane, granules XOR-swizzled by row) and read back 16 bytes per lane, RPI whole rows per instruction, the same
     // data leaves in 32/RPI stores of whole rows.
     if (!wave_on) return;
-    const float l = sum_across_halves(l_sum);
-    const float inv = l > 0.f ? 1.f / l : 0.f;
+    float inv[2];
+#pragma unroll
+    for (int qb = 0; qb < 2; ++qb) {
+        const float l = sum_across_quads(l_sum[qb]);
+        inv[qb] = l > 0.f ? 1.f / l : 0.f;
+    }
     {
         const int free_stage = (n_active & 1);   // the last tile sat in stage (n_active - 1) & 1
         const uint32_t so = kAliasRows ? lds_addr(&kv_lds[0][0]) + free_stage * STAGE_BYTES + w * ROWS_BYTES : lds_addr(q_stage);
@@ -688,12 +701,13 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
 #pragma unroll
         for (int db = 0; db < DB; ++db) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
+            for (int qb = 0; qb < 2; ++qb) {
                 u32x2 pk;
-                pk.x = T::pack2(o_acc[db][4 * j + 0] * inv, o_acc[db][4 * j + 1] * inv);
-                pk.y = T::pack2(o_acc[db][4 * j + 2] * inv, o_acc[db][4 * j + 3] * inv);
-                const int gi = 4 * db + j;   // 16-byte granule of the row: columns 8gi..8gi+7, this lane's half 4h..4h+3
-                *(lds_u32x2*)(uintptr_t)(so + l32 * RB + 16 * (gi ^ (l32 & (G - 1))) + 8 * h) = pk;
+                pk.x = T::pack2(o_acc[db][qb][0] * inv[qb], o_acc[db][qb][1] * inv[qb]);
+                pk.y = T::pack2(o_acc[db][qb][2] * inv[qb], o_acc[db][qb][3] * inv[qb]);
+                const int row = 16 * qb + l16;
+                const int gi = 2 * db + (quad >> 1);   // 16-byte granule of the row: columns 8gi..8gi+7, this lane's half 4(quad&1)..+3
+                *(lds_u32x2*)(uintptr_t)(so + row * RB + 16 * (gi ^ (row & (G - 1))) + 8 * (quad & 1)) = pk;
             }
         }
         if (q_row0 + 32 <= seq_len) {   // every row exists: a wave-uniform base per store plus one 32-bit lane offset
