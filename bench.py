@@ -603,8 +603,8 @@ def main():
                            "workload": "prefill B=1 Hq=8 Hkv=2 S=256 D=64 causal dense-mask, fp32 inputs rounded to fp16 for the GPU op (BASELINE configs[0]); launch-bound"}
     rec["calibration"] = {"mfma_only_f16_random": sus_f16, "mfma_only_bf16_random": sus_bf16,
                           "attention_mix_f16_random": mix_f16, "attention_mix_bf16_random": mix_bf16,
-                          "note": "mfma_only: v_mfma_f32_32x32x16 alone, two waves per SIMD on every compute unit, operands 0.5*N(0,1); "
-                                  "attention_mix: the prefill kernel's per-tile instructions (32 MFMAs, 48 LDS fragment reads, the softmax's vector work) "
+                          "note": "mfma_only: v_mfma_f32_16x16x32 alone (the instruction the prefill and GEMM kernels use), two waves per SIMD on every compute unit, operands 0.5*N(0,1); "
+                                  "attention_mix: the prefill kernel's per-tile instructions (64 MFMAs, 48 LDS fragment reads, the softmax's vector work) "
                                   "on tiles that stay in LDS, nothing else in the loop; frac_of_sustained and frac_of_attention_mix = achieved / these, "
                                   "reported beside frac (= achieved / nominal peak), measured in this run on this box"}
     rec["rmsnorm"] = {"value": n_gbs, "unit": "GB/s", "ms": n_avg_ms, "median_ms": n_med_ms,

@@ -335,18 +335,21 @@ int minfer_rope_kv_append_q8_0(int dtype, int style, void* q, const void* k, con
 
 /*
  * Calibration, not an operator (no counterpart in the reference): `workgroups` workgroups of 8 waves issue
- * 8 * iters v_mfma_f32_32x32x16 (f16 or bf16) each, back to back on four accumulators, from 16 operand fragments
- * (64 lanes x 16 bytes each, 16 KiB in all) that every wave reads once from `operands`; 32 768 flop per instruction,
- * i.e. workgroups * 8 * 8 * iters * 32768 flop per launch.  Timed by the caller, it gives the matrix rate the chip
- * sustains on the caller's operand values (random values cost more power than constant ones), the figure the
- * attention and GEMM kernels' fractions of the nominal peak can be read against.  sink: workgroups * 512 floats.
+ * 16 * iters v_mfma_f32_16x16x32 (f16 or bf16) each, the instruction the prefill and GEMM kernels are built on, back to
+ * back on eight accumulator blocks, from 16 operand fragments (64 lanes x 16 bytes each, 16 KiB in all) that every wave
+ * reads once from `operands`; 16 384 flop per instruction, i.e. workgroups * 8 * 8 * iters * 32768 flop per launch.
+ * Timed by the caller, it gives the matrix rate the chip sustains on the caller's operand values (random values cost
+ * more power than constant ones), the figure the attention and GEMM kernels' fractions of the nominal peak can be read
+ * against.  minfer_calib_mfma_rate_32x32x16 issues 8 * iters v_mfma_f32_32x32x16 on four blocks instead (the same
+ * flops): on random fp16 operands the chip sustains 15-18 % less of that instruction.  sink: workgroups * 512 floats.
  */
 #define MINFER_CALIB_MFMA_OPERAND_BYTES 16384
 #define MINFER_CALIB_MFMA_FLOP_PER_ITER (8 * 8 * 32768)   /* per workgroup */
 int minfer_calib_mfma_rate(int dtype, const void* operands, int64_t iters, int64_t workgroups, float* sink, void* stream);
+int minfer_calib_mfma_rate_32x32x16(int dtype, const void* operands, int64_t iters, int64_t workgroups, float* sink, void* stream);
 
 /*
- * Calibration as well: the prefill kernel's per-tile instruction mix at head_dim 128 (32 MFMAs, 16 + 32 LDS fragment
+ * Calibration as well: the prefill kernel's per-tile instruction mix at head_dim 128 (64 MFMAs, 16 + 32 LDS fragment
  * reads, the softmax's maximum / exponential / pack / denominator instructions) on one K and one V tile that stay in
  * LDS, with no global memory traffic, barrier, mask or bookkeeping in the loop; `iters` tiles per wave, 32 * 32768
  * flop each, workgroups * 8 waves.  lds_reads = 0 keeps the fragments in registers, softmax = 0 feeds the second GEMM

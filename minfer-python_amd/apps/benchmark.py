@@ -206,19 +206,21 @@ def gemm(backend: str, which: str):
 
 
 def mfma_rate(backend: str, which: str):
-    """Calibration, not an operator: the rate the chip sustains on v_mfma_f32_32x32x16 alone (two waves per SIMD on
-    every compute unit, nothing else in the loop), for random, constant and zero operand values, fp16 and bf16.  `ref`
-    runs torch.matmul (the vendor library) at 8192^3 for comparison.  The nominal dense peak is 2500 TFLOP/s."""
+    """Calibration, not an operator: the rate the chip sustains on v_mfma_f32_16x16x32 alone, the instruction the prefill
+    and GEMM kernels use, and on v_mfma_f32_32x32x16 (two waves per SIMD on every compute unit, nothing else in the
+    loop), for random, constant and zero operand values, fp16 and bf16.  `ref` runs torch.matmul (the vendor library) at
+    8192^3 for comparison.  The nominal dense peak is 2500 TFLOP/s."""
     import calibration
     if which == "minfer":
-        print(f"{'dtype':<10}{'operands':<12}{'TFLOP/s':>10}{'of 2500':>10}   (launches of ~5 ms back to back, 200 ms timed after 150 ms of warm-up)")
-        for dtype in (torch.float16, torch.bfloat16):
-            for kind in ("random", "constant", "zero"):
-                r = calibration.mfma_rate(dtype, kind)
-                print(f"{r['dtype']:<10}{kind:<12}{r['tflops']:>10.1f}{r['tflops'] / 2500.0:>10.3f}")
+        print(f"{'instruction':<22}{'dtype':<10}{'operands':<12}{'TFLOP/s':>10}{'of 2500':>10}   (launches of ~5 ms back to back, 200 ms timed after 150 ms of warm-up)")
+        for shape32 in (False, True):
+            for dtype in (torch.float16, torch.bfloat16):
+                for kind in ("random", "constant", "zero"):
+                    r = calibration.mfma_rate(dtype, kind, shape32=shape32)
+                    print(f"{r['instruction']:<22}{r['dtype']:<10}{kind:<12}{r['tflops']:>10.1f}{r['tflops'] / 2500.0:>10.3f}")
         # the prefill kernel's per-tile instruction mix without any memory traffic, barrier or bookkeeping: what each kind
         # of co-running work costs the matrix rate, and what a kernel with no fixed cost at all would reach
-        print(f"{'dtype':<10}{'operands':<12}{'fragments':<12}{'softmax':<10}{'TFLOP/s':>10}{'of 2500':>10}   (32 MFMAs per wave and 64-key tile, head_dim 128)")
+        print(f"{'dtype':<10}{'operands':<12}{'fragments':<12}{'softmax':<10}{'TFLOP/s':>10}{'of 2500':>10}   (64 MFMAs of 16x16x32 per wave and 64-key tile, head_dim 128)")
         for dtype in (torch.float16, torch.bfloat16):
             for kind in ("random", "zero"):
                 for lds_reads, softmax in ((False, False), (True, False), (False, True), (True, True)):

@@ -10,7 +10,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(os.path.dirname(HERE), "lib", "libminfer_attn.so")
 DTYPE_CODE = {torch.float16: 1, torch.bfloat16: 30}
 OPERAND_BYTES = 16384
-FLOP_PER_ITER = 8 * 8 * 32768     # per workgroup, minfer_calib_mfma_rate
+FLOP_PER_ITER = 8 * 8 * 32768     # per workgroup, minfer_calib_mfma_rate (and _32x32x16)
 MIX_FLOP_PER_ITER = 8 * 32 * 32768  # per workgroup, minfer_calib_attn_mix (one 64-key tile per wave)
 
 _lib = None
@@ -22,8 +22,9 @@ def _load():
         if not os.path.exists(LIB_PATH):
             raise RuntimeError(f"{LIB_PATH} is not built; run python minfer-python_amd/build.py")
         _lib = ctypes.CDLL(LIB_PATH)
-        _lib.minfer_calib_mfma_rate.restype = ctypes.c_int
-        _lib.minfer_calib_mfma_rate.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
+        for fn in (_lib.minfer_calib_mfma_rate, _lib.minfer_calib_mfma_rate_32x32x16):
+            fn.restype = ctypes.c_int
+            fn.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_void_p, ctypes.c_void_p]
         _lib.minfer_calib_attn_mix.restype = ctypes.c_int
         _lib.minfer_calib_attn_mix.argtypes = [ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
                                                ctypes.c_void_p, ctypes.c_void_p]
@@ -45,9 +46,10 @@ def mfma_operands(dtype, kind: str, device="cuda", seed=0):
     raise ValueError(f"unknown operand kind {kind}")
 
 
-def launch_mfma_rate(operands, iters: int, workgroups: int, sink):
-    rc = _load().minfer_calib_mfma_rate(DTYPE_CODE[operands.dtype], operands.data_ptr(), iters, workgroups, sink.data_ptr(),
-                                        ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
+def launch_mfma_rate(operands, iters: int, workgroups: int, sink, shape32: bool = False):
+    fn = _load().minfer_calib_mfma_rate_32x32x16 if shape32 else _load().minfer_calib_mfma_rate
+    rc = fn(DTYPE_CODE[operands.dtype], operands.data_ptr(), iters, workgroups, sink.data_ptr(),
+            ctypes.c_void_p(torch.cuda.current_stream().cuda_stream))
     if rc != 0:
         raise RuntimeError(_load().minfer_attn_last_error().decode())
 
@@ -80,12 +82,13 @@ def _sustained(launch, flop_per_iter, first_iters, timed_ms, prewarm_ms, device)
     return {"tflops": flop / (ms * 1e-3) / 1e12, "ms_per_launch": ms, "iters": iters, "workgroups": wgs, "launches": n}
 
 
-def mfma_rate(dtype=torch.float16, kind="random", timed_ms=200.0, prewarm_ms=150.0, device="cuda"):
-    """Sustained rate of v_mfma_f32_32x32x16 on the whole chip, TFLOP/s: one workgroup of 8 waves per compute unit,
-    launches of ~5 ms run back to back for `prewarm_ms` (the clocks settle), then for `timed_ms` between two events."""
+def mfma_rate(dtype=torch.float16, kind="random", timed_ms=200.0, prewarm_ms=150.0, device="cuda", shape32=False):
+    """Sustained rate of v_mfma_f32_16x16x32 (shape32: v_mfma_f32_32x32x16) on the whole chip, TFLOP/s: one workgroup of 8
+    waves per compute unit, launches of ~5 ms run back to back for `prewarm_ms` (the clocks settle), then for `timed_ms`
+    between two events."""
     ops = mfma_operands(dtype, kind, device)
-    r = _sustained(lambda iters, wgs, sink: launch_mfma_rate(ops, iters, wgs, sink), FLOP_PER_ITER, 2000, timed_ms, prewarm_ms, device)
-    r.update({"operands": kind, "dtype": str(dtype).replace("torch.", "")})
+    r = _sustained(lambda iters, wgs, sink: launch_mfma_rate(ops, iters, wgs, sink, shape32), FLOP_PER_ITER, 2000, timed_ms, prewarm_ms, device)
+    r.update({"operands": kind, "dtype": str(dtype).replace("torch.", ""), "instruction": "v_mfma_f32_32x32x16" if shape32 else "v_mfma_f32_16x16x32"})
     return r
 
 

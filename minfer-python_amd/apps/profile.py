@@ -271,10 +271,10 @@ def copy(backend: str, which: str, workload: str, repeat: int):
 
 
 def mfma_rate(backend: str, which: str, workload: str, repeat: int):
-    """Calibration like `copy`: the library's matrix-instruction-only loop (v_mfma_f32_32x32x16_f16, two waves per SIMD
+    """Calibration like `copy`: the library's matrix-instruction-only loop (v_mfma_f32_16x16x32_f16, two waves per SIMD
     on every compute unit), ~5 ms per launch, on random operand values (--workload reference: constant ones).  The
     kernel's duration in a trace, or MFMA counters over it, give the rate the matrix pipes sustain when nothing else
-    runs: 256 workgroups x 8 waves x 8 x iters instructions of 32 768 flop."""
+    runs: 256 workgroups x 8 waves x 16 x iters instructions of 16 384 flop."""
     import calibration
     ops = calibration.mfma_operands(torch.float16, "constant" if workload == "reference" else "random")
     wgs = torch.cuda.get_device_properties(0).multi_processor_count

@@ -606,35 +606,31 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         // order the two transpose reads of a V^T fragment deliver.  The weights of the next (chunk, query block) are
         // computed before the MFMAs of the current one are issued, so they run while those are in the matrix pipe.
         float ls[2] = {0.f, 0.f};
-        auto weights = [&](int ck, int qb) -> s16x8 {
-            uint32_t pk[4];
-#pragma unroll
-            for (int i = 0; i < 8; i += 2) {
-                const int kb = 2 * ck + (i >> 2), r = i & 3;
-                pk[i >> 1] = T::pack2(fast_exp2(e_acc[kb][qb][r]), fast_exp2(e_acc[kb][qb][r + 1]));
-                ls[qb] = T::add_pair(pk[i >> 1], ls[qb]);   // the denominator sums the rounded weights the MFMA uses
-            }
-            uint4 pu; pu.x = pk[0]; pu.y = pk[1]; pu.z = pk[2]; pu.w = pk[3];
-            return __builtin_bit_cast(s16x8, pu);
+        // quarter i of the weights of (chunk ck, query block qb): two exponentials, packed
+        auto weights_quarter = [&](int ck, int qb, int i) __attribute__((always_inline)) -> uint32_t {
+            const int kb = 2 * ck + (i >> 1), r = 2 * (i & 1);
+            const uint32_t pk = T::pack2(fast_exp2(e_acc[kb][qb][r]), fast_exp2(e_acc[kb][qb][r + 1]));
+            ls[qb] = T::add_pair(pk, ls[qb]);   // the denominator sums the rounded weights the MFMA uses
+            asm volatile("" : "+v"(ls[qb]));     // ... here, not in one run after the tile's last MFMA
+            return pk;
         };
-        s16x8 pcur = weights(0, 0);
+        uint32_t pw[2][4];   // the packed weights in use and the next ones in the making
+#pragma unroll
+        for (int i = 0; i < 4; ++i) pw[0][i] = weights_quarter(0, 0, i);
         pin();
 #pragma unroll
         for (int s = 0; s < 4; ++s) {   // (ck, qb) = (s >> 1, s & 1)
             const int ck = s >> 1, qb = s & 1;
-            s16x8 pnext = pcur;
-            if (s + 1 < 4) pnext = weights((s + 1) >> 1, (s + 1) & 1);
+            uint4 pu; pu.x = pw[s & 1][0]; pu.y = pw[s & 1][1]; pu.z = pw[s & 1][2]; pu.w = pw[s & 1][3];
+            const s16x8 pcur = __builtin_bit_cast(s16x8, pu);
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
                 o_acc[db][qb] = T::mfma16(va[db], pcur, o_acc[db][qb]);
-                if (qb == 1 && ck == 0) {   // the chunk's fragments are used for the last time: the next chunk's take their place
-                    pin();
-                    va[db] = read_v(1, db);
-                    pin();
-                }
+                pin();
+                if (qb == 1 && ck == 0) va[db] = read_v(1, db);   // used for the last time: the next chunk's fragment takes its place
+                if (s + 1 < 4 && db < 4) pw[(s + 1) & 1][db] = weights_quarter((s + 1) >> 1, (s + 1) & 1, db);
+                pin();
             }
-            pin();
-            pcur = pnext;
         }
         l_sum[0] += ls[0];
         l_sum[1] += ls[1];
