@@ -166,18 +166,21 @@ MA_DEV s16x4 lds_read_tr16(uint32_t addr, int imm) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uintptr_t)(addr + imm));
 }
 
-// Value of x held by lane (l ^ 32), combined with the lane's own by max / sum.
+// Value of x held by lane (l ^ 32), combined with the lane's own by max / sum.  (The maximum of two values as their
+// median with +inf: one instruction, where fmaxf on values that come out of a lane swap costs three, the compiler quieting
+// each possible signalling NaN first.)
+MA_DEV float max2(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, __builtin_inff()); }
 MA_DEV float max_across_halves(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
-    return fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
+    return max2(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1]));
 }
 // The same over the four lanes l, l ^ 16, l ^ 32, l ^ 48 (the 16-lane groups of a 16x16 MFMA block's column): rows
 // 1 and 3 of one operand are swapped with rows 0 and 2 of the other, then the halves.
 MA_DEV float max_across_quads(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
-    return max_across_halves(fmaxf(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1])));
+    return max_across_halves(max2(__builtin_bit_cast(float, (uint32_t)r[0]), __builtin_bit_cast(float, (uint32_t)r[1])));
 }
 MA_DEV float sum_across_halves(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);

@@ -456,6 +456,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
     // exceeds it by more than kLazyLog2, so most tiles rescale nothing and weights stay below 2^kLazyLog2.
     float m_ref[2] = {-INFINITY, -INFINITY}, l_sum[2] = {0.f, 0.f};
     constexpr float kLazyLog2 = 8.f;
+    float grow_at[2] = {-INFINITY, -INFINITY};
     f32x4 neg_ref[2];   // -m_ref in every register (0 while there is no reference): the MFMA C operand of Q K^T
     neg_ref[0] = neg_ref[1] = f32x4{0.f, 0.f, 0.f, 0.f};
 
@@ -577,8 +578,8 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
                     for (int e = 0; e < 4; ++e) x = fmaxf(x, e_acc[kb][qb][e]);
                 mx[qb] = max_across_quads(x);   // largest exponent of the row in this tile, relative to the reference
             }
-            const bool grow0 = mx[0] > kLazyLog2 || (m_ref[0] == -INFINITY && mx[0] > -INFINITY);
-            const bool grow1 = mx[1] > kLazyLog2 || (m_ref[1] == -INFINITY && mx[1] > -INFINITY);
+            // (grow_at: kLazyLog2 once the row has a reference, -inf before: one compare per row says whether it moves)
+            const bool grow0 = mx[0] > grow_at[0], grow1 = mx[1] > grow_at[1];
             if (__any(grow0 || grow1)) {  // wave-uniform branch
 #pragma unroll
                 for (int qb = 0; qb < 2; ++qb) {
@@ -586,6 +587,7 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
                     const float delta = grow ? mx[qb] : 0.f;
                     const float alpha = (m_ref[qb] == -INFINITY) ? 0.f : fast_exp2(-delta);
                     m_ref[qb] = grow ? ((m_ref[qb] == -INFINITY) ? mx[qb] : m_ref[qb] + mx[qb]) : m_ref[qb];
+                    grow_at[qb] = (m_ref[qb] == -INFINITY) ? -INFINITY : kLazyLog2;
                     const float nr = (m_ref[qb] == -INFINITY) ? 0.f : -m_ref[qb];
                     neg_ref[qb] = f32x4{nr, nr, nr, nr};
                     l_sum[qb] *= alpha;

@@ -193,7 +193,8 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     // row 16 b + l16 does not depend on b.
     constexpr int M16 = 2 * MB, N16 = 2 * NB, BLK = kRowTile / 4;
     const int l16 = lane & 15, quad = lane >> 4;
-    uint32_t m_rd[2], n_rd[4];
+    constexpr int NRD = N16 < 4 ? 4 : N16;
+    uint32_t m_rd[2], n_rd[NRD];
     {
         const int sw = swz_row_tile(l16);
 #pragma unroll
@@ -205,11 +206,10 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
         if (!NT) {
             // n fragments through transpose reads of the [k][n] sub-tile: the 16-lane group `quad` addresses k rows
             // 8 quad + 0..3 (second read: + 4) of the slice, 16 columns, and lane l16 receives column l16
-            static_assert(NT || N16 <= 4, "one read address per 16-column block");
             const int krow = 8 * quad + (l16 >> 2);
             const int swv = swz_col_tile(krow);
 #pragma unroll
-            for (int nb = 0; nb < 4; ++nb) {
+            for (int nb = 0; nb < NRD; ++nb) {
                 const int n = 16 * (N16 * wn + (nb < N16 ? nb : 0)), col = (n & 127) + 4 * (l16 & 3);
                 n_rd[nb] = lds_addr(&b_lds[0][0]) + (n >> 7) * kColTile + krow * 256 + 16 * ((col >> 3) ^ swv) + 2 * (col & 7);
             }
