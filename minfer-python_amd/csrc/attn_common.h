@@ -166,10 +166,18 @@ MA_DEV s16x4 lds_read_tr16(uint32_t addr, int imm) {
     return __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(uintptr_t)(addr + imm));
 }
 
-// Value of x held by lane (l ^ 32), combined with the lane's own by max / sum.  (The maximum of two values as their
-// median with +inf: one instruction, where fmaxf on values that come out of a lane swap costs three, the compiler quieting
-// each possible signalling NaN first.)
-MA_DEV float max2(float a, float b) { return __builtin_amdgcn_fmed3f(a, b, __builtin_inff()); }
+// Value of x held by lane (l ^ 32), combined with the lane's own by max / sum.  (The maximum of the two values of a lane
+// swap as one instruction: fmaxf on them costs three, the compiler quieting each possible signalling NaN first.)
+MA_DEV float max2(float a, float b) {
+    float r;
+    asm("v_max_f32 %0, %1, %2" : "=v"(r) : "v"(a), "v"(b));
+    return r;
+}
+MA_DEV float max3(float a, float b, float c) {
+    float r;
+    asm("v_max3_f32 %0, %1, %2, %3" : "=v"(r) : "v"(a), "v"(b), "v"(c));
+    return r;
+}
 MA_DEV float max_across_halves(float x) {
     uint32_t u = __builtin_bit_cast(uint32_t, x);
     auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);

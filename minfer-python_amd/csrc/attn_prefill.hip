@@ -571,11 +571,15 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
             float mx[2];
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-                float x = e_acc[0][qb][0];
+                // the lane's 16 exponents of the row, three-operand maxima written out (through fmaxf every operand that comes
+                // out of an MFMA is first passed through an instruction of its own that quiets a signalling NaN)
+                float x = max3(e_acc[0][qb][0], e_acc[0][qb][1], e_acc[0][qb][2]);
+                x = max3(x, e_acc[0][qb][3], e_acc[1][qb][0]);
 #pragma unroll
-                for (int kb = 0; kb < 4; ++kb)
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) x = fmaxf(x, e_acc[kb][qb][e]);
+                for (int kb = 1; kb < 4; ++kb) {
+                    x = max3(x, e_acc[kb][qb][1], e_acc[kb][qb][2]);
+                    x = kb < 3 ? max3(x, e_acc[kb][qb][3], e_acc[kb + 1][qb][0]) : max2(x, e_acc[kb][qb][3]);
+                }
                 mx[qb] = max_across_quads(x);   // largest exponent of the row in this tile, relative to the reference
             }
             // (grow_at: kLazyLog2 once the row has a reference, -inf before: one compare per row says whether it moves)
