@@ -34,25 +34,25 @@ DECODE_TRAFFIC_BYTES = 1092850 * 1024
 ROPE_TRAFFIC_BYTES = 393314 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
 NORM_TRAFFIC_BYTES = 786691 * 1024          # rmsnorm on [8,4096,6144]
-GEMM_TRAFFIC_BYTES = 230399 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
+GEMM_TRAFFIC_BYTES = 229729 * 1024          # gemm 4096^3 (A and B panels are re-read by several XCDs)
 DECODE_Q8_TRAFFIC_BYTES = 598274 * 1024     # decode over Q8_0 caches (split + combine)
 APPEND_Q8_TRAFFIC_BYTES = 737591 * 1024     # rope_kv_append into Q8_0 caches
 APPEND_NORM_TRAFFIC_BYTES = 786609 * 1024   # rope_kv_append_norm, the same shape
-QKV_TRAFFIC_BYTES = 378518 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
+QKV_TRAFFIC_BYTES = 377962 * 1024           # qkv in one launch, M=K=4096, N=4096+1024+1024
 LONG_TRAFFIC_BYTES = 2721732 * 1024         # long-context prefill (classify + main), S=32768 bf16: the 1 GiB mask once, K/V re-fetched past the 4 MiB L2s
-RAGGED_TRAFFIC_BYTES = 748602 * 1024        # packed ragged prefill (T=20514, Hq=64)
+RAGGED_TRAFFIC_BYTES = 747982 * 1024        # packed ragged prefill (T=20514, Hq=64)
 GEMM_Q8_TRAFFIC_BYTES = 61124 * 1024        # one token against a 14336 x 4096 weight of Q8_0 blocks
 GEMM_DECODE_TRAFFIC_BYTES = 120705 * 1024   # 64 tokens against the same weight in fp16, [N, K]
 # The kernel sources the counter runs were made against (first 12 hex digits of each file's sha1).  A row one of whose
 # sources has changed since carries "traffic_stale": true, so a constant that describes an earlier kernel says so.
 TRAFFIC_MEASURED_AGAINST = {
-    "attn_common.h": "4188ced83d04",
-    "attn_prefill.hip": "9a7e568fd938",
+    "attn_common.h": "4dea1f54fd55",
+    "attn_prefill.hip": "90dbd3456e56",
     "attn_decode.hip": "af41b9ac94d8",
     "quant_q8.h": "4fea6a94e300",
     "rope.hip": "b4fd0618b44e",
     "rmsnorm.hip": "f6c4e575f461",
-    "gemm.hip": "eba33e8b9ad5",
+    "gemm.hip": "7941349430d6",
 }
 TRAFFIC_ROW_SOURCES = {
     "": ("attn_common.h", "attn_prefill.hip"), "long_context": ("attn_common.h", "attn_prefill.hip"), "ragged": ("attn_common.h", "attn_prefill.hip"),

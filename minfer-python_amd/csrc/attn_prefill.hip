@@ -3,16 +3,16 @@
 // Work decomposition.  One workgroup = 8 waves (two per SIMD, so one wave's softmax overlaps the
 // other's MFMAs) = one KV head x (HPW query heads of that KV head's GQA group) x (QBW consecutive
 // 32-row query blocks), HPW*QBW = 8, so the K/V tiles a workgroup stages in LDS are shared by
-// every query head of the group.  Each wave owns 32 query rows of one head and keeps its Q
-// fragments, the 64x32 score tile and the Dx32 output accumulator in registers.
+// every query head of the group.  Each wave owns 32 query rows of one head (two blocks of 16) and keeps
+// its Q fragments, the 64x32 score tile and the Dx32 output accumulator in registers.
 //
-// Per 64-key tile a wave computes S^T = K Q^T (K from LDS as the MFMA A operand, Q as B), so
-// that a lane holds 16 keys of ONE query row per 32x32 block: row max / row sum need a single
-// exchange with lane^32.  The exponentiated scores are, without any data movement, the B operand
-// of O^T += V^T P^T; V^T fragments come from LDS transpose reads.  K and V tiles are copied
-// global->LDS directly (no VGPR staging) and double-buffered: the copy of tile t+1 is issued
-// right after the barrier that opens tile t.  The K fragments of a tile pass through a ring of
-// two register buffers, so the next fragment is requested while the current one feeds its MFMAs.
+// Per 64-key tile a wave computes S^T = K Q^T with v_mfma_f32_16x16x32 (K from LDS as the MFMA A operand,
+// Q as B), so that a lane holds four keys of each of its two query rows per 16x16 block: a row maximum /
+// row sum needs two lane swaps (lanes l ^ 16, l ^ 32).  The exponentiated scores of two key blocks are,
+// without any data movement, the B operand of a 32-key chunk of O^T += V^T P^T; V^T fragments come from
+// LDS transpose reads.  K and V tiles are copied global->LDS directly (no VGPR staging) and
+// double-buffered: the copy of tile t+1 is issued right after the barrier that opens tile t.  The K
+// fragments of a tile pass through a ring of two register buffers, refilled two chunks ahead.
 //
 // Query rows in, output rows out.  Every wave has a private 8 KiB LDS area.  Its 32 query rows
 // are copied there global->LDS as whole rows (full 128/256-byte lines per request) and read back

@@ -9,12 +9,12 @@
 // too small to fill the chip with large tiles) and walks K in steps of 64; the A and B panels of a step (32 KB
 // each) are copied global->LDS without passing through registers, double-buffered, one barrier per step
 // (placed inside the step, so that the matrix pipe keeps running across step boundaries).
-// Every wave owns 128 (64) rows (m) x 64 columns (n) as 4 (2) x 2 accumulator blocks of 32x32
-// and computes the transposed product D^T = B^T A^T, so that a lane ends up with 4 consecutive n of one row m
-// and the epilogue stores 8 bytes per register quadruple: B supplies the MFMA A operand (for the [K, N] layout
-// through LDS transpose reads, the same way the attention kernel reads V^T; for [N, K] through plain 16-byte
-// reads) and A supplies the B operand (16-byte reads).  LDS panels are split into sub-tiles whose geometry
-// and XOR swizzles are those of the attention kernel's K and V tiles, so both read patterns are free of bank
+// Every wave owns 128 (64) rows (m) x 64 columns (n) as 8 (4) x 4 accumulator blocks of 16x16
+// (v_mfma_f32_16x16x32) and computes the transposed product D^T = B^T A^T, so that a lane ends up with 4
+// consecutive n of one row m and the epilogue stores 8 bytes per block: B supplies the MFMA A operand (for the
+// [K, N] layout through LDS transpose reads, the same way the attention kernel reads V^T; for [N, K] through
+// plain 16-byte reads) and A supplies the B operand (16-byte reads).  LDS panels are split into sub-tiles
+// with XOR swizzles of the kind the attention kernel's K and V tiles use, so both read patterns are free of bank
 // conflicts.  Workgroup ids are dealt so that one XCD works on consecutive tiles of a tile row (they share the
 // A panel in that XCD's L2).
 #include <algorithm>
@@ -29,7 +29,7 @@ namespace minfer_attn {
 
 constexpr int kBK = 64;
 // Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
-// 128 x 128 otherwise.  A wave owns 32*MB rows x 32*NB columns; OCC waves per SIMD.
+// 128 x 128 otherwise.  A wave owns 32*MB rows x 32*NB columns (as blocks of 16 x 16); OCC waves per SIMD.
 template <int MB_, int NB_, int WAVES_N_, int OCC_, int WAVES_M_ = 2> struct GemmShape {
     static constexpr int MB = MB_, NB = NB_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N, OCC = OCC_;
     static constexpr int BM = 32 * MB * WAVES_M, BN = 32 * NB * WAVES_N;
@@ -37,11 +37,9 @@ template <int MB_, int NB_, int WAVES_N_, int OCC_, int WAVES_M_ = 2> struct Gem
     static constexpr int A_COPIES = A_PANEL / 1024 / WAVES, B_COPIES = B_PANEL / 1024 / WAVES;   // wave-wide copies per wave
 };
 // (4 waves with 128 x 128 each, GemmShape<4, 4, 2, 1>, read a third fewer LDS bytes per flop.  Compiled as it stands
-// that shape spills (its 256 accumulators leave the allocator no register to move anything with) and runs 3.2x slower;
+// that shape spills: its 256 accumulators leave the allocator no register to move anything with.  On 32 x 32 blocks,
 // with 14 of the 16 accumulator blocks pinned to the accumulation registers and 2 to the vector registers by inline
-// assembly, one copy offset per panel, and the LDS reads and global->LDS copies issued one after each MFMA, since no
-// second wave covers a burst of them, it is spill-free and ends level with the 8-wave shape at 4096^3 (122.5 against
-// 124.0 us) and 4 % behind at 8192^3: the LDS bytes are not what bounds this kernel.)
+// assembly, it was spill-free and ended level with the 8-wave shape at 4096^3 and 4 % behind at 8192^3.)
 using GemmBig = GemmShape<4, 2, 4, 2>;
 using GemmSmall = GemmShape<2, 2, 2, 2>;
 // 256 x 192 (8 waves as 4 x 2, a wave owns 64 x 96): for widths that are multiples of 192 whose 256 x 256 tiles would
