@@ -230,6 +230,24 @@ def test_q8_0_validation_rejects_before_launch():
     assert app(B=0) == capi.OK and app(Ln=0) == capi.OK
 
 
+def test_calibration_validation_rejects_before_launch():
+    L = capi.lib()
+    i64 = ctypes.c_int64
+    for fn in (L.minfer_calib_mfma_rate, L.minfer_calib_mfma_rate_32x32x16):
+        fn.restype = ctypes.c_int
+        fn.argtypes = [ctypes.c_int, ctypes.c_void_p, i64, i64, ctypes.c_void_p, ctypes.c_void_p]
+        assert fn(7, 0x1000, 10, 1, 0x2000, None) == capi.EINVAL and "dtype" in capi.last_error()
+        assert fn(capi.F16, 0x1008, 10, 1, 0x2000, None) == capi.EINVAL and "aligned" in capi.last_error()
+        assert fn(capi.F16, 0x1000, -1, 1, 0x2000, None) == capi.EINVAL and "iters" in capi.last_error()
+        assert fn(capi.F16, 0x1000, 10, 0, 0x2000, None) == capi.EINVAL
+        assert fn(capi.F16, 0x1000, 10, 1, None, None) == capi.EINVAL
+    mix = L.minfer_calib_attn_mix
+    mix.restype = ctypes.c_int
+    mix.argtypes = [ctypes.c_int, ctypes.c_void_p, i64, i64, ctypes.c_int, ctypes.c_int, ctypes.c_void_p, ctypes.c_void_p]
+    assert mix(7, 0x1000, 10, 1, 1, 1, 0x2000, None) == capi.EINVAL and "dtype" in capi.last_error()
+    assert mix(capi.BF16, None, 10, 1, 1, 1, 0x2000, None) == capi.EINVAL
+
+
 def test_python_surface_matches_reference_names(kerns):
     from minfer.const import GGML_QUANT_SIZES, GGMLQuantizationType
     from minfer.kernels import KernelBackend, refs
