@@ -184,8 +184,8 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     };
 
     // ---- per-lane LDS read addresses (stage 0; stage, sub-tile and block offsets are immediates) ---------
-    // The matrix instruction is v_mfma_f32_16x16x32 (on random operands the chip sustains 1.86-1.90 PFLOP/s of it and
-    // 1.57-1.62 of v_mfma_f32_32x32x16, whose rate is what a power-bound GEMM then runs at).  A K step is two slices of
+    // The matrix instruction is v_mfma_f32_16x16x32 (on random fp16 operands the chip sustains 1.80-1.90 PFLOP/s of it and
+    // 1.56-1.62 of v_mfma_f32_32x32x16, and a power-bound GEMM runs at what its matrix instruction sustains).  A K step is two slices of
     // 32 values; a fragment is 16 rows x 32 k, lane (l16, quad) holding row l16, k = 8 quad + 0..7 of the slice: 16 bytes
     // at granule (4 slice + quad) ^ swizzle of the row.  A 16-row block is a quarter of a 64-row sub-tile; the swizzle of
     // row 16 b + l16 does not depend on b.
