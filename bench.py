@@ -47,7 +47,7 @@ GEMM_DECODE_TRAFFIC_BYTES = 120705 * 1024   # 64 tokens against the same weight 
 # sources has changed since carries "traffic_stale": true, so a constant that describes an earlier kernel says so.
 TRAFFIC_MEASURED_AGAINST = {
     "attn_common.h": "4dea1f54fd55",
-    "attn_prefill.hip": "90dbd3456e56",
+    "attn_prefill.hip": "366ca412a479",
     "attn_decode.hip": "af41b9ac94d8",
     "quant_q8.h": "4fea6a94e300",
     "rope.hip": "b4fd0618b44e",

@@ -770,10 +770,13 @@ static int dispatch_prefill(int dtype, int64_t D, const PrefillParams& p, int wa
 #endif
 // Measured, 4 against 8 waves, 32 query heads over 8 KV heads: 128 packed sequences of 128 rows 87 / 98 us, 64 of 512
 // rows 256 / 263 us, dense B=16 L=512 68 / 73 us, B=8 L=1024 95.5 / 97.8 us, B=4 L=2048 159 / 156 us, L=4096 157 / 146 us.
+// At head_dim 64 a tile has half the MFMAs for the same vector work and the small workgroups win at every length
+// (clocks settled, 4 / 8 waves: B=8 L=1024 54.6 / 65.2 us, B=4 L=2048 88 / 102, B=1 L=8192 292 / 330, L=16384 1113 / 1267;
+// head_dim 128 for comparison: L=1536 180 / 182, L=2048 151.5 / 149.6, L=4096 143.7 / 134.4, L=8192 506 / 494).
 constexpr int64_t kSmallWorkgroupMaxRows = 1024;
-static int prefill_waves(int64_t longest) {
+static int prefill_waves(int64_t longest, int64_t D) {
     if (MINFER_PREFILL_FORCE_WAVES) return MINFER_PREFILL_FORCE_WAVES;
-    return longest <= kSmallWorkgroupMaxRows ? kWavesSmall : kWavesBig;
+    return (D == 64 || longest <= kSmallWorkgroupMaxRows) ? kWavesSmall : kWavesBig;
 }
 
 // The global->LDS copies of K/V tiles and query rows and the output stores address a block's rows with a 32-bit unsigned
@@ -825,7 +828,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn(int dtype, const void* q, const void* k
     hipStream_t stream = (hipStream_t)stream_v;
 
     PrefillParams p{};
-    const int kWaves = prefill_waves(L);
+    const int kWaves = prefill_waves(L, D);
     fill_common(p, q, k, v, out, Hq, Hkv, D, st, kWaves);
     p.mask = mask; p.cls = (const uint8_t*)workspace; p.cu = nullptr;
     p.L = (int)L; p.B = (int)B;
@@ -871,7 +874,7 @@ MINFER_ATTN_EXPORT int minfer_flash_attn_varlen(int dtype, const void* q, const 
     // must be at least the longest sequence (as in every varlen attention interface).
     const int64_t max_len = (max_seqlen > 0 && max_seqlen < T) ? max_seqlen : T;
     PrefillParams p{};
-    const int kWaves = prefill_waves(max_len);
+    const int kWaves = prefill_waves(max_len, D);
     fill_common(p, q, k, v, out, Hq, Hkv, D, st, kWaves);
     p.mask = nullptr; p.cls = nullptr; p.cu = cu_seqlens;
     p.L = (int)T; p.B = 1;
