@@ -1371,8 +1371,11 @@ static int gemm_splits(int64_t M, int64_t N, int64_t K) {
     if (tiles > 256 || kt < 8) return 1;
     int64_t s = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(256 / tiles, kt / 4), 32));
     // 64-127 tiles get two or three slices that way and fill the chip once; twice as many, while a slice stays 16 steps long,
-    // keep two workgroups on a compute unit ([K,N] 4096 x 14336 at 1-16 rows: 27.5 -> 22 us; 128 rows 37 -> 32)
-    if (tiles >= 64 && tiles * s <= 256 && kt / (2 * s) >= 16) s *= 2;
+    // keep two workgroups on a compute unit ([K,N] 4096 x 14336 at 1-16 rows: 27.5 -> 22 us; 128 rows 37 -> 32).  Tiles that
+    // fill the chip by themselves (129-256) are cut in two only for long rows: the second launch and the partial sums cost
+    // what the second workgroup per unit gains at K = 8192 and less (clocks settled, sliced / not: 512 x 8192 x 8192 89.0 /
+    // 76.8 us, 1024 x 4096 x 4096 47.0 / 44.7, 256 x 14336 x 4096 47.5 / 44.9; 1024 x 4096 x 14336 134 / 146)
+    if (tiles >= 64 && tiles * s <= 256 && kt / (2 * s) >= 16 && (s >= 2 || kt >= 192)) s *= 2;
     return (int)s;
 }
 
