@@ -52,7 +52,7 @@ TRAFFIC_MEASURED_AGAINST = {
     "quant_q8.h": "4fea6a94e300",
     "rope.hip": "b4fd0618b44e",
     "rmsnorm.hip": "f6c4e575f461",
-    "gemm.hip": "3d5db10f45fd",
+    "gemm.hip": "89047d798694",
 }
 TRAFFIC_ROW_SOURCES = {
     "": ("attn_common.h", "attn_prefill.hip"), "long_context": ("attn_common.h", "attn_prefill.hip"), "ragged": ("attn_common.h", "attn_prefill.hip"),

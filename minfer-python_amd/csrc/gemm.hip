@@ -30,8 +30,9 @@ namespace minfer_attn {
 constexpr int kBK = 64;
 // Two tile shapes: 8 waves (2 x 4) on 256 x 256 for problems that fill the chip with such tiles, 4 waves (2 x 2) on
 // 128 x 128 otherwise.  A wave owns 32*MB rows x 32*NB columns (as blocks of 16 x 16); OCC waves per SIMD.
-template <int MB_, int NB_, int WAVES_N_, int OCC_, int WAVES_M_ = 2> struct GemmShape {
+template <int MB_, int NB_, int WAVES_N_, int OCC_, int WAVES_M_ = 2, int NS_ = 2> struct GemmShape {
     static constexpr int MB = MB_, NB = NB_, WAVES_M = WAVES_M_, WAVES_N = WAVES_N_, WAVES = WAVES_M * WAVES_N, OCC = OCC_;
+    static constexpr int NS = NS_;   // stages of the K ring in LDS: NS - 1 steps in flight while one is multiplied
     static constexpr int BM = 32 * MB * WAVES_M, BN = 32 * NB * WAVES_N;
     static constexpr int A_PANEL = BM * 128, B_PANEL = BN * 128;   // bytes of one K step
     static constexpr int A_COPIES = A_PANEL / 1024 / WAVES, B_COPIES = B_PANEL / 1024 / WAVES;   // wave-wide copies per wave
@@ -42,6 +43,12 @@ template <int MB_, int NB_, int WAVES_N_, int OCC_, int WAVES_M_ = 2> struct Gem
 // assembly, it was spill-free and ended level with the 8-wave shape at 4096^3 and 4 % behind at 8192^3.)
 using GemmBig = GemmShape<4, 2, 4, 2>;
 using GemmSmall = GemmShape<2, 2, 2, 2>;
+// The same tile with three stages (96 KiB of LDS: one workgroup per compute unit) for launches of at most one workgroup per
+// compute unit anyway: two steps in flight instead of one (clocks settled, 512 x 6144 x 4096 as 192 tiles 43.6 -> 36.6 us,
+// 1024 x 4096 x 4096 as 256 tiles 44.9 -> 40.1, 256 x 14336 x 4096 44.9 -> 38.5; with more workgroups than compute units
+// two resident workgroups of two stages are ahead, 2048 x 4096 x 4096 66.9 against 78.6; four stages lose to three throughout).
+using GemmSmall3 = GemmShape<2, 2, 2, 2, 2, 3>;
+static bool one_workgroup_per_unit(int64_t workgroups) { return workgroups <= 256; }
 // 256 x 192 (8 waves as 4 x 2, a wave owns 64 x 96): for widths that are multiples of 192 whose 256 x 256 tiles would
 // leave half the chip idle in their last round (4096 x 6144 is 384 large tiles, one and a half rounds on 256 compute
 // units, but 512 of these, two full rounds of three quarters the work each).  [N, K] weights only: its 192 columns are
@@ -87,8 +94,10 @@ template <class T, bool NT, class SH, bool GROUPED = false, bool SPLIT = false, 
 __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const GemmParams p) {
     static_assert(!CONCAT || (GROUPED && NT && !SPLIT && SH::WAVES == 8), "CONCAT: grouped [N, K] weights, one sub-tile per copy index");
     constexpr int kBM = SH::BM, kBN = SH::BN, NW = SH::WAVES, MB = SH::MB, NB = SH::NB, CA = SH::A_COPIES, CB = SH::B_COPIES;
-    __shared__ __attribute__((aligned(1024))) char a_lds[2][SH::A_PANEL];
-    __shared__ __attribute__((aligned(1024))) char b_lds[2][SH::B_PANEL];
+    constexpr int NS = SH::NS;
+    static_assert(NS >= 2 && NS <= 4, "two to four stages");
+    __shared__ __attribute__((aligned(1024))) char a_lds[NS][SH::A_PANEL];
+    __shared__ __attribute__((aligned(1024))) char b_lds[NS][SH::B_PANEL];
 
     const int lane = threadIdx.x & 63, w = wave_id();
     const int h = lane >> 5, l32 = lane & 31;
@@ -167,15 +176,19 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     const int kt_all = p.K / kBK;
     const int kt_first = SPLIT ? (int)((int64_t)slice * kt_all / p.splits) : 0;
     const int KT = SPLIT ? (int)((int64_t)(slice + 1) * kt_all / p.splits) - kt_first : kt_all;
+    // (With three stages the compiler runs out of scalar registers in some instantiations and moves the panel bases from
+    // vector registers right in front of every copy, closer than a copy may follow such a move: those wait the documented
+    // distance inside the copy, see copy16_global_to_lds; the build's scan of the generated code is what finds such cases.)
+    constexpr bool kFreshBases = SH::NS > 2;
     // copy c of a step (the wave's A copies, then its B copies) into a stage
     auto copy_one = [&](int kt_rel, int stage, int c) __attribute__((always_inline)) {
         const int kt = kt_first + kt_rel;
         if (c < CA) {
-            copy16_global_to_lds(Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK, a_off[c], &a_lds[stage][a_dst[c]]);
+            copy16_global_to_lds<kFreshBases>(Ag + (int64_t)m0 * p.lda + (int64_t)kt * kBK, a_off[c], &a_lds[stage][a_dst[c]]);
         } else {
             const int j = c - CA;
             const short* bbase = NT ? Bg + (int64_t)n0 * ldb + (int64_t)kt * kBK : Bg + (int64_t)kt * kBK * ldb + n0;
-            copy16_global_to_lds(CONCAT ? b_src[CONCAT ? j : 0] + (int64_t)kt * kBK : bbase, b_off[j], &b_lds[stage][b_dst[j]]);
+            copy16_global_to_lds<kFreshBases>(CONCAT ? b_src[CONCAT ? j : 0] + (int64_t)kt * kBK : bbase, b_off[j], &b_lds[stage][b_dst[j]]);
         }
     };
     auto issue = [&](int kt_rel, int stage) __attribute__((always_inline)) {
@@ -248,7 +261,14 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     auto pin = [&]() __attribute__((always_inline)) { __builtin_amdgcn_sched_barrier(0); };
     // one slice: MFMAs on nf[buf] and mf; `next_tag`/`ks_next` name the slice read meanwhile (has_next: there is one);
     // SECOND: the step's second slice, with the barrier after group 0 and, if copy_kt >= 0, that step's copies after it
-    auto k_slice = [&](auto next_tag, int ks_next, int buf, bool has_next, auto second_tag, int copy_kt, auto stage_tag) __attribute__((always_inline)) {
+    // this wave's copies of all but the `later` most recently issued steps have landed (copies retire in order)
+    auto wait_stages = [&](int later) __attribute__((always_inline)) {
+        if (NS >= 4 && later >= 3) wait_vmcnt<(NS >= 4 ? 3 : 0) * NC>();
+        else if (NS >= 3 && later == 2) wait_vmcnt<(NS >= 3 ? 2 : 0) * NC>();
+        else if (later == 1) wait_vmcnt<NC>();
+        else wait_vmcnt<0>();
+    };
+    auto k_slice = [&](auto next_tag, int ks_next, int buf, bool has_next, auto second_tag, int copy_kt, auto stage_tag, int later = 0) __attribute__((always_inline)) {
         constexpr bool SECOND = decltype(second_tag)::value;
         constexpr int STAGE = decltype(stage_tag)::value;
 #pragma unroll
@@ -274,7 +294,7 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
             }
             if (SECOND && nb == 0) {
                 asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");   // this wave has read everything it needs from this stage
-                wait_vmcnt<0>();                                       // and its share of the next stage has landed
+                wait_stages(later);                                    // and its share of the next stage has landed
                 __syncthreads();
                 pin();
             }
@@ -282,22 +302,26 @@ __global__ __launch_bounds__(SH::WAVES * 64, SH::OCC) void gemm_kernel(const Gem
     };
     auto step = [&](auto stage_tag, int kt) __attribute__((always_inline)) {
         constexpr int STAGE = decltype(stage_tag)::value;
-        using Next = std::integral_constant<int, STAGE ^ 1>;
+        using Next = std::integral_constant<int, (STAGE + 1) % NS>;
         pin();
         k_slice(stage_tag, 1, 0, true, std::false_type{}, -1, stage_tag);
-        k_slice(Next{}, 0, 1, kt + 1 < KT, std::true_type{}, kt + 2 < KT ? kt + 2 : -1, stage_tag);
+        // at the barrier the next step's stage must have landed; the steps after it, up to NS - 2 of them, may be in flight
+        k_slice(Next{}, 0, 1, kt + 1 < KT, std::true_type{}, kt + NS < KT ? kt + NS : -1, stage_tag, min(NS - 2, KT - 2 - kt));
     };
-    issue(0, 0);
-    if (KT > 1) issue(1, 1);
-    if (KT > 1) wait_vmcnt<CA + CB>(); else wait_vmcnt<0>();   // the copies of step 0 retire first
+#pragma unroll
+    for (int st = 0; st < NS; ++st)
+        if (st < KT) issue(st, st);
+    wait_stages(min(NS, KT) - 1);   // the copies of step 0 retire first
     __syncthreads();
 #pragma unroll
     for (int nb = 0; nb < N16; ++nb) nf[0][nb] = read_n(std::integral_constant<int, 0>{}, 0, nb);
 #pragma unroll
     for (int mb = 0; mb < M16; ++mb) mf[mb] = read_m(std::integral_constant<int, 0>{}, 0, mb);
-    for (int kt = 0; kt < KT; kt += 2) {
+    for (int kt = 0; kt < KT; kt += NS) {
         step(std::integral_constant<int, 0>{}, kt);
         if (kt + 1 < KT) step(std::integral_constant<int, 1>{}, kt + 1);
+        if constexpr (NS > 2) if (kt + 2 < KT) step(std::integral_constant<int, 2 % NS>{}, kt + 2);
+        if constexpr (NS > 3) if (kt + 3 < KT) step(std::integral_constant<int, 3 % NS>{}, kt + 3);
     }
 
     // ---- epilogue: D = alpha * acc + beta * C; register e of a block is n = 4 quad + e, m = l16 ----
@@ -1393,7 +1417,9 @@ static int launch_split(GemmParams& p, hipStream_t stream) {
     p.tiles_m = (p.M + SH::BM - 1) / SH::BM;
     p.tiles_n = (p.N + SH::BN - 1) / SH::BN;
     p.per_xcd = 0;
-    hipLaunchKernelGGL((gemm_kernel<T, NT, SH, false, true>), dim3(p.tiles_m * p.tiles_n * p.splits), dim3(SH::WAVES * 64), 0, stream, p);
+    const int64_t wgs = (int64_t)p.tiles_m * p.tiles_n * p.splits;
+    if (one_workgroup_per_unit(wgs)) hipLaunchKernelGGL((gemm_kernel<T, NT, GemmSmall3, false, true>), dim3((unsigned)wgs), dim3(SH::WAVES * 64), 0, stream, p);
+    else hipLaunchKernelGGL((gemm_kernel<T, NT, SH, false, true>), dim3((unsigned)wgs), dim3(SH::WAVES * 64), 0, stream, p);
     if (int rc = check_launch("gemm_kernel (K slices)")) return rc;
     const int grid = (int)std::min<int64_t>(((int64_t)p.M * (p.N / 4) + 255) / 256, 256 * 8);
     hipLaunchKernelGGL((gemm_reduce_kernel<T>), dim3(grid), dim3(256), 0, stream, p);
@@ -1439,7 +1465,9 @@ static int launch_gemm(GemmParams& p, bool fast, hipStream_t stream) {
                 wide_shape_pays(big_tiles, (int64_t)((p.M + GemmWide::BM - 1) / GemmWide::BM) * (p.N / GemmWide::BN)))
                 return launch_tiled<T, NT, GemmWide>(p, stream);
         }
-        return big_tiles >= 160 ? launch_tiled<T, NT, GemmBig>(p, stream) : launch_tiled<T, NT, GemmSmall>(p, stream);
+        if (big_tiles >= 160) return launch_tiled<T, NT, GemmBig>(p, stream);
+        const int64_t small_tiles = (int64_t)((p.M + GemmSmall::BM - 1) / GemmSmall::BM) * ((p.N + GemmSmall::BN - 1) / GemmSmall::BN);
+        return one_workgroup_per_unit(small_tiles) ? launch_tiled<T, NT, GemmSmall3>(p, stream) : launch_tiled<T, NT, GemmSmall>(p, stream);
     }
     const int grid = (int)std::min<int64_t>(((int64_t)p.M * p.N + 255) / 256, 256 * 16);
     hipLaunchKernelGGL((gemm_plain_kernel<T, NT>), dim3(grid), dim3(256), 0, stream, p);
@@ -1525,6 +1553,7 @@ static int launch_grouped(GemmParams& p, int n_w, hipStream_t stream) {
     p.tiles_n = fill_ends(bn);
     p.per_xcd = (p.tiles_m * p.tiles_n + 7) / 8;
     if (big) hipLaunchKernelGGL((gemm_kernel<T, true, GemmBig, true>), dim3(p.per_xcd * 8), dim3(GemmBig::WAVES * 64), 0, stream, p);
+    else if (one_workgroup_per_unit((int64_t)p.per_xcd * 8)) hipLaunchKernelGGL((gemm_kernel<T, true, GemmSmall3, true>), dim3(p.per_xcd * 8), dim3(GemmSmall::WAVES * 64), 0, stream, p);
     else hipLaunchKernelGGL((gemm_kernel<T, true, GemmSmall, true>), dim3(p.per_xcd * 8), dim3(GemmSmall::WAVES * 64), 0, stream, p);
     return check_launch("gemm_kernel (grouped)");
 }
