@@ -568,11 +568,14 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
         }
         // ---- reference update (rare after the first tiles) --------------------------------------
         {
+            // The lane's largest exponent of each row (16 registers; three-operand maxima written out: through fmaxf every
+            // operand that comes out of an MFMA is first passed through an instruction of its own that quiets a signalling
+            // NaN).  A row moves its reference when its largest exponent exceeds grow_at (kLazyLog2 once the row has a
+            // reference, -inf before), which is the case exactly when one of the row's four lanes sees it: the lane swaps
+            // that make the row's maximum are left to the branch.
             float mx[2];
 #pragma unroll
             for (int qb = 0; qb < 2; ++qb) {
-                // the lane's 16 exponents of the row, three-operand maxima written out (through fmaxf every operand that comes
-                // out of an MFMA is first passed through an instruction of its own that quiets a signalling NaN)
                 float x = max3(e_acc[0][qb][0], e_acc[0][qb][1], e_acc[0][qb][2]);
                 x = max3(x, e_acc[0][qb][3], e_acc[1][qb][0]);
 #pragma unroll
@@ -580,11 +583,12 @@ __global__ __launch_bounds__(NW * 64, 2) void prefill_kernel(const PrefillParams
                     x = max3(x, e_acc[kb][qb][1], e_acc[kb][qb][2]);
                     x = kb < 3 ? max3(x, e_acc[kb][qb][3], e_acc[kb + 1][qb][0]) : max2(x, e_acc[kb][qb][3]);
                 }
-                mx[qb] = max_across_quads(x);   // largest exponent of the row in this tile, relative to the reference
+                mx[qb] = x;
             }
-            // (grow_at: kLazyLog2 once the row has a reference, -inf before: one compare per row says whether it moves)
-            const bool grow0 = mx[0] > grow_at[0], grow1 = mx[1] > grow_at[1];
-            if (__any(grow0 || grow1)) {  // wave-uniform branch
+            if (__any(mx[0] > grow_at[0] || mx[1] > grow_at[1])) {  // wave-uniform branch
+                mx[0] = max_across_quads(mx[0]);   // largest exponent of the row in this tile, relative to the reference
+                mx[1] = max_across_quads(mx[1]);
+                const bool grow0 = mx[0] > grow_at[0], grow1 = mx[1] > grow_at[1];
 #pragma unroll
                 for (int qb = 0; qb < 2; ++qb) {
                     const bool grow = qb == 0 ? grow0 : grow1;
