@@ -29,7 +29,7 @@ PEAK_HBM_GBS = 8000.0       # MI355X HBM3E
 # same counter reads for a 1 GiB copy: x2.0 and x1.0), classify+main and split+combine respectively
 # These are figures from those earlier counter runs, not measured in the run that prints them.
 TRAFFIC_SOURCE = "profiles/hbm_traffic_all_kernels_pmc.md (rocprofv3 --pmc runs of the same workloads; not re-measured by this run)"
-PREFILL_TRAFFIC_BYTES = 107400 * 1024
+PREFILL_TRAFFIC_BYTES = 107080 * 1024
 DECODE_TRAFFIC_BYTES = 1092850 * 1024
 ROPE_TRAFFIC_BYTES = 393314 * 1024          # il_rope on [8,4096,48,128], rotary 64
 APPEND_TRAFFIC_BYTES = 786532 * 1024        # rope_kv_append, B=8 L=4096 Llama-3-8B heads
@@ -47,7 +47,7 @@ GEMM_DECODE_TRAFFIC_BYTES = 120705 * 1024   # 64 tokens against the same weight 
 # sources has changed since carries "traffic_stale": true, so a constant that describes an earlier kernel says so.
 TRAFFIC_MEASURED_AGAINST = {
     "attn_common.h": "4dea1f54fd55",
-    "attn_prefill.hip": "366ca412a479",
+    "attn_prefill.hip": "d7de40fffd05",
     "attn_decode.hip": "af41b9ac94d8",
     "quant_q8.h": "4fea6a94e300",
     "rope.hip": "b4fd0618b44e",
